@@ -1,0 +1,204 @@
+// Attention-side kernels: QK RMSNorm + partial rotary + KV page write, and the universal paged attention kernel.
+#include "common.h"
+
+// Per-step row plan shared by the attention kernels (device arrays made once a step):
+//   pos[t]        absolute position of row t in its request
+//   row_entry[t]  index of the row's request among the step's entries
+//   tables        [n_entries, max_blocks] page ids of each entry in this cache group (-1: page given back)
+// Cache layout per layer and side: [page][kv_head][token_in_page][head_dim].
+
+enum : int { QKNORM_NONE = 0, QKNORM_PROJECTION = 1, QKNORM_HEAD = 2 };
+
+struct QkvArgs {
+    const float* qkv;  // [T, q_width + 2 kv_width] f32: q | k | v
+    const float* q_weight;
+    const float* k_weight;
+    const float* cos_sin;  // [positions, rotary_dim] f32: cos of the rotary_dim/2 pairs, then sin
+    const int* pos;
+    const int* row_entry;
+    const int* tables;
+    void* q_out;  // [T, q_width] in the activation type
+    void* k_cache;
+    void* v_cache;
+    float eps;
+    int n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode;
+    int page_tokens, max_blocks, write_kv;
+};
+
+// One block per row.  Norm over the whole projection: the sum of squares of the row's q (or k) values, strided per
+// thread, butterfly per wave, waves in order.  Then y = x * (r * w) and the NeoX rotation of pairs (i, i + R/2) of
+// each head: a' = fma(-b, sin, a*cos), b' = fma(a, sin, b*cos); dims [R, D) pass through.
+template <typename TQ, typename TKV>
+__global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
+    __shared__ float scratch[4];
+    const int t = blockIdx.x;
+    const int D = a.head_dim, half = a.rotary_dim / 2;
+    const int qw = a.n_heads * D, kw = a.n_kv_heads * D;
+    const float* row = a.qkv + (size_t)t * (qw + 2 * kw);
+    const int p = a.pos[t];
+    const float* cs = a.cos_sin + (size_t)p * a.rotary_dim;
+
+    float rq = 1.0f, rk = 1.0f;
+    if (a.norm_mode == QKNORM_PROJECTION) {
+        float s = 0.0f;
+        for (int i = threadIdx.x; i < qw; i += 256) s = fmaf(row[i], row[i], s);
+        s = block_sum<4>(s, scratch);
+        rq = 1.0f / sqrtf(s / (float)qw + a.eps);
+        s = 0.0f;
+        for (int i = threadIdx.x; i < kw; i += 256) s = fmaf(row[qw + i], row[qw + i], s);
+        s = block_sum<4>(s, scratch);
+        rk = 1.0f / sqrtf(s / (float)kw + a.eps);
+    }
+    const bool normed = a.norm_mode != QKNORM_NONE;
+
+    // q: every (head, dim) once; the rotated pair is recomputed by both of its threads
+    TQ* q_out = (TQ*)a.q_out + (size_t)t * qw;
+    for (int i = threadIdx.x; i < qw; i += 256) {
+        const int d = i % D;
+        float x = row[i];
+        if (normed) x = x * (rq * a.q_weight[i]);
+        if (d < a.rotary_dim) {
+            const int j = d < half ? d : d - half;
+            const int other = d < half ? i + half : i - half;
+            float y = row[other];
+            if (normed) y = y * (rq * a.q_weight[other]);
+            const float c = cs[j], s = cs[half + j];
+            x = d < half ? fmaf(-y, s, x * c) : fmaf(y, s, x * c);
+        }
+        st(q_out + i, x);
+    }
+    if (!a.write_kv) return;
+    const int e = a.row_entry[t];
+    const int page = a.tables[(size_t)e * a.max_blocks + p / a.page_tokens];
+    const int slot = p % a.page_tokens;
+    TKV* kc = (TKV*)a.k_cache;
+    TKV* vc = (TKV*)a.v_cache;
+    for (int i = threadIdx.x; i < kw; i += 256) {
+        const int h = i / D, d = i % D;
+        float x = row[qw + i];
+        if (normed) x = x * (rk * a.k_weight[i]);
+        if (d < a.rotary_dim) {
+            const int j = d < half ? d : d - half;
+            const int other = d < half ? i + half : i - half;
+            float y = row[qw + other];
+            if (normed) y = y * (rk * a.k_weight[other]);
+            const float c = cs[j], s = cs[half + j];
+            x = d < half ? fmaf(-y, s, x * c) : fmaf(y, s, x * c);
+        }
+        const size_t at = (((size_t)page * a.n_kv_heads + h) * a.page_tokens + slot) * D + d;
+        st(kc + at, x);
+        st(vc + at, row[qw + kw + i]);
+    }
+}
+
+extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight, const float* k_weight, const float* cos_sin, const int* pos,
+                                        const int* row_entry, const int* tables, void* q_out, void* k_cache, void* v_cache, int dtype,
+                                        float eps, int rows, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int norm_mode,
+                                        int page_tokens, int max_blocks, int write_kv, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (norm_mode != QKNORM_NONE && norm_mode != QKNORM_PROJECTION) return -2;
+    QkvArgs a{qkv, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
+              n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv};
+    if (dtype == LLMX_F32)
+        hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<float, float>), dim3(rows), dim3(256), 0, stream, a);
+    else
+        hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<bf16_t, bf16_t>), dim3(rows), dim3(256), 0, stream, a);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// Universal paged attention: one wave per (row, head).  Keys lo..p of the row's request are walked in tiles of 64 in
+// position order with an online softmax; lo = max(0, p - window + 1) under a window, else 0.  Lane j of a tile owns key
+// lo + 64*tile + j for the scores; for the value sum lane d owns dims d, d+64, ... and walks the tile's keys in order.
+// A row's arithmetic depends on its own position and request only.
+struct AttnArgs {
+    const void* q;  // [T, n_heads, head_dim]
+    const void* k_cache;
+    const void* v_cache;
+    const int* pos;
+    const int* row_entry;
+    const int* tables;
+    void* out;  // [T, n_heads * head_dim]
+    float scale;
+    int n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
+};
+
+#define ATT_MAX_D 256
+
+template <typename T>
+__global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a) {
+    __shared__ float qs[ATT_MAX_D];
+    __shared__ float ps[64];
+    __shared__ int pages[64];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int D = a.head_dim;
+    const int kvh = h / (a.n_heads / a.n_kv_heads);
+    const int p = a.pos[t];
+    const int* table = a.tables + (size_t)a.row_entry[t] * a.max_blocks;
+    const T* q = (const T*)a.q + ((size_t)t * a.n_heads + h) * D;
+    const T* kc = (const T*)a.k_cache;
+    const T* vc = (const T*)a.v_cache;
+    for (int d = lane; d < D; d += 64) qs[d] = ld(q + d);
+    __syncthreads();
+
+    const int lo = (a.window > 0 && p - a.window + 1 > 0) ? p - a.window + 1 : 0;
+    float m = -INFINITY, l = 0.0f;
+    float acc[ATT_MAX_D / 64];
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_D / 64; ++i) acc[i] = 0.0f;
+
+    for (int j0 = lo; j0 <= p; j0 += 64) {
+        const int j = j0 + lane;
+        float s = -INFINITY;
+        size_t base = 0;
+        if (j <= p) {
+            const int page = table[j / a.page_tokens];
+            base = (((size_t)page * a.n_kv_heads + kvh) * a.page_tokens + j % a.page_tokens) * D;
+            float dot = 0.0f;
+            for (int d = 0; d < D; ++d) dot = fmaf(qs[d], ld(kc + base + d), dot);
+            s = dot * a.scale;
+        }
+        const float tile_max = wave_max(s);
+        const float m_new = fmaxf(m, tile_max);
+        const float w = j <= p ? expf(s - m_new) : 0.0f;
+        const float correction = expf(m - m_new);  // 0 on the first tile (m = -inf)
+        // the tile's weights summed in key order by every lane alike
+        ps[lane] = w;
+        pages[lane] = j <= p ? (int)(base / D) : -1;  // row index of the key in units of D
+        __syncthreads();
+        float tile_sum = 0.0f;
+        const int n = min(64, p - j0 + 1);
+        for (int i = 0; i < n; ++i) tile_sum += ps[i];
+        l = l * correction + tile_sum;
+#pragma unroll
+        for (int i = 0; i < ATT_MAX_D / 64; ++i) {
+            const int d = lane + 64 * i;
+            if (d < D) {
+                float v = acc[i] * correction;
+                for (int jj = 0; jj < n; ++jj) v = fmaf(ps[jj], ld(vc + (size_t)pages[jj] * D + d), v);
+                acc[i] = v;
+            }
+        }
+        m = m_new;
+        __syncthreads();
+    }
+    T* out = (T*)a.out + ((size_t)t * a.n_heads + h) * D;
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_D / 64; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) st(out + d, acc[i] / l);
+    }
+}
+
+extern "C" int llmx_paged_attention_generic(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
+                                            const int* tables, void* out, int dtype, float scale, int rows, int n_heads, int n_kv_heads,
+                                            int head_dim, int page_tokens, int max_blocks, int window, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (head_dim > ATT_MAX_D || n_heads % n_kv_heads) return -2;
+    AttnArgs a{q, k_cache, v_cache, pos, row_entry, tables, out, scale, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
+    if (dtype == LLMX_F32)
+        hipLaunchKernelGGL(paged_attention_generic_kernel<float>, dim3(rows, n_heads), dim3(64), 0, stream, a);
+    else
+        hipLaunchKernelGGL(paged_attention_generic_kernel<bf16_t>, dim3(rows, n_heads), dim3(64), 0, stream, a);
+    return LLMX_CHECK_LAUNCH();
+}

@@ -1,0 +1,136 @@
+// Routing kernels: scored top-k selection and the expert-sorted list of (token, slot) pairs.
+#include "common.h"
+
+enum : int { SCORE_SIGMOID = 0, SCORE_SOFTMAX = 1 };
+
+#define ROUTE_MAX_EXPERTS 1024
+#define ROUTE_MAX_K 256
+
+// One wave per row.  score s_e = sigmoid(z_e) (or softmax over the row); the pick key is b_e = s_e + bias_e; k times
+// the largest key not yet taken is picked, the lowest id on ties; the weight is the unbiased s_e, divided by the
+// picks' sum (added in pick order) when `normalize`, then times `scale`.  A row with a non-finite key gets ids -1 and
+// weights 0.  Ids and weights come out in pick order, best first.
+__global__ void __launch_bounds__(64) route_topk_kernel(const float* __restrict__ z, const float* __restrict__ bias, int* __restrict__ ids,
+                                                       float* __restrict__ weights, int n_experts, int k, int score, int normalize,
+                                                       float scale) {
+    __shared__ float s[ROUTE_MAX_EXPERTS];
+    __shared__ float b[ROUTE_MAX_EXPERTS];
+    __shared__ float chosen[ROUTE_MAX_K];
+    const int r = blockIdx.x, lane = threadIdx.x;
+    const float* row = z + (size_t)r * n_experts;
+    float row_max = -INFINITY;
+    if (score == SCORE_SOFTMAX) {
+        for (int e = lane; e < n_experts; e += 64) row_max = fmaxf(row_max, row[e]);
+        row_max = wave_max(row_max);
+    }
+    int finite = 1;
+    for (int e = lane; e < n_experts; e += 64) {
+        const float x = row[e];
+        const float v = score == SCORE_SIGMOID ? 1.0f / (1.0f + expf(-x)) : expf(x - row_max);
+        s[e] = v;
+    }
+    __syncthreads();
+    if (score == SCORE_SOFTMAX) {
+        // the row's sum in expert order, the same in every lane
+        float total = 0.0f;
+        for (int e = 0; e < n_experts; ++e) total += s[e];
+        __syncthreads();
+        for (int e = lane; e < n_experts; e += 64) s[e] = s[e] / total;
+        __syncthreads();
+    }
+    for (int e = lane; e < n_experts; e += 64) {
+        const float key = bias ? s[e] + bias[e] : s[e];
+        b[e] = key;
+        if (!isfinite(key)) finite = 0;
+    }
+    finite = __all(finite);
+    __syncthreads();
+    if (!finite) {
+        for (int j = lane; j < k; j += 64) {
+            ids[(size_t)r * k + j] = -1;
+            weights[(size_t)r * k + j] = 0.0f;
+        }
+        return;
+    }
+    for (int j = 0; j < k; ++j) {
+        // lane's best: first larger key in its ids in increasing order, so a lane's tie keeps its lowest id
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+        for (int e = lane; e < n_experts; e += 64) {
+            const float key = b[e];
+            if (key > best) {
+                best = key;
+                at = e;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, 64);
+            const int oa = __shfl_xor(at, o, 64);
+            if (ob > best || (ob == best && oa < at)) {
+                best = ob;
+                at = oa;
+            }
+        }
+        if (lane == 0) {
+            ids[(size_t)r * k + j] = at;
+            chosen[j] = s[at];
+            b[at] = -INFINITY;  // taken: below every finite key, so never picked again while an untaken id is left (k <= experts)
+        }
+        __syncthreads();
+    }
+    if (lane == 0) {
+        float total = 0.0f;
+        for (int j = 0; j < k; ++j) total += chosen[j];
+        const bool divide = normalize && (score == SCORE_SIGMOID || k > 1);
+        for (int j = 0; j < k; ++j) weights[(size_t)r * k + j] = (divide ? chosen[j] / total : chosen[j]) * scale;
+    }
+}
+
+extern "C" int llmx_route_topk(const float* z, const float* bias, int* ids, float* weights, int rows, int n_experts, int k, int score,
+                               int normalize, float scale, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (n_experts > ROUTE_MAX_EXPERTS || k > ROUTE_MAX_K || k > n_experts || k <= 0) return -2;
+    hipLaunchKernelGGL(route_topk_kernel, dim3(rows), dim3(64), 0, stream, z, bias, ids, weights, n_experts, k, score, normalize, scale);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// The pairs p = t*k + j of a step grouped by expert, each expert's pairs in increasing p (stable), without atomics:
+// pass 1 counts each expert's pairs, pass 2 derives each expert's offset from the counts and places its pairs.
+__global__ void __launch_bounds__(64) moe_count_kernel(const int* __restrict__ ids, int n_pairs, int* __restrict__ counts) {
+    const int e = blockIdx.x, lane = threadIdx.x;
+    int c = 0;
+    for (int p = lane; p < n_pairs; p += 64) c += ids[p] == e;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+    if (lane == 0) counts[e] = c;
+}
+
+__global__ void __launch_bounds__(64) moe_place_kernel(const int* __restrict__ ids, int n_pairs, int n_experts, const int* __restrict__ counts,
+                                                      int* __restrict__ offsets, int* __restrict__ list) {
+    const int e = blockIdx.x, lane = threadIdx.x;
+    int before = 0;
+    for (int i = lane; i < e; i += 64) before += counts[i];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o, 64);
+    if (lane == 0) {
+        offsets[e] = before;
+        if (e == n_experts - 1) offsets[n_experts] = before + counts[e];
+    }
+    int at = before;
+    for (int p0 = 0; p0 < n_pairs; p0 += 64) {
+        const int p = p0 + lane;
+        const bool mine = p < n_pairs && ids[p] == e;
+        const unsigned long long mask = __ballot(mine);
+        if (mine) list[at + __popcll(mask & ((1ull << lane) - 1ull))] = p;
+        at += __popcll(mask);
+    }
+}
+
+extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* counts, int* offsets, int* list, hipStream_t stream) {
+    if (n_pairs <= 0 || n_experts <= 0) return 0;
+    hipLaunchKernelGGL(moe_count_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, counts);
+    hipLaunchKernelGGL(moe_place_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, n_experts, counts, offsets, list);
+    return LLMX_CHECK_LAUNCH();
+}

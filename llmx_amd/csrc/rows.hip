@@ -1,0 +1,130 @@
+// Row-wise kernels: embedding gather, RMSNorm, row gather for the head.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// Embedding: x[t,:] = f32(table[id[t],:]).  Ids are checked on the host before any launch.
+template <typename TW>
+__global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ ids, float* __restrict__ x, int width) {
+    const int t = blockIdx.x;
+    const TW* row = table + (size_t)ids[t] * width;
+    float* out = x + (size_t)t * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = ld(row + i);
+}
+
+extern "C" int llmx_embed_gather(const void* table, int table_dtype, const int* ids, float* x, int rows, int width, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (table_dtype == LLMX_F32)
+        hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)table, ids, x, width);
+    else
+        hipLaunchKernelGGL(embed_gather_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, (const bf16_t*)table, ids, x, width);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm of f32 rows: s = sum x^2 (strided per thread, butterfly per wave, waves in order),
+// r = 1/sqrt(s/n + eps), y = x * (r * w).  Optional row gather on the input (the head reads only wanted rows).
+// Writes the result in the activation type and/or as f32 (the router reads unrounded rows).
+template <typename TO>
+__global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ pick, const float* __restrict__ w,
+                                                    float eps, TO* __restrict__ out, float* __restrict__ out32, int n) {
+    __shared__ float scratch[4];
+    const int r = blockIdx.x;
+    const float* row = x + (size_t)(pick ? pick[r] : r) * n;
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const float v = row[i];
+        s = fmaf(v, v, s);
+    }
+    s = block_sum<4>(s, scratch);
+    const float scale = 1.0f / sqrtf(s / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const float y = row[i] * (scale * w[i]);
+        if (out) st(out + (size_t)r * n + i, y);
+        if (out32) out32[(size_t)r * n + i] = y;
+    }
+}
+
+extern "C" int llmx_rmsnorm(const float* x, const int* pick, const float* w, float eps, void* out, int out_dtype, float* out32,
+                            int rows, int n, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (out_dtype == LLMX_F32)
+        hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(rows), dim3(256), 0, stream, x, pick, w, eps, (float*)out, out32, n);
+    else
+        hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, x, pick, w, eps, (bf16_t*)out, out32, n);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// Expert combine: x[t,:] += sum_j w[t,j] * y[t*k+j,:], j in slot order; a slot without an expert (id < 0) adds nothing.
+__global__ void moe_combine_kernel(float* __restrict__ x, const float* __restrict__ y, const int* __restrict__ ids,
+                                   const float* __restrict__ w, int k, int width, int accumulate) {
+    const int t = blockIdx.x;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float s = 0.0f;
+        for (int j = 0; j < k; ++j)
+            if (ids[t * k + j] >= 0) s += w[t * k + j] * y[((size_t)t * k + j) * width + i];
+        float* o = x + (size_t)t * width + i;
+        *o = accumulate ? *o + s : s;
+    }
+}
+
+extern "C" int llmx_moe_combine(float* x, const float* y, const int* ids, const float* w, int rows, int k, int width, int accumulate,
+                                hipStream_t stream) {
+    if (rows <= 0) return 0;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(rows), dim3(256), 0, stream, x, y, ids, w, k, width, accumulate);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// Fill with a constant (graph-safe replacement for a memset) and plain f32 add, used by toy parts and tests.
+__global__ void fill_i32_kernel(int* p, int v, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+extern "C" int llmx_fill_i32(int* p, int v, long n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, v, (size_t)n);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// Seeded fill: element i of a tensor is a function of (key, i) only.  h = mix64(key + i * golden);
+// normal: a + b * sqrt(-2 ln u1) * cos(2 pi u2) with u1 = (top 24 bits + 1) / 2^24, u2 = (next 24 bits) / 2^24;
+// uniform: a + (b - a) * (top 24 bits) / 2^24.
+__device__ __forceinline__ uint64_t mix64(uint64_t x) {
+    x ^= x >> 30;
+    x *= 0xBF58476D1CE4E5B9ull;
+    x ^= x >> 27;
+    x *= 0x94D049BB133111EBull;
+    x ^= x >> 31;
+    return x;
+}
+
+template <typename T>
+__global__ void fill_random_kernel(T* __restrict__ out, size_t n, uint64_t key, int kind, float a, float b) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const uint64_t h = mix64(key + i * 0x9E3779B97F4A7C15ull);
+        const float hi = (float)(uint32_t)(h >> 40);
+        float v;
+        if (kind == 0) {
+            const float u1 = (hi + 1.0f) * 5.9604644775390625e-8f;
+            const float u2 = (float)(uint32_t)((h >> 8) & 0xFFFFFFull) * 5.9604644775390625e-8f;
+            v = a + b * (sqrtf(-2.0f * logf(u1)) * cosf(6.2831853f * u2));
+        } else {
+            v = a + (b - a) * (hi * 5.9604644775390625e-8f);
+        }
+        st(out + i, v);
+    }
+}
+
+extern "C" int llmx_fill_random(void* out, int dtype, long n, unsigned long long key, int kind, float a, float b, hipStream_t stream) {
+    if (n <= 0) return 0;
+    long blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == LLMX_F32)
+        hipLaunchKernelGGL(fill_random_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream, (float*)out, (size_t)n, (uint64_t)key, kind, a, b);
+    else
+        hipLaunchKernelGGL(fill_random_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)out, (size_t)n, (uint64_t)key, kind, a, b);
+    return LLMX_CHECK_LAUNCH();
+}

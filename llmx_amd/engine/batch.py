@@ -1,0 +1,110 @@
+"""One step's rows as the parts see them: the row plan on the device and scratch storage.
+
+The row plan follows the reference's `begin` (/root/reference/src/model/passes.hpp:369-392): token ids, positions that
+continue each request's length, the rows whose logits are wanted; it is uploaded in one copy.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Hashable, List, Sequence, Tuple
+
+import numpy as np
+import torch
+
+
+@dataclass(frozen=True)
+class StepEntry:
+    """A request's next tokens in a step, and the places among them whose logits are wanted."""
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass(frozen=True)
+class EntryView:
+    request: Hashable
+    slot: int      # the request's state slot
+    row0: int      # its first row in the step
+    n: int         # its number of rows
+    past: int      # tokens it held before the step
+
+
+class Workspace:
+    """Scratch tensors by name; a name keeps its storage and grows when a larger shape is asked for."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self._store: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+
+    def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        count = 1
+        for d in shape:
+            count *= int(d)
+        key = (name, dtype)
+        flat = self._store.get(key)
+        if flat is None or flat.numel() < count:
+            flat = torch.empty(max(count, 1), dtype=dtype, device=self.device)
+            self._store[key] = flat
+        return flat[:count].view(*shape)
+
+    def bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self._store.values())
+
+
+class StepState:
+    """What the parts read of a step (see parts/base.py for the interface)."""
+
+    def __init__(self, workspace: Workspace, act_dtype: torch.dtype):
+        self._ws = workspace
+        self.act_dtype = act_dtype
+        self.device = workspace.device
+        self.rows = 0
+        self.entries: List[EntryView] = []
+        self.token_ids = self.positions = self.row_entry = self.entry_slots = self.pick = None
+        self._tables: List[torch.Tensor] = []
+        self.max_rows_per_entry = 0
+        self.run_index = -1          # which item of the run order is running
+        self.observer = None         # callable(step, kind, **tensors) that sees what parts choose to show, or None
+
+    def buf(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        return self._ws.get(name, shape, dtype)
+
+    def tables(self, group: int) -> torch.Tensor:
+        return self._tables[group]
+
+    def observe(self, kind: str, **tensors) -> None:
+        """Shows intermediate tensors (a router's picks, for instance) to the engine's observer, when one is set."""
+        if self.observer is not None:
+            self.observer(self, kind, **tensors)
+
+
+class RowPlanUploader:
+    """Packs the row plan into one pinned int32 buffer and copies it to the device once."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self._host = None
+        self._dev = None
+        self._done = None
+
+    def upload(self, arrays: List[np.ndarray]) -> List[torch.Tensor]:
+        total = sum(a.size for a in arrays)
+        if self._host is None or self._host.numel() < total:
+            cap = max(1024, 2 * total)
+            self._host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+            self._dev = torch.empty(cap, dtype=torch.int32, device=self.device)
+            self._done = None
+        if self._done is not None:
+            self._done.synchronize()  # the previous copy has left the pinned buffer
+        host = self._host.numpy()
+        at = 0
+        views = []
+        for a in arrays:
+            host[at:at + a.size] = a.reshape(-1)
+            views.append(self._dev[at:at + a.size].view(*a.shape))
+            at += a.size
+        self._dev[:total].copy_(self._host[:total], non_blocking=True)
+        self._done = torch.cuda.Event()
+        self._done.record()
+        return views

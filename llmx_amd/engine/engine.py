@@ -1,0 +1,285 @@
+"""The engine: a built model, its cache on the device, and the one step function everything else drives.
+
+`step` takes a batch of (request, its next tokens): portions of prompts beside single decoded tokens, cut anywhere.
+It runs only the tokens it is given, as one batch, from the cache earlier steps left, and returns the logits at the
+wanted places.  The transaction follows the reference's pass (/root/reference/src/model/passes.hpp:271-413 refusals
+before anything is reserved, :633-653 reserve pages, :771-830 run, :1007-1032 commit, :1124-1134 roll back).
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Dict, Hashable, List, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..cache import CacheManager, GroupSpec, OutOfPages
+from ..models import registry
+from ..parts.base import BuildContext, LayerCache
+from ..parts.spec import KVNeed, ModelSpec, StateNeed
+from ..weights import ModelFiles, RandomInit, load as load_weights
+from ..weights.loader import device_dtype
+from ..weights.random_init import stored_dtype
+from ..weights.device_init import fill_random
+from .batch import EntryView, RowPlanUploader, StepEntry, StepState, Workspace
+from .model import BuiltModel
+
+_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
+           "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
+
+
+class StepError(ValueError):
+    """A batch the step function refuses; nothing was reserved or run."""
+
+
+def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype in (torch.float32, torch.bfloat16):
+            return dtype
+    elif dtype in _DTYPES:
+        return _DTYPES[dtype]
+    raise ValueError(f"dtype {dtype!r} is not float32 or bfloat16")
+
+
+class Engine:
+    def __init__(self, config, spec: ModelSpec, dtype: Union[str, torch.dtype] = "bfloat16", *, kv_tokens: int,
+                 page_tokens: int = 16, max_requests: int = 8, device: Union[str, torch.device] = "cuda:0", weights=None):
+        """`weights(engine)` returns the device tensors by name; it runs before the cache is allocated, so weights that
+        do not fit the model are refused before anything large exists."""
+        if not torch.cuda.is_available():
+            raise RuntimeError("llmx_amd runs on a GPU only: no GPU is visible and there is no CPU path")
+        ops.lib()  # fail now, loudly, when the kernel library is missing
+        self.config = config
+        self.spec = spec
+        self.device = torch.device(device)
+        self.act_dtype = resolve_dtype(dtype)
+        if page_tokens <= 0 or kv_tokens <= 0:
+            raise ValueError("page_tokens and kv_tokens must be positive")
+        self.page_tokens = int(page_tokens)
+        self.kv_tokens = -(-int(kv_tokens) // self.page_tokens) * self.page_tokens
+        self.max_requests = int(max_requests)
+        self.max_positions = min(spec.max_positions, self.kv_tokens)
+        torch.cuda.set_device(self.device)
+        ctx = BuildContext(self.act_dtype, self.device, self.max_positions)
+        self.model = BuiltModel(spec, ctx)
+        self._loaded = False
+        if weights is not None:
+            self.model.load(weights(self))
+            self._loaded = True
+        self._workspace = Workspace(self.device)
+        self._uploader = RowPlanUploader(self.device)
+        #: callable(step, kind, **tensors): sees what parts show of a step (the reference's route hook,
+        #: /root/reference/src/model/arch/blocks.hpp:118-138); None in serving
+        self.observer = None
+        self._make_cache()
+
+    # -- construction -----------------------------------------------------------
+    @classmethod
+    def load(cls, folder: Union[str, Path], dtype="bfloat16", **options) -> "Engine":
+        """An engine for the model folder (config.json + safetensors); the model class is chosen by config.json."""
+        config, spec = registry.read_model_dir(folder)
+        files = ModelFiles(folder)
+
+        def from_files(eng: "Engine"):
+            specs = eng.model.tensor_specs(set(files.names()))
+            return load_weights(specs, files, eng.device, eng.act_dtype == torch.float32)
+
+        try:
+            return cls(config, spec, dtype, weights=from_files, **options)
+        finally:
+            files.close()
+
+    @classmethod
+    def from_random(cls, config, init: RandomInit = RandomInit(), dtype="bfloat16", **options) -> "Engine":
+        """An engine whose weights are generated on the device from (seed, tensor name); nothing is read or written."""
+        def generate(eng: "Engine"):
+            tensors = {}
+            for s in eng.model.tensor_specs():
+                dt = device_dtype(s, stored_dtype(s, init), eng.act_dtype == torch.float32)
+                t = torch.empty(s.shape, dtype=dt, device=eng.device)
+                fill_random(t, s, init)
+                tensors[s.name] = t
+            return tensors
+
+        return cls(config, registry.assemble(config), dtype, weights=generate, **options)
+
+    def _make_cache(self) -> None:
+        needs = self.model.cache_needs()
+        n_pages = self.kv_tokens // self.page_tokens
+        keys: List[KVNeed] = []
+        self._group_of: List[int] = []          # cache number -> group (or -1)
+        self._index_in_group: List[int] = []
+        counts: List[int] = []
+        for need in needs:
+            if isinstance(need, KVNeed):
+                if need not in keys:
+                    keys.append(need)
+                    counts.append(0)
+                g = keys.index(need)
+                self._group_of.append(g)
+                self._index_in_group.append(counts[g])
+                counts[g] += 1
+            else:
+                self._group_of.append(-1)
+                self._index_in_group.append(-1)
+        self.group_needs = keys
+        groups = [GroupSpec(f"kv{g}", self.page_tokens, n_pages, need.window) for g, need in enumerate(keys)]
+        self.cache = CacheManager(groups, self.max_requests)
+        # [cache in group, K|V, page, kv head, token in page, head dim]
+        self._kv = [torch.zeros((counts[g], 2, n_pages, need.kv_heads, self.page_tokens, need.head_dim), dtype=self.act_dtype,
+                                device=self.device) for g, need in enumerate(keys)]
+        self._state: List[Optional[torch.Tensor]] = []
+        for need in needs:
+            if isinstance(need, StateNeed):
+                self._state.append(torch.zeros((self.max_requests, *need.shape), dtype=getattr(torch, need.dtype), device=self.device))
+            else:
+                self._state.append(None)
+        self._layer_caches: List[LayerCache] = []
+        for e in self.spec.run_order:
+            g = self._group_of[e.cache]
+            if g >= 0:
+                store = self._kv[g][self._index_in_group[e.cache]]
+                self._layer_caches.append(LayerCache(group=g, k=store[0], v=store[1], writes=e.writes))
+            else:
+                self._layer_caches.append(LayerCache(state=self._state[e.cache], writes=e.writes))
+
+    # -- requests ---------------------------------------------------------------
+    def add_request(self, request: Hashable) -> int:
+        """Opens a request: a state slot is taken and its state cleared; pages come with its first tokens."""
+        slot = self.cache.open(request)
+        for s in self._state:
+            if s is not None:
+                s[slot].zero_()
+        return slot
+
+    def end_request(self, request: Hashable) -> None:
+        """The request is finished: what it holds is given back."""
+        self.cache.close(request)
+
+    def has_request(self, request: Hashable) -> bool:
+        return self.cache.is_open(request)
+
+    def length(self, request: Hashable) -> int:
+        return self.cache.length(request)
+
+    @property
+    def vocab_size(self) -> int:
+        return self.spec.vocab_size
+
+    # -- the step ---------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Runs the entries' tokens as one batch; returns float32 logits [wanted, vocab] in the order of entries and `want`.
+
+        The returned tensor is scratch storage: it is valid until the next step.
+        """
+        if not self._loaded:
+            raise RuntimeError("the engine has no weights yet")
+        entries = list(entries)
+        if not entries:
+            raise StepError("step: an empty batch")
+        seen = set()
+        V = self.spec.vocab_size
+        views: List[EntryView] = []
+        row0 = 0
+        for e in entries:
+            if e.request in seen:
+                raise StepError(f"step: request {e.request!r} appears twice in one batch")
+            seen.add(e.request)
+            if not self.cache.is_open(e.request):
+                raise StepError(f"step: request {e.request!r} is not open")
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"step: request {e.request!r} brings no tokens")
+            past = self.cache.length(e.request)
+            if past + n > self.max_positions:
+                raise StepError(f"step: context length exceeded: request {e.request!r} would hold {past + n} tokens of {self.max_positions}")
+            for t in e.tokens:
+                if not 0 <= int(t) < V:
+                    raise StepError(f"step: token id {t} is outside the embedding's rows")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"step: request {e.request!r} wants the logits of place {w} among {n} tokens")
+            views.append(EntryView(e.request, self.cache.slot(e.request), row0, n, past))
+            row0 += n
+        T = row0
+
+        prepared: List[Hashable] = []
+        try:
+            for e, v in zip(entries, views):
+                self.cache.prepare(e.request, v.n)
+                prepared.append(e.request)
+        except OutOfPages:
+            for r in prepared:
+                self.cache.abort(r)
+            raise
+        try:
+            logits = self._run(entries, views, T)
+        except BaseException:
+            for r in prepared:
+                self.cache.abort(r)
+            raise
+        for r in prepared:
+            self.cache.commit(r)
+        return logits
+
+    def _run(self, entries: List[StepEntry], views: List[EntryView], T: int) -> torch.Tensor:
+        n_e = len(entries)
+        token_ids = np.empty(T, dtype=np.int32)
+        positions = np.empty(T, dtype=np.int32)
+        row_entry = np.empty(T, dtype=np.int32)
+        pick: List[int] = []
+        for i, (e, v) in enumerate(zip(entries, views)):
+            token_ids[v.row0:v.row0 + v.n] = np.asarray(e.tokens, dtype=np.int32)
+            positions[v.row0:v.row0 + v.n] = np.arange(v.past, v.past + v.n, dtype=np.int32)
+            row_entry[v.row0:v.row0 + v.n] = i
+            pick.extend(v.row0 + int(w) for w in e.want)
+        slots = np.asarray([v.slot for v in views], dtype=np.int32)
+        arrays = [token_ids, positions, row_entry, slots, np.asarray(pick if pick else [0], dtype=np.int32)]
+        for g in range(len(self.cache.groups)):
+            tables = [self.cache.table(e.request, g) for e in entries]
+            width = max(1, max(len(t) for t in tables))
+            width = -(-width // 8) * 8
+            packed = np.full((n_e, width), -1, dtype=np.int32)
+            for i, t in enumerate(tables):
+                packed[i, :len(t)] = t
+            arrays.append(packed)
+        dev = self._uploader.upload(arrays)
+
+        step = StepState(self._workspace, self.act_dtype)
+        step.rows = T
+        step.entries = views
+        step.token_ids, step.positions, step.row_entry, step.entry_slots = dev[0], dev[1], dev[2], dev[3]
+        step.pick = dev[4][:len(pick)]
+        step._tables = dev[5:]
+        step.max_rows_per_entry = max(v.n for v in views)
+
+        E = self.spec.hidden_size
+        x = step.buf("residual", (T, E), torch.float32)
+        self.model.embedding.forward(step, x)
+        step.observer = self.observer
+        for i, (entry, cache) in enumerate(zip(self.spec.run_order, self._layer_caches)):
+            step.run_index = i
+            self.model.blocks[entry.layer].forward(step, x, cache)
+        W = len(pick)
+        if W == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        rows = step.buf("head.rows", (W, E), self.act_dtype)
+        self.model.final_norm.forward(step, x, rows, None, step.pick)
+        logits = step.buf("logits", (W, self.spec.vocab_size), torch.float32)
+        self.model.head.forward(step, rows, logits)
+        return logits
+
+    # -- accounting -------------------------------------------------------------
+    def weight_bytes(self) -> int:
+        seen, total = set(), 0
+        for p in self.model.parts():
+            for v in vars(p).values():
+                if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
+                    seen.add(v.data_ptr())
+                    total += v.numel() * v.element_size()
+        return total
+
+    def cache_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self._kv) + sum(t.numel() * t.element_size() for t in self._state if t is not None)

@@ -1,0 +1,244 @@
+"""Python face of the gfx950 kernel library.
+
+Each function checks on the host that its operands are what the kernel and its
+grid assume (device, dtype, contiguity, shapes, index ranges that the host
+knows) and then launches on torch's current stream.  There is no CPU path: a
+missing library or a tensor that is not on the GPU is an error.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+from typing import Optional
+
+import torch
+
+from .csrc import build as _build
+
+F32, BF16 = 0, 1
+EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
+QKNORM_NONE, QKNORM_PROJECTION, QKNORM_HEAD = 0, 1, 2
+SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def lib():
+    """The loaded kernel library; built at the first call when nothing is built."""
+    global _lib
+    if _lib is None:
+        path = _build.load_path()
+        try:
+            handle = ctypes.CDLL(str(path))
+        except OSError as e:
+            raise KernelError(f"the kernel library {path} could not be loaded: {e}") from None
+        _declare(handle)
+        handle._path = str(path)
+        _lib = handle
+    return _lib
+
+
+def library_path() -> str:
+    return lib()._path
+
+
+def _declare(h) -> None:
+    P, I, F, L = c_void_p, c_int, c_float, c_long
+    sigs = {
+        "llmx_embed_gather": [P, I, P, P, I, I, P],
+        "llmx_rmsnorm": [P, P, P, F, P, I, P, I, I, P],
+        "llmx_moe_combine": [P, P, P, P, I, I, I, I, P],
+        "llmx_fill_i32": [P, I, L, P],
+        "llmx_fill_random": [P, I, L, ctypes.c_ulonglong, I, F, F, P],
+        "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
+        "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
+        "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
+        "llmx_route_topk": [P, P, P, P, I, I, I, I, I, F, P],
+        "llmx_moe_align": [P, I, I, P, P, P, P],
+        "llmx_argmax_rows": [P, P, P, I, I, P],
+        "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
+    }
+    for name, args in sigs.items():
+        try:
+            fn = getattr(h, name)
+        except AttributeError:
+            raise KernelError(f"the kernel library lacks {name}; build it again from the current sources") from None
+        fn.argtypes = args
+        fn.restype = c_int
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16, not {dtype}")
+
+
+def _dev(t: Optional[torch.Tensor], name: str, dtype=None, shape=None) -> int:
+    """Checks a kernel operand and returns its address (0 for None)."""
+    if t is None:
+        return 0
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name} must be a tensor on the GPU (there is no CPU path)")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, not {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+    return t.data_ptr()
+
+
+def _check(rc: int, what: str) -> None:
+    if rc == -2:
+        raise KernelError(f"{what}: a size this kernel does not take")
+    if rc != 0:
+        raise KernelError(f"{what}: launch failed with HIP error {rc}")
+
+
+# ---------------------------------------------------------------------------
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    rows, width = out.shape
+    _check(lib().llmx_embed_gather(_dev(table, "table", shape=(table.shape[0], width)), _code(table.dtype),
+                                   _dev(ids, "ids", torch.int32, (rows,)), _dev(out, "out", torch.float32),
+                                   rows, width, _stream()), "embed_gather")
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor], out32: Optional[torch.Tensor] = None,
+            pick: Optional[torch.Tensor] = None) -> None:
+    """out[r] = norm(x[pick[r]] or x[r]); out in its own dtype, out32 an optional float32 copy."""
+    n = x.shape[-1]
+    rows = pick.shape[0] if pick is not None else x.shape[0]
+    if out is None and out32 is None:
+        raise KernelError("rmsnorm needs an output")
+    _check(lib().llmx_rmsnorm(_dev(x, "x", torch.float32), _dev(pick, "pick", torch.int32), _dev(weight, "weight", torch.float32, (n,)),
+                              float(eps), _dev(out, "out", shape=(rows, n)), _code(out.dtype) if out is not None else F32,
+                              _dev(out32, "out32", torch.float32, (rows, n)), rows, n, _stream()), "rmsnorm")
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:
+    """c[M,N] (+)= a[M,K] @ w[N,K]^T, accumulated in float32; EPI_SWIGLU: c = silu(a @ w[:N]^T) * (a @ w[N:]^T)."""
+    M, K = a.shape
+    N = w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]   # swiglu: w holds gate rows, then up rows
+    if w.shape[1] != K or tuple(c.shape) != (M, N):
+        raise KernelError(f"gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
+    _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
+                                   M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm")
+
+
+def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor, a_div: int,
+                 epilogue: int = EPI_STORE) -> None:
+    """For each group g: rows p in pairs[offsets[g]:offsets[g+1]] get c[p] = a[p // a_div] @ w[g]^T.
+
+    With EPI_SWIGLU w[g] holds gate rows then up rows and c[p] = silu(gate) * up.
+    """
+    G, NW, K = w.shape
+    N = NW // 2 if epilogue == EPI_SWIGLU else NW
+    if a.shape[1] != K or c.shape[1] != N:
+        raise KernelError(f"grouped_gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
+    n_pairs = pairs.shape[0]
+    if c.shape[0] < n_pairs or a.shape[0] * a_div < n_pairs:
+        raise KernelError("grouped_gemm: more pairs than rows")
+    _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
+                                   n_pairs, N, K, K, K, N, epilogue, G, _dev(offsets, "offsets", torch.int32, (G + 1,)),
+                                   _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
+           "grouped_gemm")
+
+
+def qknorm_rope_kvwrite(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], cos_sin: torch.Tensor,
+                        pos: torch.Tensor, row_entry: torch.Tensor, tables: torch.Tensor, q_out: torch.Tensor,
+                        k_cache: torch.Tensor, v_cache: torch.Tensor, eps: float, n_heads: int, n_kv_heads: int, head_dim: int,
+                        rotary_dim: int, norm_mode: int, write_kv: bool = True) -> None:
+    rows = qkv.shape[0]
+    qw, kw = n_heads * head_dim, n_kv_heads * head_dim
+    n_pages, hk, page_tokens, d = k_cache.shape
+    if (hk, d) != (n_kv_heads, head_dim) or v_cache.shape != k_cache.shape or k_cache.dtype != q_out.dtype or v_cache.dtype != q_out.dtype:
+        raise KernelError("qknorm_rope_kvwrite: cache shape or dtype does not fit the heads")
+    if rotary_dim % 2 or rotary_dim > head_dim or cos_sin.shape[1] != rotary_dim:
+        raise KernelError("qknorm_rope_kvwrite: rotary width does not fit")
+    if norm_mode == QKNORM_PROJECTION:
+        _dev(q_weight, "q_weight", torch.float32, (qw,))
+        _dev(k_weight, "k_weight", torch.float32, (kw,))
+    elif norm_mode != QKNORM_NONE:
+        raise KernelError("qknorm_rope_kvwrite: only a norm over the whole projection, or none, is built")
+    _check(lib().llmx_qknorm_rope_kvwrite(
+        _dev(qkv, "qkv", torch.float32, (rows, qw + 2 * kw)), _dev(q_weight, "q_weight"), _dev(k_weight, "k_weight"),
+        _dev(cos_sin, "cos_sin", torch.float32), _dev(pos, "pos", torch.int32, (rows,)), _dev(row_entry, "row_entry", torch.int32, (rows,)),
+        _dev(tables, "tables", torch.int32), _dev(q_out, "q_out", shape=(rows, qw)), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
+        _code(q_out.dtype), float(eps), rows, n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, tables.shape[1],
+        1 if write_kv else 0, _stream()), "qknorm_rope_kvwrite")
+
+
+def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
+                    tables: torch.Tensor, out: torch.Tensor, scale: float, n_heads: int, window: int = 0) -> None:
+    rows = q.shape[0]
+    n_pages, n_kv_heads, page_tokens, head_dim = k_cache.shape
+    if q.shape[1] != n_heads * head_dim or out.shape != q.shape or q.dtype != k_cache.dtype or out.dtype != q.dtype:
+        raise KernelError("paged_attention: shapes or dtypes do not agree")
+    if head_dim > 256 or n_heads % n_kv_heads:
+        raise KernelError(f"paged_attention: head_dim {head_dim} above 256 or heads {n_heads} not a multiple of KV heads {n_kv_heads}")
+    _check(lib().llmx_paged_attention_generic(
+        _dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache", shape=k_cache.shape), _dev(pos, "pos", torch.int32, (rows,)),
+        _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32), _dev(out, "out"), _code(q.dtype),
+        float(scale), rows, n_heads, n_kv_heads, head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention")
+
+
+def route_topk(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
+               normalize: bool, scale: float) -> None:
+    rows, n_experts = z.shape
+    if n_experts > 1024 or k > 256 or k > n_experts:
+        raise KernelError(f"route_topk takes at most 1024 experts and 256 picks, not {n_experts} and {k}")
+    _check(lib().llmx_route_topk(_dev(z, "z", torch.float32), _dev(bias, "bias", torch.float32, (n_experts,)),
+                                 _dev(ids, "ids", torch.int32, (rows, k)), _dev(weights, "weights", torch.float32, (rows, k)),
+                                 rows, n_experts, k, score, 1 if normalize else 0, float(scale), _stream()), "route_topk")
+
+
+def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor) -> None:
+    n_pairs = ids.numel()
+    _check(lib().llmx_moe_align(_dev(ids, "ids", torch.int32), n_pairs, n_experts, _dev(counts, "counts", torch.int32, (n_experts,)),
+                                _dev(offsets, "offsets", torch.int32, (n_experts + 1,)), _dev(pairs, "pairs", torch.int32, (n_pairs,)),
+                                _stream()), "moe_align")
+
+
+def moe_combine(x: torch.Tensor, y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, accumulate: bool = True) -> None:
+    rows, width = x.shape
+    k = ids.shape[1]
+    _check(lib().llmx_moe_combine(_dev(x, "x", torch.float32), _dev(y, "y", torch.float32, (rows * k, width)),
+                                  _dev(ids, "ids", torch.int32, (rows, k)), _dev(weights, "weights", torch.float32, (rows, k)),
+                                  rows, k, width, 1 if accumulate else 0, _stream()), "moe_combine")
+
+
+def fill_i32(t: torch.Tensor, value: int) -> None:
+    _check(lib().llmx_fill_i32(_dev(t, "t", torch.int32), int(value), t.numel(), _stream()), "fill_i32")
+
+
+def fill_random(t: torch.Tensor, key: int, kind: int, a: float, b: float) -> None:
+    """Seeded fill: kind 0 = a + b * normal, kind 1 = uniform in [a, b); element i depends on (key, i) only."""
+    _check(lib().llmx_fill_random(_dev(t, "t"), _code(t.dtype), t.numel(), key & ((1 << 64) - 1), int(kind), float(a), float(b),
+                                  _stream()), "fill_random")
+
+
+def argmax_rows(scores: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Tensor] = None) -> None:
+    rows, n = scores.shape
+    _check(lib().llmx_argmax_rows(_dev(scores, "scores", torch.float32), _dev(skip, "skip", torch.int32, (rows,)),
+                                  _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()), "argmax_rows")
+
+
+def sample_all(scores: torch.Tensor, temp: torch.Tensor, unit: torch.Tensor, out: torch.Tensor, min_p: Optional[torch.Tensor] = None,
+               skip: Optional[torch.Tensor] = None) -> None:
+    rows, n = scores.shape
+    _check(lib().llmx_sample_all(_dev(scores, "scores", torch.float32), _dev(temp, "temp", torch.float32, (rows,)),
+                                 _dev(unit, "unit", torch.float32, (rows,)), _dev(min_p, "min_p", torch.float32, (rows,)),
+                                 _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()),
+           "sample_all")

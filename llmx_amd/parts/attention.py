@@ -1,0 +1,88 @@
+"""Causal grouped-query softmax attention over the paged cache.
+
+Per row: q, k, v projections of the normed input (no biases); an optional RMSNorm over the whole q and the whole k
+projection; rotation of the first `rotary_dim` values of each head at the row's position; k and v written to the
+request's pages; softmax(q.k * head_dim^-1/2) over keys 0..p (or the last `window`) of the same request, head h reading
+KV head h / (heads / kv_heads); output projection.  Formula order: /root/reference/src/backends/cpu/cpu_backend.hpp:971-1104
+(attention), :1461-1480 (rotation); the norm over the whole projection is this architecture's variant of the
+reference's per-head norm (/root/reference/src/model/arch/minimax_m3.hpp:258-259).
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .. import ops
+from .base import BuildContext, LayerCache, Mixer, build_part, register
+from .spec import KVNeed, PartSpec, TensorSpec
+
+_NORM_MODES = {"none": ops.QKNORM_NONE, "projection": ops.QKNORM_PROJECTION}
+
+
+class Attention(Mixer):
+    """params: hidden, heads, kv_heads, head_dim, qk_norm ("projection" | "none"), eps, window (None | int), position (PartSpec)."""
+
+    def __init__(self, params, prefix, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        p = params
+        self.hidden = int(p["hidden"])
+        self.heads = int(p["heads"])
+        self.kv_heads = int(p["kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.eps = float(p.get("eps", 0.0))
+        self.window = p.get("window")
+        if self.heads % self.kv_heads:
+            raise ValueError("the head count must be divisible by the KV head count")
+        if p.get("qk_norm", "none") not in _NORM_MODES:
+            raise ValueError(f"qk_norm {p.get('qk_norm')!r} is not one of {sorted(_NORM_MODES)}")
+        self.norm_mode = _NORM_MODES[p.get("qk_norm", "none")]
+        self.position = build_part("position", p.get("position") or PartSpec("none"), ctx)
+        self.scale = float(np.float32(1.0) / np.sqrt(np.float32(self.head_dim)))
+        self.q_width = self.heads * self.head_dim
+        self.kv_width = self.kv_heads * self.head_dim
+        self.wqkv = self.wo = self.q_norm = self.k_norm = None
+
+    def cache_need(self):
+        return KVNeed(self.kv_heads, self.head_dim, self.window)
+
+    def tensor_specs(self, available):
+        specs = [
+            TensorSpec(self.name("q_proj.weight"), (self.q_width, self.hidden)),
+            TensorSpec(self.name("k_proj.weight"), (self.kv_width, self.hidden)),
+            TensorSpec(self.name("v_proj.weight"), (self.kv_width, self.hidden)),
+            TensorSpec(self.name("o_proj.weight"), (self.hidden, self.q_width)),
+        ]
+        if self.norm_mode == ops.QKNORM_PROJECTION:
+            specs += [TensorSpec(self.name("q_norm.weight"), (self.q_width,), "norm"),
+                      TensorSpec(self.name("k_norm.weight"), (self.kv_width,), "norm")]
+        return specs
+
+    def load(self, tensors):
+        q, k, v = (tensors[self.name(n + "_proj.weight")] for n in "qkv")
+        if not (q.dtype == k.dtype == v.dtype):
+            raise ValueError(f"{self.prefix}: q, k and v projections are stored in different types")
+        # one product for the three projections: rows q | k | v
+        self.wqkv = torch.cat([q, k, v], dim=0).contiguous()
+        self.wo = tensors[self.name("o_proj.weight")]
+        if self.norm_mode == ops.QKNORM_PROJECTION:
+            self.q_norm = tensors[self.name("q_norm.weight")]
+            self.k_norm = tensors[self.name("k_norm.weight")]
+
+    def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
+        T = step.rows
+        act = step.act_dtype
+        qkv = step.buf("attention.qkv", (T, self.q_width + 2 * self.kv_width), torch.float32)
+        ops.gemm(h, self.wqkv, qkv)
+        q = step.buf("attention.q", (T, self.q_width), act)
+        cos_sin, rotary = self.position.rotation()
+        tables = step.tables(cache.group)
+        ops.qknorm_rope_kvwrite(qkv, self.q_norm, self.k_norm, cos_sin, step.positions, step.row_entry, tables, q, cache.k, cache.v,
+                                self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode, write_kv=cache.writes)
+        o = step.buf("attention.out", (T, self.q_width), act)
+        ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
+                            window=int(self.window or 0))
+        ops.gemm(o, self.wo, out, ops.EPI_ADD if accumulate else ops.EPI_STORE)
+
+
+register("mixer", "attention", Attention)

@@ -1,0 +1,214 @@
+"""The engine against the plain implementation, under every way of cutting the same tokens into steps.
+
+For each tiny configuration and both dtypes: each request alone and whole; most of it in one step and the last 32
+tokens one by one; portions of changing size down to two tokens; and mixed, up to four live requests, portions of some
+beside decoded tokens of others, with so few pages that they are used again.  In float32 the cuttings must agree with
+each other bit for bit (every kernel's per-row arithmetic is independent of the batch) and with the plain
+implementation within F32_TOL; in bfloat16 with the plain implementation rounded at the same places within BF16_TOL.
+"""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+import helpers
+from helpers import TINY, RoutingRecorder, model_folder, plain_logits, plain_logits_with_picks, portions, tokens_for
+
+pytestmark = pytest.mark.gpu
+
+# Bounds on |engine - plain| over all logits, relative to the largest |logit| of the sequence.
+# float32: the engine sums in float32 in its own order, the plain implementation in float64.
+F32_TOL = 2e-5
+# bfloat16: both round at the same places; what is left are float32 sums of bfloat16 products whose last-bit
+# differences flip a bfloat16 rounding (2^-8 relative) of single activations here and there.  Such a flip can also
+# turn a router's near-tie (the tiny models' closest keys lie 1e-5 apart), so in bfloat16 the plain implementation is
+# given the engine's picks, after checking that each pick's key is within rounding of the best k.
+BF16_TOL = 2e-2
+
+LENGTHS = {"A": (5, 17, 32, 75), "B": (1, 9, 23, 40, 67)}
+
+
+def make_engine(name, dtype, kv_tokens=1024, max_requests=8):
+    from llmx_amd.engine import Engine
+    return Engine.load(model_folder(name), dtype=dtype, kv_tokens=kv_tokens, page_tokens=TINY[name][2], max_requests=max_requests)
+
+
+def watch(engine, name, dtype):
+    """In bfloat16 the engine's expert picks are recorded for the comparison; float32 must pick as the plain router does."""
+    engine.observer = RoutingRecorder(TINY[name][0]["num_hidden_layers"]) if dtype == "bfloat16" else None
+    return engine
+
+
+@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16")],
+                ids=lambda p: f"{p[0]}-{p[1]}")
+def setup(request):
+    name, dtype = request.param
+    return name, dtype, watch(make_engine(name, dtype), name, dtype)
+
+
+def run_whole(engine, rid, tokens):
+    from llmx_amd.engine import StepEntry
+    engine.add_request(rid)
+    logits = engine.step([StepEntry(rid, tokens, list(range(len(tokens))))]).clone()
+    engine.end_request(rid)
+    return logits.cpu()
+
+
+def run_cut(engine, rid, tokens, cuts):
+    from llmx_amd.engine import StepEntry
+    engine.add_request(rid)
+    rows = []
+    for a, b in cuts:
+        rows.append(engine.step([StepEntry(rid, tokens[a:b], list(range(b - a)))]).clone())
+    engine.end_request(rid)
+    return torch.cat(rows).cpu()
+
+
+def check_against_plain(name, dtype, length, seed, got, engine=None, rid=None):
+    if dtype == "bfloat16":
+        want = plain_logits_with_picks(name, tokens_for(name, length, seed), engine.observer.of(rid, length))
+    else:
+        want = plain_logits(name, length, seed, False)
+    tol = F32_TOL if dtype == "float32" else BF16_TOL
+    scale = float(want.abs().max())
+    err = float((got.double() - want).abs().max())
+    assert err <= tol * scale, f"{name} {dtype} length {length}: max error {err:.3e} against scale {scale:.3e}"
+
+
+def test_whole_alone(setup):
+    name, dtype, engine = setup
+    for length in LENGTHS[name]:
+        tokens = tokens_for(name, length, 0)
+        got = run_whole(engine, "w", tokens)
+        assert got.shape == (length, TINY[name][0]["vocab_size"])
+        assert torch.isfinite(got).all()
+        check_against_plain(name, dtype, length, 0, got, engine, "w")
+    assert engine.cache.pages_in_use() == 0
+
+
+def test_last_32_one_by_one(setup):
+    name, dtype, engine = setup
+    length = 75 if name == "A" else 67
+    tokens = tokens_for(name, length, 0)
+    whole = run_whole(engine, "w", tokens)
+    cuts = [(0, length - 32)] + [(i, i + 1) for i in range(length - 32, length)]
+    got = run_cut(engine, "d", tokens, cuts)
+    check_against_plain(name, dtype, length, 0, got, engine, "d")
+    if dtype == "float32":
+        assert torch.equal(got, whole), "decoding one by one differs from the whole prompt in float32"
+
+
+def test_portions_of_changing_size(setup):
+    name, dtype, engine = setup
+    length = 75 if name == "A" else 67
+    tokens = tokens_for(name, length, 0)
+    whole = run_whole(engine, "w", tokens)
+    got = run_cut(engine, "p", tokens, portions(length))
+    check_against_plain(name, dtype, length, 0, got, engine, "p")
+    if dtype == "float32":
+        assert torch.equal(got, whole), "portions differ from the whole prompt in float32"
+
+
+def test_first_tokens(setup):
+    """The first tokens of a sequence: lengths 1 and 2, and the first rows of a longer one."""
+    name, dtype, engine = setup
+    for length in (1, 2, 3):
+        tokens = tokens_for(name, 67 if name == "B" else 75, 0)[:length]
+        got = run_whole(engine, "f", tokens)
+        if dtype == "bfloat16":
+            want = plain_logits_with_picks(name, tokens, engine.observer.of("f", length))
+        else:
+            want = plain_logits(name, 67 if name == "B" else 75, 0, False)[:length]
+        tol = F32_TOL if dtype == "float32" else BF16_TOL
+        assert float((got.double() - want).abs().max()) <= tol * float(want.abs().max())
+
+
+def test_mixed_requests_with_page_reuse(setup):
+    """Up to four live requests; portions of some beside decoded tokens of others; the pool is so small that pages
+    freed by finished requests are handed out again."""
+    from llmx_amd.engine import StepEntry
+    name, dtype, _ = setup
+    page = TINY[name][2]
+    lengths = [40, 23, 67, 9, 31, 52]
+    seeds = [1, 2, 3, 4, 5, 6]
+    # four live requests of at most 67 tokens: pages for 4 * 72 tokens, far fewer than all six hold together
+    engine = watch(make_engine(name, dtype, kv_tokens=4 * (-(-67 // page) * page), max_requests=4), name, dtype)
+    toks = [tokens_for(name, n, s) for n, s in zip(lengths, seeds)]
+    got = {i: [] for i in range(len(lengths))}
+    at = {i: 0 for i in range(len(lengths))}
+    waiting = list(range(len(lengths)))
+    live = []
+    used_pages = set()
+    step_no = 0
+    while waiting or live:
+        while waiting and len(live) < 4:
+            i = waiting.pop(0)
+            engine.add_request(i)
+            live.append(i)
+        entries = []
+        for slot, i in enumerate(live):
+            n_left = lengths[i] - at[i]
+            prefill_end = lengths[i] - 8          # the last 8 tokens of every request are decoded one by one
+            if at[i] >= prefill_end:
+                n = 1
+            else:
+                n = min((5, 2, 11, 3)[(step_no + slot) % 4], prefill_end - at[i])
+            if (step_no + i) % 5 == 4 and len(live) > 1:
+                continue                           # a request may be left out of a step and go on later
+            entries.append(StepEntry(i, toks[i][at[i]:at[i] + n], list(range(n))))
+        if entries:
+            logits = engine.step(entries).clone().cpu()
+            row = 0
+            for e in entries:
+                n = len(e.tokens)
+                got[e.request].append(logits[row:row + n])
+                row += n
+                at[e.request] += n
+                for g in range(len(engine.cache.groups)):
+                    used_pages.update(engine.cache.table(e.request, g))
+        for i in list(live):
+            if at[i] == lengths[i]:
+                engine.end_request(i)
+                live.remove(i)
+        step_no += 1
+        assert step_no < 1000
+    assert engine.cache.pages_in_use() == 0
+    total_pages = sum(-(-n // page) for n in lengths)
+    assert len(used_pages) < total_pages, "the pool was large enough that no page was used again"
+    alone = make_engine(name, dtype)
+    for i, (n, s) in enumerate(zip(lengths, seeds)):
+        mixed = torch.cat(got[i])
+        check_against_plain(name, dtype, n, s, mixed, engine, i)
+        if dtype == "float32":
+            assert torch.equal(mixed, run_whole(alone, "w", toks[i])), f"request {i} in the mix differs from its run alone"
+
+
+def test_long_decoding(setup):
+    """A short prompt, then 200 tokens decoded one by one across many page edges."""
+    name, dtype, engine = setup
+    length = 8 + 200
+    tokens = tokens_for(name, length, 7)
+    cuts = [(0, 8)] + [(i, i + 1) for i in range(8, length)]
+    got = run_cut(engine, "l", tokens, cuts)
+    check_against_plain(name, dtype, length, 7, got, engine, "l")
+
+
+def test_refusals_leave_nothing_behind(setup):
+    from llmx_amd.engine import StepEntry, StepError
+    name, dtype, engine = setup
+    vocab = TINY[name][0]["vocab_size"]
+    engine.add_request("r")
+    before = engine.cache.pages_in_use()
+    with pytest.raises(StepError, match="outside the embedding"):
+        engine.step([StepEntry("r", [1, vocab], [0])])
+    with pytest.raises(StepError, match="twice"):
+        engine.step([StepEntry("r", [1], [0]), StepEntry("r", [2], [0])])
+    with pytest.raises(StepError, match="not open"):
+        engine.step([StepEntry("nobody", [1], [0])])
+    with pytest.raises(StepError, match="no tokens"):
+        engine.step([StepEntry("r", [], [])])
+    with pytest.raises(StepError, match="empty"):
+        engine.step([])
+    assert engine.cache.pages_in_use() == before and engine.length("r") == 0
+    engine.end_request("r")
