@@ -17,9 +17,15 @@ def __getattr__(name):
     if name in ("Engine", "StepEntry", "StepError"):
         from . import engine
         return getattr(engine, name)
-    if name in ("generate", "SamplingParams", "Scheduler", "Request"):
+    if name in ("generate", "Generator"):
         from .engine import generation
         return getattr(generation, name)
+    if name in ("Scheduler", "Request"):
+        from .engine import scheduler
+        return getattr(scheduler, name)
+    if name == "SamplingParams":
+        from .sampling import SamplingParams
+        return SamplingParams
     if name == "write_random_model":
         from .weights.folder import write_random_model
         return write_random_model
@@ -27,4 +33,4 @@ def __getattr__(name):
 
 
 __all__ = ["ConfigError", "MiniMaxM3Config", "RandomInit", "WeightsError", "Engine", "StepEntry", "StepError", "generate",
-           "SamplingParams", "Scheduler", "Request", "write_random_model"]
+           "Generator", "SamplingParams", "Scheduler", "Request", "write_random_model"]

@@ -1,0 +1,214 @@
+"""The command line, in the reference's manner (/root/reference/src/cli/main.cpp): `llmx generate MODEL [PROMPT]`.
+
+Flags keep the reference's names and meanings where it has them (main.cpp:2018-2038 sampling, :541-574 execution):
+--max-tokens/-n, --temp, --topk, --topp, --min-p, --penalty, --presence-penalty, --frequency-penalty, --seed,
+--ignore-eos, --dtype, --ubatch, --kv-tokens, --verbose.  There is no tokenizer here: a prompt is a list of token ids
+(comma or space separated), given on the line, with --file, or made up with --prompt-len.  A usage error exits with
+status 2 (main.cpp:100-103); a flag given twice is refused (:129-159).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import re
+import sys
+import time
+from pathlib import Path
+
+
+class _Once(argparse.Action):
+    """A second value for the same setting is refused rather than overwriting the first."""
+
+    def __call__(self, parser, namespace, values, option_string=None):
+        seen = getattr(namespace, "_given", set())
+        if self.dest in seen:
+            parser.error(f"{option_string}: given twice")
+        seen.add(self.dest)
+        namespace._given = seen
+        setattr(namespace, self.dest, True if self.nargs == 0 else values)
+
+
+def _add_sampling(p):
+    from .sampling.params import SamplingParams
+    d = SamplingParams()
+    p.add_argument("--max-tokens", "-n", type=int, default=d.max_tokens, action=_Once, help="tokens generated at most (default %(default)s)")
+    p.add_argument("--temp", type=float, default=d.temp, action=_Once, help="temperature, 0 is greedy (default %(default)s)")
+    p.add_argument("--topk", type=int, default=d.top_k, action=_Once, help="keep the k likeliest tokens, 0 keeps all (default %(default)s)")
+    p.add_argument("--topp", type=float, default=d.top_p, action=_Once, help="nucleus share of the kept weight (default %(default)s)")
+    p.add_argument("--min-p", type=float, default=d.min_p, action=_Once, help="drop tokens below this share of the likeliest (default %(default)s)")
+    p.add_argument("--penalty", type=float, default=d.penalty, action=_Once, help="repetition penalty, 1 is none (default %(default)s)")
+    p.add_argument("--presence-penalty", type=float, default=d.presence_penalty, action=_Once)
+    p.add_argument("--frequency-penalty", type=float, default=d.frequency_penalty, action=_Once)
+    p.add_argument("--seed", type=int, default=d.seed, action=_Once, help="0 keeps the fixed default generator state")
+    p.add_argument("--ignore-eos", nargs=0, default=False, action=_Once, help="the end token is never drawn")
+
+
+def _add_exec(p):
+    p.add_argument("--dtype", choices=["f32", "bf16", "float32", "bfloat16"], default="bf16", action=_Once,
+                   help="bf16: the serving path; f32: everything in true 32-bit")
+    p.add_argument("--ubatch", type=int, default=512, action=_Once, help="tokens a step takes at most (default %(default)s)")
+    p.add_argument("--kv-tokens", type=int, default=0, action=_Once, help="the cache's token budget; 0 sizes it to the run")
+    p.add_argument("--page-tokens", type=int, default=16, action=_Once, help="tokens a cache page holds (default %(default)s)")
+    p.add_argument("--max-seqs", type=int, default=8, action=_Once, help="requests running together at most (default %(default)s)")
+    p.add_argument("--verbose", nargs=0, default=False, action=_Once)
+
+
+def _ids(text: str):
+    parts = [t for t in re.split(r"[,\s]+", text.strip()) if t]
+    try:
+        return [int(t) for t in parts]
+    except ValueError:
+        raise SystemExit2(f"a prompt is a list of token ids, not {text[:40]!r}")
+
+
+class SystemExit2(Exception):
+    pass
+
+
+def _params(a):
+    from .sampling.params import SamplingParams
+    return SamplingParams(max_tokens=a.max_tokens, temp=a.temp, top_k=a.topk, top_p=a.topp, min_p=a.min_p, penalty=a.penalty,
+                          presence_penalty=a.presence_penalty, frequency_penalty=a.frequency_penalty, seed=a.seed,
+                          ignore_eos=bool(a.ignore_eos)).validate()
+
+
+def _lcg_ids(n: int, vocab: int, seed: int = 1):
+    """Fixed token ids spread over the vocabulary (the reference's bench ids, main.cpp:1185-1189, are an LCG too)."""
+    x, out = seed & 0xFFFFFFFF, []
+    for _ in range(n):
+        x = (x * 1664525 + 1013904223) & 0xFFFFFFFF
+        out.append((x >> 8) % vocab)
+    return out
+
+
+def cmd_generate(a) -> int:
+    from .engine import Engine
+    from .engine.generation import Generator
+    from .engine.scheduler import Request
+    from .models import read_model_dir
+    params = _params(a)
+    cfg, _ = read_model_dir(a.model)
+    if a.file:
+        prompts = [_ids(line) for line in Path(a.file).read_text().splitlines() if line.strip()]
+    elif a.prompt is not None:
+        prompts = [_ids(a.prompt)]
+    elif a.prompt_len:
+        prompts = [_lcg_ids(a.prompt_len, cfg.vocab_size)]
+    else:
+        raise SystemExit2("generate needs a prompt: token ids on the line, --file, or --prompt-len")
+    if any(not p for p in prompts):
+        raise SystemExit2("generate: empty prompt")
+    need = sum(len(p) + params.max_tokens for p in prompts[:a.max_seqs]) if len(prompts) > 1 else len(prompts[0]) + params.max_tokens
+    kv_tokens = a.kv_tokens or max(need + a.page_tokens * a.max_seqs, max(len(p) for p in prompts) + params.max_tokens)
+    engine = Engine.load(a.model, dtype=a.dtype, kv_tokens=kv_tokens, page_tokens=a.page_tokens, max_requests=a.max_seqs)
+    gen = Generator(engine, a.max_seqs, a.ubatch)
+    for i, p in enumerate(prompts):
+        import copy
+        gen.submit(Request(i, p, copy.copy(params)))
+    if a.verbose:
+        print(f"prompt tokens: {sum(len(p) for p in prompts)}")
+    import torch
+    finished = gen.run()
+    torch.cuda.synchronize()
+    for i in range(len(prompts)):
+        print(" ".join(str(t) for t in finished[i].generated))
+    st = gen.stats
+    pp_ms, tg_ms = st.prompt_seconds * 1e3, st.decode_seconds * 1e3
+    print(f"pp: {st.prompt_tokens} tok, {pp_ms:.0f} ms, {st.prompt_tokens / max(pp_ms, 1e-9) * 1e3:.2f} tok/s", file=sys.stderr)
+    print(f"tg: {st.generated_tokens} tok, {tg_ms:.0f} ms, {st.generated_tokens / max(tg_ms, 1e-9) * 1e3:.2f} tok/s", file=sys.stderr)
+    if a.verbose:
+        print(f"kv: allocated {engine.cache_bytes()} bytes", file=sys.stderr)
+        for i in range(len(prompts)):
+            print("ids: " + ",".join(str(t) for t in finished[i].generated) + f"  ({finished[i].finish_reason})", file=sys.stderr)
+    return 0
+
+
+def cmd_logits(a) -> int:
+    """Top-N logits of the last positions, whole or token by token (the reference's `llmx logits`, main.cpp:934-980)."""
+    from .engine import Engine, StepEntry
+    ids = _ids(a.prompt) if a.prompt is not None else _ids(Path(a.file).read_text())
+    engine = Engine.load(a.model, dtype=a.dtype, kv_tokens=a.kv_tokens or len(ids) + a.page_tokens, page_tokens=a.page_tokens, max_requests=1)
+    engine.add_request(0)
+    last = min(a.last or 1, len(ids))
+    rows = []
+    if a.per_token:
+        for i, t in enumerate(ids):
+            lg = engine.step([StepEntry(0, [t], [0])])
+            if i >= len(ids) - last:
+                rows.append(lg[0].clone())
+    else:
+        for s in range(0, len(ids), a.ubatch):
+            part = ids[s:s + a.ubatch]
+            want = [i - s for i in range(max(s, len(ids) - last), s + len(part))]
+            lg = engine.step([StepEntry(0, part, want)])
+            rows.extend(r.clone() for r in lg)
+    print(f"tokens: {len(ids)}")
+    for off, row in enumerate(rows):
+        vals, idx = row.topk(min(a.top, row.numel()))
+        print(f"{len(ids) - len(rows) + off} " + " ".join(f"{int(i)} {float(v):.6f}" for v, i in zip(vals, idx)))
+    return 0
+
+
+def cmd_random(a) -> int:
+    """Writes a model folder (config.json, model.safetensors) with seeded random weights."""
+    from .models import read_config
+    from .weights import RandomInit
+    from .weights.folder import write_random_model
+    cfg = read_config(json.loads(Path(a.config).read_text()))
+    write_random_model(a.out, cfg, RandomInit(seed=a.seed, std=a.std, norm_std=a.norm_std, bias_range=a.bias_range, storage=a.storage))
+    print(a.out)
+    return 0
+
+
+def build_parser():
+    ap = argparse.ArgumentParser(prog="llmx", description="MiniMax-M3 on one MI355X: generate, logits, random, bench")
+    sub = ap.add_subparsers(dest="command", required=True)
+    g = sub.add_parser("generate", help="generate tokens after a prompt of token ids")
+    g.add_argument("model", help="model folder (config.json + model.safetensors)")
+    g.add_argument("prompt", nargs="?", default=None, help="token ids, comma or space separated")
+    g.add_argument("--file", "-f", default=None, help="a file with one prompt of token ids per line")
+    g.add_argument("--prompt-len", type=int, default=0, help="make up a prompt of this many fixed token ids")
+    _add_sampling(g)
+    _add_exec(g)
+    g.set_defaults(run=cmd_generate)
+    l = sub.add_parser("logits", help="top logits of the last positions of a prompt")
+    l.add_argument("model")
+    l.add_argument("prompt", nargs="?", default=None)
+    l.add_argument("--file", "-f", default=None)
+    l.add_argument("--last", type=int, default=0, help="report this many final positions")
+    l.add_argument("--per-token", action="store_true", help="feed the tokens one step each")
+    l.add_argument("--top", type=int, default=10)
+    _add_exec(l)
+    l.set_defaults(run=cmd_logits)
+    r = sub.add_parser("random", help="write a model folder with seeded random weights")
+    r.add_argument("--config", required=True, help="a config.json")
+    r.add_argument("--out", required=True)
+    r.add_argument("--seed", type=int, default=0)
+    r.add_argument("--std", type=float, default=0.02)
+    r.add_argument("--norm-std", type=float, default=0.0)
+    r.add_argument("--bias-range", type=float, default=0.0)
+    r.add_argument("--storage", choices=["bfloat16", "float32"], default="bfloat16")
+    r.set_defaults(run=cmd_random)
+    b = sub.add_parser("bench", help="decode and prefill throughput of a random-weight model (see bench.py)")
+    b.add_argument("rest", nargs=argparse.REMAINDER)
+    b.set_defaults(run=lambda a: __import__("runpy").run_path(str(Path(__file__).resolve().parent.parent / "bench.py"), run_name="__main__") and 0)
+    return ap
+
+
+def main(argv=None) -> int:
+    ap = build_parser()
+    try:
+        a = ap.parse_args(argv)
+        return a.run(a)
+    except SystemExit2 as e:
+        print(f"llmx: {e}", file=sys.stderr)
+        return 2
+    except ValueError as e:
+        # configuration, weights, sampling and scheduling refusals carry their own text
+        print(f"llmx: {e}", file=sys.stderr)
+        return 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -121,3 +121,232 @@ extern "C" int llmx_sample_all(const float* scores, const float* temp, const flo
     hipLaunchKernelGGL(sample_all_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, unit, min_p, skip, out, n);
     return LLMX_CHECK_LAUNCH();
 }
+
+// ---------------------------------------------------------------------------
+// Penalties, in place on the logits rows, one thread per (row, seen token): the repetition penalty divides a positive
+// logit and multiplies a negative one, once however often the token was seen; then presence + frequency * count comes
+// off (sampler.hpp:270-289).  Every (row, id) appears once in the list, so the in-place update has no race.
+__global__ void penalize_kernel(float* __restrict__ scores, const int* __restrict__ rows, const int* __restrict__ ids,
+                                const int* __restrict__ counts, const float* __restrict__ penalty, const float* __restrict__ presence,
+                                const float* __restrict__ frequency, int n_seen, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_seen) return;
+    const int r = rows[i], id = ids[i];
+    if (id < 0 || id >= n) return;
+    float* at = scores + (size_t)r * n + id;
+    float v = *at;
+    const float p = penalty[r];
+    if (p > 0.0f && p != 1.0f) v = v > 0.0f ? v / p : v * p;
+    if (presence[r] != 0.0f || frequency[r] != 0.0f) v -= presence[r] + frequency[r] * (float)counts[i];
+    *at = v;
+}
+
+extern "C" int llmx_penalize(float* scores, const int* rows, const int* ids, const int* counts, const float* penalty,
+                             const float* presence, const float* frequency, int n_seen, int n, hipStream_t stream) {
+    if (n_seen <= 0) return 0;
+    hipLaunchKernelGGL(penalize_kernel, dim3((n_seen + 255) / 256), dim3(256), 0, stream, scores, rows, ids, counts, penalty, presence,
+                       frequency, n_seen, n);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// Top-k (k <= SAMPLE_MAX_KEEP), then top-p, then min-p, then the draw (sampler.hpp:293-378).
+//  1. the k best by (score descending, id ascending): a radix select over the scores' ordered bits finds the k-th score,
+//     tokens above it are kept, tokens equal to it are kept lowest id first until k are held;
+//  2. the kept tokens are gathered in id order; weight = exp((score - best) / temp); their sum in id order in double;
+//  3. without top-p the draw walks the kept tokens in id order (weights below min_p count 0);
+//     with top-p the kept tokens are ranked, the nucleus is the shortest ranked prefix reaching top_p of the sum, min_p
+//     cuts its tail, and the draw walks the nucleus best first.
+#define SAMPLE_MAX_KEEP 1024
+
+__device__ __forceinline__ uint32_t ordered_bits(float score) {
+    score += 0.0f;  // -0 becomes +0, so the two zeros tie
+    const uint32_t b = __float_as_uint(score);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// exclusive scan of one int per thread over the block, in thread order; returns the exclusive prefix, total in *total
+__device__ int block_exclusive_scan(int v, int* scratch, int* total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int inc = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += up;
+    }
+    if (lane == 63) scratch[wave] = inc;
+    __syncthreads();
+    int before = 0, all = 0;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) {
+        if (w == wave) before = all;
+        all += scratch[w];
+    }
+    __syncthreads();
+    *total = all;
+    return before + inc - v;
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS) sample_topk_kernel(const float* __restrict__ scores, const float* __restrict__ temp,
+                                                                    const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                                                    const float* __restrict__ min_p, const float* __restrict__ unit,
+                                                                    const int* __restrict__ skip, int* __restrict__ out, int n) {
+    __shared__ int hist[256];
+    __shared__ int scan_scratch[SAMPLE_WAVES];
+    __shared__ uint32_t prefix_s;
+    __shared__ int remaining_s;
+    __shared__ int kept_id[SAMPLE_MAX_KEEP];
+    __shared__ float kept_score[SAMPLE_MAX_KEEP];
+    __shared__ float kept_w[SAMPLE_MAX_KEEP];
+    __shared__ int ranked[SAMPLE_MAX_KEEP];  // ranked[i] = place in kept_* of the i-th best
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float* s = scores + (size_t)r * n;
+    const int sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
+    const int m = sk < n ? n - 1 : n;
+    int keep = top_k[r];
+    if (keep <= 0 || keep > m) keep = m;  // the host sends only rows with keep <= SAMPLE_MAX_KEEP
+    if (keep > SAMPLE_MAX_KEEP) keep = SAMPLE_MAX_KEEP;
+
+    // 1. radix select of the keep-th largest ordered score, 8 bits a pass from the top
+    if (tid == 0) {
+        prefix_s = 0;
+        remaining_s = keep;
+    }
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 24 - 8 * pass;
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        const uint32_t prefix = prefix_s;
+        const uint32_t mask = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8));
+        for (int i = tid; i < n; i += SAMPLE_THREADS) {
+            if (i == sk) continue;
+            const uint32_t b = ordered_bits(s[i]);
+            if ((b & mask) == prefix) atomicAdd(&hist[(b >> shift) & 255u], 1);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int left = remaining_s, bin = 255;
+            for (; bin > 0; --bin) {
+                if (hist[bin] >= left) break;
+                left -= hist[bin];
+            }
+            prefix_s = prefix | ((uint32_t)bin << shift);
+            remaining_s = left;  // how many of this bin (finally: of the threshold's equals) are kept
+        }
+        __syncthreads();
+    }
+    const uint32_t threshold = prefix_s;
+    const int need_equal = remaining_s;
+
+    // 2. gather the kept tokens in id order: thread t owns the contiguous ids [t*c, (t+1)*c)
+    const int chunk = (n + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+    const int begin = min(n, tid * chunk), end = min(n, begin + chunk);
+    int n_equal = 0;
+    for (int i = begin; i < end; ++i)
+        if (i != sk && ordered_bits(s[i]) == threshold) ++n_equal;
+    int total_equal;
+    const int equal_before = block_exclusive_scan(n_equal, scan_scratch, &total_equal);
+    int n_mine = 0;
+    {
+        int eq = equal_before;
+        for (int i = begin; i < end; ++i) {
+            if (i == sk) continue;
+            const uint32_t b = ordered_bits(s[i]);
+            if (b > threshold || (b == threshold && eq++ < need_equal)) ++n_mine;
+        }
+    }
+    int n_kept;
+    int at = block_exclusive_scan(n_mine, scan_scratch, &n_kept);
+    {
+        int eq = equal_before;
+        for (int i = begin; i < end; ++i) {
+            if (i == sk) continue;
+            const uint32_t b = ordered_bits(s[i]);
+            if (b > threshold || (b == threshold && eq++ < need_equal)) {
+                if (at < SAMPLE_MAX_KEEP) {
+                    kept_id[at] = i;
+                    kept_score[at] = s[i];
+                }
+                ++at;
+            }
+        }
+    }
+    __syncthreads();
+    if (n_kept > SAMPLE_MAX_KEEP) n_kept = SAMPLE_MAX_KEEP;
+
+    // rank of each kept token: how many kept tokens are better (higher score, or equal score and lower id)
+    for (int i = tid; i < n_kept; i += SAMPLE_THREADS) {
+        const uint32_t bi = ordered_bits(kept_score[i]);
+        int better = 0;
+        for (int j = 0; j < n_kept; ++j) {
+            const uint32_t bj = ordered_bits(kept_score[j]);
+            better += (bj > bi) || (bj == bi && j < i);  // kept_* is in id order, so j < i is the lower id
+        }
+        ranked[better] = i;
+    }
+    __syncthreads();
+    const float best_score = kept_score[ranked[0]];
+    const float tmp = temp[r];
+    for (int i = tid; i < n_kept; i += SAMPLE_THREADS) kept_w[i] = expf((kept_score[i] - best_score) / tmp);
+    __syncthreads();
+
+    // 3. the draw, by one thread in the reference's order
+    if (tid == 0) {
+        const float cut = min_p ? min_p[r] : 0.0f;
+        const float p = top_p[r];
+        int pick = kept_id[ranked[0]];
+        double sum = 0.0;
+        for (int i = 0; i < n_kept; ++i) sum += (double)kept_w[i];
+        if (p >= 1.0f) {
+            if (cut > 0.0f) {
+                sum = 0.0;
+                for (int i = 0; i < n_kept; ++i) {
+                    if (kept_w[i] < cut) kept_w[i] = 0.0f;
+                    sum += (double)kept_w[i];
+                }
+            }
+            const double target = (double)unit[r] * sum;
+            double acc = 0.0;
+            for (int i = 0; i < n_kept; ++i) {
+                acc += (double)kept_w[i];
+                if (target < acc) {
+                    pick = kept_id[i];
+                    break;
+                }
+            }
+        } else {
+            const double goal = (double)p * sum;
+            double nucleus_weight = 0.0;
+            int nucleus = 0;
+            do {
+                nucleus_weight += (double)kept_w[ranked[nucleus]];
+                ++nucleus;
+            } while (nucleus < n_kept && nucleus_weight < goal);
+            if (cut > 0.0f) {
+                int last = nucleus;
+                while (last > 1 && kept_w[ranked[last - 1]] < cut) --last;
+                if (last < nucleus) {
+                    nucleus = last;
+                    nucleus_weight = 0.0;
+                    for (int i = 0; i < nucleus; ++i) nucleus_weight += (double)kept_w[ranked[i]];
+                }
+            }
+            const double target = (double)unit[r] * nucleus_weight;
+            double acc = 0.0;
+            for (int i = 0; i < nucleus; ++i) {
+                acc += (double)kept_w[ranked[i]];
+                if (target < acc) {
+                    pick = kept_id[ranked[i]];
+                    break;
+                }
+            }
+        }
+        out[r] = pick;
+    }
+}
+
+extern "C" int llmx_sample_topk(const float* scores, const float* temp, const int* top_k, const float* top_p, const float* min_p,
+                                const float* unit, const int* skip, int* out, int rows, int n, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n);
+    return LLMX_CHECK_LAUNCH();
+}

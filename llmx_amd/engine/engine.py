@@ -271,6 +271,19 @@ class Engine:
         self.model.head.forward(step, rows, logits)
         return logits
 
+    # -- for measurement ----------------------------------------------------------
+    def assume_context(self, request: Hashable, n: int) -> None:
+        """Marks the request's next n positions as held without computing them: their keys and values are whatever
+        the pages hold.  For measuring decode at a given depth without paying for the prompt; never for serving."""
+        self.cache.prepare(request, n)
+        self.cache.commit(request)
+
+    def fill_cache_random(self, seed: int = 1) -> None:
+        """Writes seeded N(0,1) values into every page of keys and values (see assume_context)."""
+        from ..weights.random_init import mix64
+        for g, store in enumerate(self._kv):
+            ops.fill_random(store, mix64(seed * 1315423911 + g), 0, 0.0, 1.0)
+
     # -- accounting -------------------------------------------------------------
     def weight_bytes(self) -> int:
         seen, total = set(), 0

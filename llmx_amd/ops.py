@@ -63,6 +63,8 @@ def _declare(h) -> None:
         "llmx_moe_align": [P, I, I, P, P, P, P],
         "llmx_argmax_rows": [P, P, P, I, I, P],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
+        "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
+        "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
     }
     for name, args in sigs.items():
         try:
@@ -242,3 +244,25 @@ def sample_all(scores: torch.Tensor, temp: torch.Tensor, unit: torch.Tensor, out
                                  _dev(unit, "unit", torch.float32, (rows,)), _dev(min_p, "min_p", torch.float32, (rows,)),
                                  _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()),
            "sample_all")
+
+
+def sample_topk(scores: torch.Tensor, temp: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,
+                unit: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Tensor] = None) -> None:
+    """Top-k (1..1024 per row), top-p, min-p and the draw; rows whose top_k is outside 1..1024 must not be read from `out`."""
+    rows, n = scores.shape
+    _check(lib().llmx_sample_topk(_dev(scores, "scores", torch.float32), _dev(temp, "temp", torch.float32, (rows,)),
+                                  _dev(top_k, "top_k", torch.int32, (rows,)), _dev(top_p, "top_p", torch.float32, (rows,)),
+                                  _dev(min_p, "min_p", torch.float32, (rows,)), _dev(unit, "unit", torch.float32, (rows,)),
+                                  _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()),
+           "sample_topk")
+
+
+def penalize(scores: torch.Tensor, rows: torch.Tensor, ids: torch.Tensor, counts: torch.Tensor, penalty: torch.Tensor,
+             presence: torch.Tensor, frequency: torch.Tensor) -> None:
+    """In place: for each (rows[i], ids[i]) seen counts[i] times, the repetition, presence and frequency penalties."""
+    W, n = scores.shape
+    n_seen = rows.shape[0]
+    _check(lib().llmx_penalize(_dev(scores, "scores", torch.float32), _dev(rows, "rows", torch.int32), _dev(ids, "ids", torch.int32, (n_seen,)),
+                               _dev(counts, "counts", torch.int32, (n_seen,)), _dev(penalty, "penalty", torch.float32, (W,)),
+                               _dev(presence, "presence", torch.float32, (W,)), _dev(frequency, "frequency", torch.float32, (W,)),
+                               n_seen, n, _stream()), "penalize")

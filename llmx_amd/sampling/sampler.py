@@ -1,0 +1,77 @@
+"""Draws the next token of each wanted row on the device.
+
+Order of operations as the reference's sampler (/root/reference/src/inference/sampler.hpp:258-378): penalties from the
+raw logit, then greedy, or top-k, top-p, min-p and the draw; one uniform number is taken from the request's generator
+per sampled (non-greedy) row, before the branch.
+"""
+
+from __future__ import annotations
+
+from collections import Counter
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import ops
+from .params import SamplingParams, XorShift64
+
+
+class Sampler:
+    def __init__(self, vocab_size: int, device: torch.device):
+        self.vocab = vocab_size
+        self.device = device
+
+    def _f32(self, values) -> torch.Tensor:
+        return torch.tensor(np.asarray(values, dtype=np.float32), device=self.device)
+
+    def _i32(self, values) -> torch.Tensor:
+        return torch.tensor(np.asarray(values, dtype=np.int32), device=self.device)
+
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], generated: Sequence[Sequence[int]],
+               rngs: Sequence[XorShift64], eos: Optional[int]) -> List[int]:
+        """One token id for each row of `logits` [W, vocab]; `generated` holds each row's tokens so far (for the penalties).
+
+        The logits are scratch of the step and are changed in place by the penalties.
+        """
+        W = logits.shape[0]
+        if not (len(params) == len(generated) == len(rngs) == W):
+            raise ValueError("sampler: one set of settings, one history and one generator per row")
+        if W == 0:
+            return []
+        # penalties, in place: one list entry per (row, distinct seen token)
+        rows, ids, counts = [], [], []
+        for r, (p, gen) in enumerate(zip(params, generated)):
+            if p.penalized and gen:
+                for tok, c in Counter(gen).items():
+                    rows.append(r)
+                    ids.append(tok)
+                    counts.append(c)
+        if rows:
+            ops.penalize(logits, self._i32(rows), self._i32(ids), self._i32(counts), self._f32([p.penalty for p in params]),
+                         self._f32([p.presence_penalty for p in params]), self._f32([p.frequency_penalty for p in params]))
+        skip = None
+        if eos is not None and any(p.ignore_eos for p in params):
+            skip = self._i32([eos if p.ignore_eos else -1 for p in params])
+        out = torch.empty(W, dtype=torch.int32, device=self.device)
+        if all(p.greedy for p in params):
+            ops.argmax_rows(logits, out, skip)
+            return out.tolist()
+        units = [0.0 if p.greedy else rng.unit() for p, rng in zip(params, rngs)]
+        temp = self._f32([p.temp for p in params])
+        unit = self._f32(units)
+        min_p = self._f32([p.min_p for p in params])
+        # ids a draw can give: all, less a masked end token; a top_k that leaves them all is no top_k
+        m = [self.vocab - (1 if (eos is not None and p.ignore_eos and 0 <= eos < self.vocab and self.vocab > 1) else 0) for p in params]
+        all_kept = [p.greedy or ((p.top_k <= 0 or p.top_k >= mr) and p.top_p >= 1.0) for p, mr in zip(params, m)]
+        if all(all_kept):
+            ops.sample_all(logits, temp, unit, out, min_p, skip)
+            return out.tolist()
+        # mixed settings: both kernels run over all rows and each row takes the result of its own
+        top = torch.empty(W, dtype=torch.int32, device=self.device)
+        ops.sample_topk(logits, temp, self._i32([p.top_k for p in params]), self._f32([p.top_p for p in params]), min_p, unit, top, skip)
+        if any(all_kept):
+            ops.sample_all(logits, temp, unit, out, min_p, skip)
+            picks_all, picks_top = out.tolist(), top.tolist()
+            return [a if k else t for a, t, k in zip(picks_all, picks_top, all_kept)]
+        return top.tolist()
