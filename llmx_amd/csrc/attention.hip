@@ -5,7 +5,8 @@
 //   pos[t]        absolute position of row t in its request
 //   row_entry[t]  index of the row's request among the step's entries
 //   tables        [n_entries, max_blocks] page ids of each entry in this cache group (-1: page given back)
-// Cache layout per layer and side: [page][kv_head][token_in_page][head_dim].
+// Cache layout per layer: keys [page][kv_head][token_in_page][head_dim], values transposed [page][kv_head][head_dim][token_in_page]
+// (the value product on the matrix cores reads several keys of one dim at a time).
 
 enum : int { QKNORM_NONE = 0, QKNORM_PROJECTION = 1, QKNORM_HEAD = 2 };
 
@@ -85,9 +86,9 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
             const float c = cs[j], s = cs[half + j];
             x = d < half ? fmaf(-y, s, x * c) : fmaf(y, s, x * c);
         }
-        const size_t at = (((size_t)page * a.n_kv_heads + h) * a.page_tokens + slot) * D + d;
-        st(kc + at, x);
-        st(vc + at, row[qw + kw + i]);
+        const size_t head_at = (size_t)page * a.n_kv_heads + h;
+        st(kc + (head_at * a.page_tokens + slot) * D + d, x);
+        st(vc + (head_at * D + d) * a.page_tokens + slot, row[qw + kw + i]);
     }
 }
 
@@ -129,7 +130,8 @@ template <typename T>
 __global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a) {
     __shared__ float qs[ATT_MAX_D];
     __shared__ float ps[64];
-    __shared__ int pages[64];
+    __shared__ int heads_at[64];  // page * kv_heads + kv_head of each key of the tile
+    __shared__ int slots[64];     // its place in the page
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int D = a.head_dim;
     const int kvh = h / (a.n_heads / a.n_kv_heads);
@@ -150,10 +152,12 @@ __global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a)
     for (int j0 = lo; j0 <= p; j0 += 64) {
         const int j = j0 + lane;
         float s = -INFINITY;
-        size_t base = 0;
+        int head_at = 0, slot = 0;
         if (j <= p) {
             const int page = table[j / a.page_tokens];
-            base = (((size_t)page * a.n_kv_heads + kvh) * a.page_tokens + j % a.page_tokens) * D;
+            head_at = page * a.n_kv_heads + kvh;
+            slot = j % a.page_tokens;
+            const size_t base = ((size_t)head_at * a.page_tokens + slot) * D;
             float dot = 0.0f;
             for (int d = 0; d < D; ++d) dot = fmaf(qs[d], ld(kc + base + d), dot);
             s = dot * a.scale;
@@ -164,7 +168,8 @@ __global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a)
         const float correction = expf(m - m_new);  // 0 on the first tile (m = -inf)
         // the tile's weights summed in key order by every lane alike
         ps[lane] = w;
-        pages[lane] = j <= p ? (int)(base / D) : -1;  // row index of the key in units of D
+        heads_at[lane] = head_at;
+        slots[lane] = slot;
         __syncthreads();
         float tile_sum = 0.0f;
         const int n = min(64, p - j0 + 1);
@@ -175,7 +180,7 @@ __global__ void __launch_bounds__(64) paged_attention_generic_kernel(AttnArgs a)
             const int d = lane + 64 * i;
             if (d < D) {
                 float v = acc[i] * correction;
-                for (int jj = 0; jj < n; ++jj) v = fmaf(ps[jj], ld(vc + (size_t)pages[jj] * D + d), v);
+                for (int jj = 0; jj < n; ++jj) v = fmaf(ps[jj], ld(vc + ((size_t)heads_at[jj] * D + d) * a.page_tokens + slots[jj]), v);
                 acc[i] = v;
             }
         }

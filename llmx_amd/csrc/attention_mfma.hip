@@ -1,0 +1,236 @@
+// Paged attention on the matrix cores (bfloat16 cache, pages of a multiple of 16 tokens, head_dim a multiple of 16).
+//
+// One wave owns a work item: up to 16 columns that share one request and one KV head, over a range of keys.
+// A column is a (row, query head) pair: for decoding the 16 columns are the query heads that read one KV head
+// (each K/V byte is read once for all of them), for a prompt portion they are 16 consecutive rows of one head.
+// Keys are walked 32 at a time (two tiles of 16):
+//   scores^T[key][col] = K_tile[16 keys x D] . Q^T[D x 16 cols]        (A = K straight from the page, B = Q in registers)
+//   online softmax per column in float32 (columns live in lanes l%16, keys in lane groups l/16 and registers)
+//   out^T[dim][col]  += V^T_tile[16 dims x 32 keys] . P^T[32 keys x 16 cols]
+// The value pages are stored transposed ([dim][token]) so that V^T's rows are contiguous, and the 32 keys of a step are
+// assigned to the product's k-slots in the order the score accumulators already hold them: no data moves between lanes.
+// A long context is split over several items whose partial (max, sum, out) are merged in split order by a second kernel.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+#define AM_MAX_D 256
+#define AM_ITEM_INTS 8
+
+// item: {row0, n_rows, head0, n_heads, split, n_splits, slot, unused}
+//   columns c = 0 .. n_rows*n_heads-1: row = row0 + c / n_heads, head = head0 + c % n_heads
+//   slot < 0: the item writes the final output; otherwise partials go to part_*[(slot) * 16 + c]
+struct AttnMfmaArgs {
+    const bf16_t* q;        // [T, n_heads, D]
+    const bf16_t* k_cache;  // [pages, kv_heads, page_tokens, D]
+    const bf16_t* v_cache;  // [pages, kv_heads, D, page_tokens]
+    const int* pos;
+    const int* row_entry;
+    const int* tables;
+    const int* items;
+    bf16_t* out;            // [T, n_heads * D]
+    float* part_o;          // [slots * 16, D]
+    float* part_ml;         // [slots * 16, 2]: running max, running sum
+    float scale;
+    int n_items, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
+};
+
+template <int DT>  // DT = head_dim / 16 rounded up
+__global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs a) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int item_no = blockIdx.x * 4 + wave;
+    if (item_no >= a.n_items) return;
+    const int* it = a.items + (size_t)item_no * AM_ITEM_INTS;
+    const int row0 = it[0], n_rows = it[1], head0 = it[2], n_heads_item = it[3], split = it[4], n_splits = it[5], slot = it[6];
+    const int D = a.head_dim, bt = a.page_tokens, Hkv = a.n_kv_heads;
+    const int c = lane & 15, g = lane >> 4;
+    const int n_cols = n_rows * n_heads_item;
+    const bool col_ok = c < n_cols;
+    const int t = row0 + (col_ok ? c / n_heads_item : 0);
+    const int h = head0 + (col_ok ? c % n_heads_item : 0);
+    const int kvh = head0 / (a.n_heads / Hkv);
+    const int p_col = a.pos[t];
+    const int p_first = a.pos[row0], p_last = a.pos[row0 + n_rows - 1];
+    const int* table = a.tables + (size_t)a.row_entry[row0] * a.max_blocks;
+    const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
+    const int lo_first = (a.window > 0 && p_first - a.window + 1 > 0) ? p_first - a.window + 1 : 0;
+    // the item's keys: [lo32, p_last], cut into n_splits runs of whole 32-key steps
+    const int lo32 = lo_first & ~31;
+    const int n_steps = (p_last + 1 - lo32 + 31) >> 5;
+    const int steps_per = (n_steps + n_splits - 1) / n_splits;
+    const int key_begin = lo32 + split * steps_per * 32;
+    const int key_end = min(p_last + 1, key_begin + steps_per * 32);
+
+    // Q^T fragments: lane (column c, dims 32s + 8g ..)
+    constexpr int QS = (DT + 1) / 2;
+    bf16x8_t qf[QS];
+#pragma unroll
+    for (int s = 0; s < QS; ++s) {
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        const int d = 32 * s + 8 * g;
+        if (col_ok && d < D) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + d);
+        qf[s] = __builtin_bit_cast(bf16x8_t, v);
+    }
+    f32x4_t o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float m = -INFINITY, l = 0.0f;
+
+    for (int j0 = key_begin; j0 < key_end; j0 += 32) {
+        // the two 16-key tiles of the step: where their pages are
+        size_t k_at[2], v_at[2];
+        bool tile_in[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int key0 = j0 + 16 * u;
+            tile_in[u] = key0 < key_end;
+            int page = tile_in[u] ? table[key0 / bt] : -1;
+            if (page < 0) tile_in[u] = false;
+            const int sub = key0 % bt;
+            const size_t head_at = (size_t)(page < 0 ? 0 : page) * Hkv + kvh;
+            k_at[u] = (head_at * bt + sub) * D;
+            v_at[u] = head_at * D * bt + sub;
+        }
+        // scores^T: lane holds keys 4g + i of each tile for its column
+        f32x4_t s_acc[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s_acc[u] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            bf16x8_t kf[QS];
+#pragma unroll
+            for (int s = 0; s < QS; ++s) {
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                const int d = 32 * s + 8 * g;
+                if (tile_in[u] && d < D) v = *reinterpret_cast<const u32x4_t*>(a.k_cache + k_at[u] + (size_t)c * D + d);
+                kf[s] = __builtin_bit_cast(bf16x8_t, v);
+            }
+#pragma unroll
+            for (int s = 0; s < QS; ++s) s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s], qf[s], s_acc[u], 0, 0, 0);
+        }
+        // V^T fragments: lane (dim 16dt + c, keys 4g .. 4g+3 of each tile); loaded before the softmax so they are in flight
+        bf16x8_t vf[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            u32x2_t v0 = {0u, 0u}, v1 = {0u, 0u};
+            const int d = 16 * dt + c;
+            if (d < D) {
+                if (tile_in[0]) v0 = *reinterpret_cast<const u32x2_t*>(a.v_cache + v_at[0] + (size_t)d * bt + 4 * g);
+                if (tile_in[1]) v1 = *reinterpret_cast<const u32x2_t*>(a.v_cache + v_at[1] + (size_t)d * bt + 4 * g);
+            }
+            const u32x4_t v = {v0[0], v0[1], v1[0], v1[1]};
+            vf[dt] = __builtin_bit_cast(bf16x8_t, v);
+        }
+        // online softmax of the column over the step's 32 keys
+        float sc[8];
+        float step_max = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = j0 + 16 * u + 4 * g + i;
+                const bool ok = tile_in[u] && col_ok && key <= p_col && key >= lo_col && key < key_end;
+                const float v = ok ? s_acc[u][i] * a.scale : -INFINITY;
+                sc[4 * u + i] = v;
+                step_max = fmaxf(step_max, v);
+            }
+        step_max = fmaxf(step_max, __shfl_xor(step_max, 16, 64));
+        step_max = fmaxf(step_max, __shfl_xor(step_max, 32, 64));
+        const float m_new = fmaxf(m, step_max);
+        const float alpha = (m_new == -INFINITY) ? 1.0f : __expf(m - m_new);   // m = -inf gives 0
+        float step_sum = 0.0f;
+        float pw[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pw[i] = (sc[i] == -INFINITY) ? 0.0f : __expf(sc[i] - m_new);
+            step_sum += pw[i];
+        }
+        step_sum += __shfl_xor(step_sum, 16, 64);
+        step_sum += __shfl_xor(step_sum, 32, 64);
+        l = l * alpha + step_sum;
+        m = m_new;
+        bf16x8_t pf;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pf[i] = (__bf16)pw[i];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            o[dt] = f32x4_t{o[dt][0] * alpha, o[dt][1] * alpha, o[dt][2] * alpha, o[dt][3] * alpha};
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
+        }
+    }
+    if (!col_ok) return;
+    // lane holds dims 16dt + 4g + i of its column
+    if (slot < 0) {
+        const float inv = 1.0f / l;
+        bf16_t* dst = a.out + ((size_t)t * a.n_heads + h) * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = 16 * dt + 4 * g + i;
+                if (d < D) dst[d] = f32_to_bf16(o[dt][i] * inv);
+            }
+    } else {
+        const size_t at = (size_t)slot * 16 + c;
+        float* dst = a.part_o + at * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = 16 * dt + 4 * g + i;
+                if (d < D) dst[d] = o[dt][i];
+            }
+        if (g == 0) {
+            a.part_ml[at * 2] = m;
+            a.part_ml[at * 2 + 1] = l;
+        }
+    }
+}
+
+// merge: one block per output (row, head).  merge item: {row, head, first_slot, n_splits, column}
+__global__ void attention_merge_kernel(const int* __restrict__ merges, const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                       bf16_t* __restrict__ out, int n_heads, int D) {
+    const int* mi = merges + (size_t)blockIdx.x * AM_ITEM_INTS;
+    const int t = mi[0], h = mi[1], first = mi[2], n = mi[3], c = mi[4];
+    float mx = -INFINITY;
+    for (int s = 0; s < n; ++s) mx = fmaxf(mx, part_ml[((size_t)(first + s) * 16 + c) * 2]);
+    float total = 0.0f;
+    for (int s = 0; s < n; ++s) {
+        const size_t at = (size_t)(first + s) * 16 + c;
+        const float ms = part_ml[at * 2];
+        total += (ms == -INFINITY ? 0.0f : __expf(ms - mx)) * part_ml[at * 2 + 1];
+    }
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float acc = 0.0f;
+        for (int s = 0; s < n; ++s) {
+            const size_t at = (size_t)(first + s) * 16 + c;
+            const float ms = part_ml[at * 2];
+            acc += (ms == -INFINITY ? 0.0f : __expf(ms - mx)) * part_o[at * D + d];
+        }
+        out[((size_t)t * n_heads + h) * D + d] = f32_to_bf16(acc / total);
+    }
+}
+
+extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
+                                         const int* tables, const int* items, int n_items, const int* merges, int n_merges, void* out,
+                                         float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
+                                         int page_tokens, int max_blocks, int window, hipStream_t stream) {
+    if (n_items <= 0) return 0;
+    if (head_dim % 16 || head_dim > AM_MAX_D || page_tokens % 16 || n_heads % n_kv_heads) return -2;
+    AttnMfmaArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pos, row_entry, tables, items, (bf16_t*)out, part_o,
+                   part_ml, scale, n_items, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
+    const dim3 grid((n_items + 3) / 4), block(256);
+    switch (head_dim / 16) {
+#define AM_CASE(DT) case DT: hipLaunchKernelGGL(paged_attention_mfma_kernel<DT>, grid, block, 0, stream, a); break;
+        AM_CASE(1) AM_CASE(2) AM_CASE(3) AM_CASE(4) AM_CASE(5) AM_CASE(6) AM_CASE(7) AM_CASE(8)
+        AM_CASE(9) AM_CASE(10) AM_CASE(11) AM_CASE(12) AM_CASE(13) AM_CASE(14) AM_CASE(15) AM_CASE(16)
+#undef AM_CASE
+        default: return -2;
+    }
+    if (n_merges > 0)
+        hipLaunchKernelGGL(attention_merge_kernel, dim3(n_merges), dim3(128), 0, stream, merges, part_o, part_ml, (bf16_t*)out, n_heads, head_dim);
+    return LLMX_CHECK_LAUNCH();
+}

@@ -1,0 +1,230 @@
+// Weight-streaming bf16 product for few rows (decode): C[M,N] (+)= A[M,K] * W[N,K]^T on the matrix cores.
+//
+// A workgroup of KS waves owns one strip of 16 output features: every wave streams its share of the strip's K
+// (16 rows x 32 k = 1 KB of W per MFMA 16x16x32, 16 bytes a lane straight from HBM into the A operand), the rows of the
+// step ride along as the B operand (16 rows a tile, up to MT tiles), and the waves' partial sums are added in wave order
+// through LDS.  The step's time is the time to read W once; nothing else is read more than (rows/16) of that.
+// An output element is sum over waves (in order) of sum over that wave's k-steps (in order) of one MFMA's 32 products:
+// its bits depend on K and KS only, not on M or on the other rows.
+//
+// Grouped form: blockIdx.y walks the experts that have rows; A's rows are gathered through the expert-sorted pair list
+// and C's rows scattered to the pairs.  The SwiGLU form streams a gate strip and the matching up strip together and
+// stores silu(gate) * up.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+enum : int { SK_STORE = 0, SK_ADD = 1, SK_SWIGLU = 2 };
+
+struct SkinnyArgs {
+    const bf16_t* A;
+    const bf16_t* W;
+    void* C;
+    int M, N, K;
+    int lda, ldc;
+    // grouped
+    const int* active;         // [n_active] group ids that have rows (blockIdx.y indexes it)
+    const int* n_active;       // device scalar
+    const int* group_offsets;  // [G+1]
+    const int* list;           // expert-sorted pair ids
+    int a_div;
+    long w_group_stride;
+    int up_offset;
+};
+
+__device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p, bool in) {
+    u32x4_t v = {0u, 0u, 0u, 0u};
+    if (in) v = *reinterpret_cast<const u32x4_t*>(p);
+    return __builtin_bit_cast(bf16x8_t, v);
+}
+
+#define SK_UNROLL 4
+
+template <int KS, int MT, int EPI, typename TC, bool GROUPED>
+__global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
+    constexpr int NACC = (EPI == SK_SWIGLU) ? 2 : 1;
+    __shared__ float red[KS > 1 ? KS : 1][MT * NACC][256];
+    __shared__ int rows_a[MT * 16];
+    __shared__ int rows_c[MT * 16];
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, kg = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const bf16_t* W = g.W;
+    int row_begin = 0, row_end = g.M;
+    if (GROUPED) {
+        if ((int)blockIdx.y >= *g.n_active) return;
+        const int e = g.active[blockIdx.y];
+        row_begin = g.group_offsets[e];
+        row_end = g.group_offsets[e + 1];
+        W += (size_t)e * g.w_group_stride;
+    }
+    const int K = g.K;
+    const int steps_total = (K + 31) >> 5;
+    const int per = (steps_total + KS - 1) / KS;
+    const int s_begin = wave * per;
+    const int s_end = min(steps_total, s_begin + per);
+    const int w_row = min(n0 + r, g.N - 1);
+    const bf16_t* wp = W + (size_t)w_row * K + kg * 8;
+    const bf16_t* up = (EPI == SK_SWIGLU) ? wp + (size_t)g.up_offset * K : wp;
+
+    for (int m0 = row_begin; m0 < row_end; m0 += 16 * MT) {
+        if (tid < MT * 16) {
+            const int m = m0 + tid;
+            int ra = -1, rc = -1;
+            if (m < row_end) {
+                if (GROUPED) {
+                    const int p = g.list[m];
+                    ra = p / g.a_div;
+                    rc = p;
+                } else {
+                    ra = rc = m;
+                }
+            }
+            rows_a[tid] = ra;
+            rows_c[tid] = rc;
+        }
+        __syncthreads();
+        const bf16_t* ap[MT];
+        bool a_in[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int ra = rows_a[t * 16 + r];
+            a_in[t] = ra >= 0;
+            ap[t] = g.A + (size_t)(ra >= 0 ? ra : 0) * g.lda + kg * 8;
+        }
+        f32x4_t acc[MT][NACC];
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int a = 0; a < NACC; ++a) acc[t][a] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+        for (int s = s_begin; s < s_end; s += SK_UNROLL) {
+            bf16x8_t wf[SK_UNROLL], uf[SK_UNROLL], af[SK_UNROLL][MT];
+#pragma unroll
+            for (int u = 0; u < SK_UNROLL; ++u) {
+                const int k = (s + u) * 32 + kg * 8;
+                const bool in = (s + u) < s_end && k < K;
+                wf[u] = load_frag(wp + (size_t)(s + u) * 32, in);
+                if (EPI == SK_SWIGLU) uf[u] = load_frag(up + (size_t)(s + u) * 32, in);
+            }
+#pragma unroll
+            for (int u = 0; u < SK_UNROLL; ++u) {
+                const int k = (s + u) * 32 + kg * 8;
+                const bool in = (s + u) < s_end && k < K;
+#pragma unroll
+                for (int t = 0; t < MT; ++t) af[u][t] = load_frag(ap[t] + (size_t)(s + u) * 32, in && a_in[t]);
+            }
+#pragma unroll
+            for (int u = 0; u < SK_UNROLL; ++u) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], af[u][t], acc[t][0], 0, 0, 0);
+                    if (EPI == SK_SWIGLU) acc[t][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u], af[u][t], acc[t][1], 0, 0, 0);
+                }
+            }
+        }
+        // partial sums of the waves, added in wave order
+        if (KS > 1) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int a = 0; a < NACC; ++a) *reinterpret_cast<f32x4_t*>(&red[wave][t * NACC + a][lane * 4]) = acc[t][a];
+            __syncthreads();
+        }
+        if (wave == 0) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                f32x4_t v[NACC];
+#pragma unroll
+                for (int a = 0; a < NACC; ++a) {
+                    v[a] = acc[t][a];
+                    if (KS > 1) {
+                        v[a] = *reinterpret_cast<f32x4_t*>(&red[0][t * NACC + a][lane * 4]);
+#pragma unroll
+                        for (int w = 1; w < KS; ++w) {
+                            const f32x4_t o = *reinterpret_cast<f32x4_t*>(&red[w][t * NACC + a][lane * 4]);
+                            v[a] = f32x4_t{v[a][0] + o[0], v[a][1] + o[1], v[a][2] + o[2], v[a][3] + o[3]};
+                        }
+                    }
+                }
+                // lane: row (tile t, column r), features n0 + 4*kg + 0..3
+                const int rc = rows_c[t * 16 + r];
+                if (rc < 0) continue;
+                TC* c = (TC*)g.C + (size_t)rc * g.ldc + n0 + 4 * kg;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (n0 + 4 * kg + i >= g.N) continue;
+                    float x = v[0][i];
+                    if (EPI == SK_SWIGLU) x = (x / (1.0f + expf(-x))) * v[1][i];
+                    if (EPI == SK_ADD) x = ld(c + i) + x;
+                    st(c + i, x);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <int KS, int MT, int EPI, typename TC>
+static void launch_grouped(const SkinnyArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
+    if (grouped)
+        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true>), grid, dim3(64 * KS), 0, stream, g);
+    else
+        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false>), grid, dim3(64 * KS), 0, stream, g);
+}
+
+template <int KS, int MT>
+static int launch_epi(const SkinnyArgs& g, int epi, int c_dtype, dim3 grid, bool grouped, hipStream_t stream) {
+    if (epi == SK_SWIGLU) {
+        if (MT != 1) return -2;
+        if (c_dtype == LLMX_BF16) launch_grouped<KS, 1, SK_SWIGLU, bf16_t>(g, grid, grouped, stream);
+        else launch_grouped<KS, 1, SK_SWIGLU, float>(g, grid, grouped, stream);
+    } else if (epi == SK_ADD) {
+        if (c_dtype != LLMX_F32) return -2;
+        launch_grouped<KS, MT, SK_ADD, float>(g, grid, grouped, stream);
+    } else if (epi == SK_STORE) {
+        if (c_dtype == LLMX_BF16) launch_grouped<KS, MT, SK_STORE, bf16_t>(g, grid, grouped, stream);
+        else launch_grouped<KS, MT, SK_STORE, float>(g, grid, grouped, stream);
+    } else {
+        return -2;
+    }
+    return LLMX_CHECK_LAUNCH();
+}
+
+template <int KS>
+static int launch_mt(const SkinnyArgs& g, int mt, int epi, int c_dtype, dim3 grid, bool grouped, hipStream_t stream) {
+    switch (mt) {
+        case 1: return launch_epi<KS, 1>(g, epi, c_dtype, grid, grouped, stream);
+        case 2: return launch_epi<KS, 2>(g, epi, c_dtype, grid, grouped, stream);
+        case 4: return launch_epi<KS, 4>(g, epi, c_dtype, grid, grouped, stream);
+    }
+    return -2;
+}
+
+// A and W bfloat16, K a multiple of 8, rows of A and W 16-byte aligned.  n_groups == 0: dense, M rows.
+// n_groups > 0: grouped; `max_active` bounds the groups that have rows (grid.y), `n_active` holds their number.
+// ks: waves that share a strip's K (1, 2, 4 or 8); chosen by the caller from N and K only.
+extern "C" int llmx_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
+                                int n_groups, int max_active, const int* active, const int* n_active, const int* group_offsets,
+                                const int* list, int a_div, long w_group_stride, int up_offset, hipStream_t stream) {
+    if (N <= 0 || K <= 0) return 0;
+    if (K % 8) return -2;
+    const bool grouped = n_groups > 0;
+    if (!grouped && M <= 0) return 0;
+    if (grouped && max_active <= 0) return 0;
+    SkinnyArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, active, n_active, group_offsets, list, a_div > 0 ? a_div : 1,
+                 w_group_stride, up_offset};
+    dim3 grid((N + 15) / 16, grouped ? max_active : 1, 1);
+    int mt = 1;
+    if (!grouped && epi != SK_SWIGLU) mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    switch (ks) {
+        case 1: return launch_mt<1>(g, mt, epi, c_dtype, grid, grouped, stream);
+        case 2: return launch_mt<2>(g, mt, epi, c_dtype, grid, grouped, stream);
+        case 4: return launch_mt<4>(g, mt, epi, c_dtype, grid, grouped, stream);
+        case 8: return launch_mt<8>(g, mt, epi, c_dtype, grid, grouped, stream);
+    }
+    return -2;
+}

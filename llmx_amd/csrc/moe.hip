@@ -108,15 +108,26 @@ __global__ void __launch_bounds__(64) moe_count_kernel(const int* __restrict__ i
 }
 
 __global__ void __launch_bounds__(64) moe_place_kernel(const int* __restrict__ ids, int n_pairs, int n_experts, const int* __restrict__ counts,
-                                                      int* __restrict__ offsets, int* __restrict__ list) {
+                                                      int* __restrict__ offsets, int* __restrict__ list, int* __restrict__ active,
+                                                      int* __restrict__ n_active) {
     const int e = blockIdx.x, lane = threadIdx.x;
-    int before = 0;
-    for (int i = lane; i < e; i += 64) before += counts[i];
+    int before = 0, active_before = 0;
+    for (int i = lane; i < e; i += 64) {
+        before += counts[i];
+        active_before += counts[i] > 0;
+    }
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o, 64);
+    for (int o = 32; o > 0; o >>= 1) {
+        before += __shfl_xor(before, o, 64);
+        active_before += __shfl_xor(active_before, o, 64);
+    }
     if (lane == 0) {
         offsets[e] = before;
-        if (e == n_experts - 1) offsets[n_experts] = before + counts[e];
+        if (counts[e] > 0) active[active_before] = e;  // the experts that have rows, in increasing order
+        if (e == n_experts - 1) {
+            offsets[n_experts] = before + counts[e];
+            n_active[0] = active_before + (counts[e] > 0);
+        }
     }
     int at = before;
     for (int p0 = 0; p0 < n_pairs; p0 += 64) {
@@ -128,9 +139,11 @@ __global__ void __launch_bounds__(64) moe_place_kernel(const int* __restrict__ i
     }
 }
 
-extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* counts, int* offsets, int* list, hipStream_t stream) {
+// counts [X], offsets [X+1], list [n_pairs], active [X], n_active [1]
+extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* counts, int* offsets, int* list, int* active, int* n_active,
+                              hipStream_t stream) {
     if (n_pairs <= 0 || n_experts <= 0) return 0;
     hipLaunchKernelGGL(moe_count_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, counts);
-    hipLaunchKernelGGL(moe_place_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, n_experts, counts, offsets, list);
+    hipLaunchKernelGGL(moe_place_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
     return LLMX_CHECK_LAUNCH();
 }

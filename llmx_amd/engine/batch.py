@@ -64,6 +64,7 @@ class StepState:
         self.token_ids = self.positions = self.row_entry = self.entry_slots = self.pick = None
         self._tables: List[torch.Tensor] = []
         self.max_rows_per_entry = 0
+        self._plans = {}
         self.run_index = -1          # which item of the run order is running
         self.observer = None         # callable(step, kind, **tensors) that sees what parts choose to show, or None
 
@@ -72,6 +73,16 @@ class StepState:
 
     def tables(self, group: int) -> torch.Tensor:
         return self._tables[group]
+
+    def attention_plan(self, n_heads: int, n_kv_heads: int):
+        """The matrix-core attention kernel's work items for this step's rows (shared by layers with the same heads)."""
+        key = (n_heads, n_kv_heads)
+        plan = self._plans.get(key)
+        if plan is None:
+            from .. import ops
+            plan = ops.attention_plan([e.n for e in self.entries], [e.past + e.n for e in self.entries], n_heads, n_kv_heads, self.device)
+            self._plans[key] = plan
+        return plan
 
     def observe(self, kind: str, **tensors) -> None:
         """Shows intermediate tensors (a router's picks, for instance) to the engine's observer, when one is set."""

@@ -127,8 +127,8 @@ class Engine:
         self.group_needs = keys
         groups = [GroupSpec(f"kv{g}", self.page_tokens, n_pages, need.window) for g, need in enumerate(keys)]
         self.cache = CacheManager(groups, self.max_requests)
-        # [cache in group, K|V, page, kv head, token in page, head dim]
-        self._kv = [torch.zeros((counts[g], 2, n_pages, need.kv_heads, self.page_tokens, need.head_dim), dtype=self.act_dtype,
+        # [cache in group, K|V, page, kv head, token in page * head dim]; keys are [token][dim], values [dim][token]
+        self._kv = [torch.zeros((counts[g], 2, n_pages, need.kv_heads, self.page_tokens * need.head_dim), dtype=self.act_dtype,
                                 device=self.device) for g, need in enumerate(keys)]
         self._state: List[Optional[torch.Tensor]] = []
         for need in needs:
@@ -141,7 +141,10 @@ class Engine:
             g = self._group_of[e.cache]
             if g >= 0:
                 store = self._kv[g][self._index_in_group[e.cache]]
-                self._layer_caches.append(LayerCache(group=g, k=store[0], v=store[1], writes=e.writes))
+                need = keys[g]
+                self._layer_caches.append(LayerCache(
+                    group=g, k=store[0].view(n_pages, need.kv_heads, self.page_tokens, need.head_dim),
+                    v=store[1].view(n_pages, need.kv_heads, need.head_dim, self.page_tokens), writes=e.writes))
             else:
                 self._layer_caches.append(LayerCache(state=self._state[e.cache], writes=e.writes))
 

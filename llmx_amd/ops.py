@@ -59,8 +59,10 @@ def _declare(h) -> None:
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
+        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, P, P, I, I, I, I, I, F, P],
-        "llmx_moe_align": [P, I, I, P, P, P, P],
+        "llmx_moe_align": [P, I, I, P, P, P, P, P, P],
+        "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P],
         "llmx_argmax_rows": [P, P, P, I, I, P],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
@@ -129,21 +131,47 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[tor
                               _dev(out32, "out32", torch.float32, (rows, n)), rows, n, _stream()), "rmsnorm")
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE) -> None:
+SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores
+SKINNY_MAX_GROUPED_ROWS = 128  # routed products of at most this many token rows do
+
+
+def _split_k(n_strips: int, K: int) -> int:
+    """Waves that share one 16-feature strip's K: enough strips*waves to fill the chip, at least 4 k-steps a wave.
+    A function of the product's shape only, so a row's bits do not depend on the batch."""
+    ks = 1
+    while ks < 8 and n_strips * ks < 2048 and (K // 32) // (ks * 2) >= 4:
+        ks *= 2
+    return ks
+
+
+def _skinny_ok(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int) -> bool:
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[-1] % 8 == 0
+            and (epilogue != EPI_ADD or c.dtype == torch.float32))
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False) -> None:
     """c[M,N] (+)= a[M,K] @ w[N,K]^T, accumulated in float32; EPI_SWIGLU: c = silu(a @ w[:N]^T) * (a @ w[N:]^T)."""
     M, K = a.shape
     N = w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]   # swiglu: w holds gate rows, then up rows
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
+    if not force_generic and M <= SKINNY_MAX_ROWS and _skinny_ok(a, w, c, epilogue):
+        _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
+                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()),
+               "gemm_skinny")
+        return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm")
 
 
 def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor, a_div: int,
-                 epilogue: int = EPI_STORE) -> None:
+                 epilogue: int = EPI_STORE, active: Optional[torch.Tensor] = None, n_active: Optional[torch.Tensor] = None,
+                 token_rows: Optional[int] = None, force_generic: bool = False) -> None:
     """For each group g: rows p in pairs[offsets[g]:offsets[g+1]] get c[p] = a[p // a_div] @ w[g]^T.
 
-    With EPI_SWIGLU w[g] holds gate rows then up rows and c[p] = silu(gate) * up.
+    With EPI_SWIGLU w[g] holds gate rows then up rows and c[p] = silu(gate) * up.  `active` / `n_active` (from
+    moe_align) list the groups that have rows; with them, steps of few token rows (`token_rows`, default the pair
+    count) take the weight-streaming kernel.
     """
     G, NW, K = w.shape
     N = NW // 2 if epilogue == EPI_SWIGLU else NW
@@ -152,6 +180,16 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
     n_pairs = pairs.shape[0]
     if c.shape[0] < n_pairs or a.shape[0] * a_div < n_pairs:
         raise KernelError("grouped_gemm: more pairs than rows")
+    if token_rows is None:
+        token_rows = n_pairs
+    if (not force_generic and active is not None and n_active is not None and _skinny_ok(a, w, c, epilogue)
+            and token_rows <= SKINNY_MAX_GROUPED_ROWS):
+        _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
+                                      _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
+                                      _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
+                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
+               "grouped_gemm_skinny")
+        return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    n_pairs, N, K, K, K, N, epilogue, G, _dev(offsets, "offsets", torch.int32, (G + 1,)),
                                    _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
@@ -165,7 +203,8 @@ def qknorm_rope_kvwrite(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_w
     rows = qkv.shape[0]
     qw, kw = n_heads * head_dim, n_kv_heads * head_dim
     n_pages, hk, page_tokens, d = k_cache.shape
-    if (hk, d) != (n_kv_heads, head_dim) or v_cache.shape != k_cache.shape or k_cache.dtype != q_out.dtype or v_cache.dtype != q_out.dtype:
+    if ((hk, d) != (n_kv_heads, head_dim) or tuple(v_cache.shape) != (n_pages, hk, d, page_tokens) or k_cache.dtype != q_out.dtype
+            or v_cache.dtype != q_out.dtype):
         raise KernelError("qknorm_rope_kvwrite: cache shape or dtype does not fit the heads")
     if rotary_dim % 2 or rotary_dim > head_dim or cos_sin.shape[1] != rotary_dim:
         raise KernelError("qknorm_rope_kvwrite: rotary width does not fit")
@@ -182,18 +221,101 @@ def qknorm_rope_kvwrite(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_w
         1 if write_kv else 0, _stream()), "qknorm_rope_kvwrite")
 
 
+class AttentionPlan:
+    """Work items of the matrix-core attention kernel for one step's rows (they hold no positions, so a plan serves
+    every step with the same rows per request) and the merge list of the items that were split over the context."""
+
+    def __init__(self, items, merges, n_slots, device):
+        import numpy as np
+        self.n_items = len(items)
+        self.n_merges = len(merges)
+        self.n_slots = n_slots
+        self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 8), device=device) if items else None
+        self.merges = torch.tensor(np.asarray(merges, dtype=np.int32).reshape(-1, 8), device=device) if merges else None
+
+
+_PLAN_CACHE: dict = {}
+ATTENTION_TARGET_WAVES = 1024   # work items wanted before long contexts stop being split further
+ATTENTION_MIN_SPLIT_KEYS = 256  # a split covers at least this many keys
+
+
+def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device) -> AttentionPlan:
+    """row_counts[i]: rows of entry i in the step (entries' rows are consecutive, in order); contexts[i]: tokens the
+    entry holds after the step.  Single-row entries become one item per KV head (columns = its query heads), split over
+    the context when there are few of them; longer entries become tiles of 16 rows of one head."""
+    ratio = n_heads // n_kv_heads
+    head_chunks = [(kvh * ratio + c0, min(16, ratio - c0)) for kvh in range(n_kv_heads) for c0 in range(0, ratio, 16)]
+    single = [i for i, n in enumerate(row_counts) if n == 1]
+    n_splits = 1
+    if single:
+        base = len(single) * len(head_chunks)
+        longest = max(contexts[i] for i in single)
+        n_splits = max(1, min(-(-ATTENTION_TARGET_WAVES // base), longest // ATTENTION_MIN_SPLIT_KEYS))
+    key = (tuple(row_counts), n_heads, n_kv_heads, n_splits, str(device))
+    plan = _PLAN_CACHE.get(key)
+    if plan is not None:
+        return plan
+    items, merges, slot = [], [], 0
+    row0s, at = [], 0
+    for n in row_counts:
+        row0s.append(at)
+        at += n
+    # tiles of long entries first, latest rows (longest key ranges) first
+    for i, n in enumerate(row_counts):
+        if n == 1:
+            continue
+        for r0 in range(((n - 1) // 16) * 16, -1, -16):
+            for h in range(n_heads):
+                items.append([row0s[i] + r0, min(16, n - r0), h, 1, 0, 1, -1, 0])
+    for i in single:
+        for head0, nh in head_chunks:
+            if n_splits == 1:
+                items.append([row0s[i], 1, head0, nh, 0, 1, -1, 0])
+                continue
+            for c in range(nh):
+                merges.append([row0s[i], head0 + c, slot, n_splits, c, 0, 0, 0])
+            for sp in range(n_splits):
+                items.append([row0s[i], 1, head0, nh, sp, n_splits, slot, 0])
+                slot += 1
+    plan = AttentionPlan(items, merges, slot, device)
+    if len(_PLAN_CACHE) > 256:
+        _PLAN_CACHE.clear()
+    _PLAN_CACHE[key] = plan
+    return plan
+
+
+def attention_mfma_ok(dtype: torch.dtype, head_dim: int, page_tokens: int) -> bool:
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256 and page_tokens % 16 == 0
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: torch.Tensor, row_entry: torch.Tensor,
-                    tables: torch.Tensor, out: torch.Tensor, scale: float, n_heads: int, window: int = 0) -> None:
+                    tables: torch.Tensor, out: torch.Tensor, scale: float, n_heads: int, window: int = 0,
+                    plan: Optional[AttentionPlan] = None, scratch=None) -> None:
+    """Causal attention of each row over its request's pages.  With a `plan` (and bfloat16, head_dim a multiple of 16,
+    pages of a multiple of 16 tokens) the matrix-core kernel runs; `scratch(name, shape, dtype)` gives it storage for
+    the partial results of split contexts.  Otherwise the universal kernel runs."""
     rows = q.shape[0]
     n_pages, n_kv_heads, page_tokens, head_dim = k_cache.shape
     if q.shape[1] != n_heads * head_dim or out.shape != q.shape or q.dtype != k_cache.dtype or out.dtype != q.dtype:
         raise KernelError("paged_attention: shapes or dtypes do not agree")
     if head_dim > 256 or n_heads % n_kv_heads:
         raise KernelError(f"paged_attention: head_dim {head_dim} above 256 or heads {n_heads} not a multiple of KV heads {n_kv_heads}")
-    _check(lib().llmx_paged_attention_generic(
-        _dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache", shape=k_cache.shape), _dev(pos, "pos", torch.int32, (rows,)),
-        _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32), _dev(out, "out"), _code(q.dtype),
-        float(scale), rows, n_heads, n_kv_heads, head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention")
+    common = (_dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache", shape=(n_pages, n_kv_heads, head_dim, page_tokens)),
+              _dev(pos, "pos", torch.int32, (rows,)), _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32))
+    if plan is not None and plan.n_items and attention_mfma_ok(q.dtype, head_dim, page_tokens):
+        part_o = part_ml = None
+        if plan.n_slots:
+            if scratch is None:
+                scratch = lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=q.device)
+            part_o = scratch("attention.part_o", (plan.n_slots * 16, head_dim), torch.float32)
+            part_ml = scratch("attention.part_ml", (plan.n_slots * 16, 2), torch.float32)
+        _check(lib().llmx_paged_attention_mfma(*common, _dev(plan.items, "items", torch.int32), plan.n_items,
+                                               _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
+                                               _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale), n_heads, n_kv_heads,
+                                               head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention_mfma")
+        return
+    _check(lib().llmx_paged_attention_generic(*common, _dev(out, "out"), _code(q.dtype), float(scale), rows, n_heads, n_kv_heads,
+                                              head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention")
 
 
 def route_topk(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
@@ -206,10 +328,14 @@ def route_topk(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor,
                                  rows, n_experts, k, score, 1 if normalize else 0, float(scale), _stream()), "route_topk")
 
 
-def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor) -> None:
+def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
+              active: torch.Tensor, n_active: torch.Tensor) -> None:
+    """Groups the pairs p = t*k + j by expert (stable): counts [X], offsets [X+1], pairs [T*k], and the experts that
+    have rows in increasing order: active [X] (first n_active[0] entries)."""
     n_pairs = ids.numel()
     _check(lib().llmx_moe_align(_dev(ids, "ids", torch.int32), n_pairs, n_experts, _dev(counts, "counts", torch.int32, (n_experts,)),
                                 _dev(offsets, "offsets", torch.int32, (n_experts + 1,)), _dev(pairs, "pairs", torch.int32, (n_pairs,)),
+                                _dev(active, "active", torch.int32, (n_experts,)), _dev(n_active, "n_active", torch.int32, (1,)),
                                 _stream()), "moe_align")
 
 

@@ -80,8 +80,11 @@ class Attention(Mixer):
         ops.qknorm_rope_kvwrite(qkv, self.q_norm, self.k_norm, cos_sin, step.positions, step.row_entry, tables, q, cache.k, cache.v,
                                 self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode, write_kv=cache.writes)
         o = step.buf("attention.out", (T, self.q_width), act)
+        plan = None
+        if ops.attention_mfma_ok(act, self.head_dim, cache.k.shape[2]):
+            plan = step.attention_plan(self.heads, self.kv_heads)
         ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
-                            window=int(self.window or 0))
+                            window=int(self.window or 0), plan=plan, scratch=step.buf)
         ops.gemm(o, self.wo, out, ops.EPI_ADD if accumulate else ops.EPI_STORE)
 
 

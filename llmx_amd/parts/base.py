@@ -13,6 +13,7 @@ What a part sees of a step (the `step` argument, an `engine.batch.StepState`):
   step.entry_slots                int32 [n_entries] on the device: each entry's state slot
   step.tables(group)              int32 [n_entries, max_blocks]: page ids of each entry in cache group `group`
   step.buf(name, shape, dtype)    a scratch tensor that lives until the step ends (same name, same storage)
+  step.attention_plan(heads, kv_heads)  work items of the matrix-core attention kernel for this step's rows
   step.run_index                  which item of the run order is running
   step.observe(kind, **tensors)   shows intermediate tensors to an observer, when the engine has one (tests, probes)
 """
@@ -80,7 +81,7 @@ class LayerCache:
     """What one run-order entry's mixer gets of the cache: pages of keys and values, or per-request state."""
     group: int = -1                          # cache group of the pages (index for step.tables)
     k: Optional[torch.Tensor] = None         # [pages, kv_heads, page_tokens, head_dim]
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None         # [pages, kv_heads, head_dim, page_tokens] (transposed within the page)
     writes: bool = True                      # False: this entry reads pages another entry wrote
     state: Optional[torch.Tensor] = None     # [slots, *StateNeed.shape]
 

@@ -92,11 +92,13 @@ class RoutedExperts(FeedForward):
         counts = step.buf("experts.counts", (X,), torch.int32)
         offsets = step.buf("experts.offsets", (X + 1,), torch.int32)
         pairs = step.buf("experts.pairs", (T * k,), torch.int32)
-        ops.moe_align(ids, X, counts, offsets, pairs)
+        active = step.buf("experts.active", (X,), torch.int32)
+        n_active = step.buf("experts.n_active", (1,), torch.int32)
+        ops.moe_align(ids, X, counts, offsets, pairs, active, n_active)
         act = step.buf("experts.act", (T * k, self.intermediate), step.act_dtype)
-        ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU)
+        ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T)
         y = step.buf("experts.y", (T * k, self.hidden), torch.float32)
-        ops.grouped_gemm(act, self.w_down, y, offsets, pairs, 1, ops.EPI_STORE)
+        ops.grouped_gemm(act, self.w_down, y, offsets, pairs, 1, ops.EPI_STORE, active, n_active, token_rows=T)
         ops.moe_combine(out, y, ids, weights, accumulate)
 
 

@@ -1,0 +1,529 @@
+"""Each kernel alone against its plain reference, at other sizes than the engine's tiny models use.
+
+References are torch expressions in float64 (or the functions of plain_model.py); sizes are ragged on purpose: rows
+1, 2, 3, 17, widths that are no power of two, head widths in steps of 16 and 24, experts without rows.
+"""
+
+from __future__ import annotations
+
+import math
+import random
+
+import pytest
+import torch
+
+import plain_model
+import sampler_reference
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def ops():
+    from llmx_amd import ops as o
+    return o
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def bf16_exact(t):
+    """The tensor's values after rounding to bfloat16, as float64 on the CPU."""
+    return t.to(torch.bfloat16).double().cpu()
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,width", [(1, 64), (3, 100), (17, 3072), (2, 7)])
+def test_embed_gather(rows, width):
+    for dtype in (torch.float32, torch.bfloat16):
+        table = rnd(50, width, dtype=dtype)
+        ids = torch.tensor([(7 * i + 3) % 50 for i in range(rows)], dtype=torch.int32, device=DEV)
+        out = torch.empty(rows, width, dtype=torch.float32, device=DEV)
+        ops().embed_gather(table, ids, out)
+        assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("rows,width,eps", [(1, 64, 1e-6), (3, 100, 1e-5), (17, 3072, 1e-6), (2, 6144, 1e-2)])
+def test_rmsnorm(rows, width, eps):
+    x = rnd(rows, width, scale=3.0)
+    w = 1.0 + 0.1 * rnd(width, seed=5)
+    want = plain_model.rms_norm(x.double().cpu(), w.double().cpu(), eps)
+    out32 = torch.empty_like(x)
+    out16 = torch.empty(rows, width, dtype=torch.bfloat16, device=DEV)
+    ops().rmsnorm(x, w, eps, out16, out32)
+    assert (out32.double().cpu() - want).abs().max() <= 2e-6 * want.abs().max()
+    assert torch.equal(out16, out32.to(torch.bfloat16)), "the bfloat16 output is not the float32 output rounded once"
+    # eps matters: a zero row gives zero, not NaN
+    z = torch.zeros(1, width, device=DEV)
+    o = torch.empty_like(z)
+    ops().rmsnorm(z, w, eps, o)
+    assert torch.equal(o, z)
+    # gathered rows
+    pick = torch.tensor([rows - 1, 0], dtype=torch.int32, device=DEV)
+    o2 = torch.empty(2, width, device=DEV)
+    ops().rmsnorm(x, w, eps, o2, None, pick)
+    assert torch.equal(o2, out32[pick.long()])
+
+
+# ---------------------------------------------------------------------------
+GEMM_SHAPES = [(1, 16, 32), (2, 48, 96), (3, 100, 72), (17, 200, 3072), (64, 96, 192), (65, 130, 264), (8, 8192, 3072), (33, 3072, 6144)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("dtypes", [("f32", "f32"), ("bf16", "bf16"), ("bf16", "f32"), ("f32", "bf16")])
+def test_gemm_generic(M, N, K, dtypes):
+    T = {"f32": torch.float32, "bf16": torch.bfloat16}
+    a = rnd(M, K, dtype=T[dtypes[0]])
+    w = rnd(N, K, dtype=T[dtypes[1]], seed=1)
+    want = a.double().cpu() @ w.double().cpu().T
+    c = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops().gemm(a, w, c, force_generic=True)
+    tol = 1e-5 * math.sqrt(K)
+    assert (c.double().cpu() - want).abs().max() <= tol * want.abs().max()
+    # a row's bits do not depend on the other rows of the product
+    if M > 1:
+        c1 = torch.empty(1, N, dtype=torch.float32, device=DEV)
+        ops().gemm(a[M - 1:M].contiguous(), w, c1, force_generic=True)
+        assert torch.equal(c1[0], c[M - 1])
+    # accumulate into an existing float32 result
+    base = rnd(M, N, seed=9)
+    acc = base.clone()
+    ops().gemm(a, w, acc, ops().EPI_ADD, force_generic=True)
+    assert torch.equal(acc, base + c)
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_skinny_bf16(M, N, K):
+    """The matrix-core kernel for few rows (it is taken for bfloat16 operands, K a multiple of 8, at most 64 rows)."""
+    o = ops()
+    a = rnd(M, K, dtype=torch.bfloat16)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=1)
+    want = a.double().cpu() @ w.double().cpu().T
+    c = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    o.gemm(a, w, c)
+    tol = 1e-5 * math.sqrt(K)
+    assert (c.double().cpu() - want).abs().max() <= tol * want.abs().max()
+    cb = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    o.gemm(a, w, cb)
+    assert torch.equal(cb, c.to(torch.bfloat16))
+    if 1 < M <= o.SKINNY_MAX_ROWS:
+        c1 = torch.empty(1, N, dtype=torch.float32, device=DEV)
+        o.gemm(a[M - 1:M].contiguous(), w, c1)
+        assert torch.equal(c1[0], c[M - 1]), "a row's bits depend on the other rows"
+    base = rnd(M, N, seed=9)
+    acc = base.clone()
+    o.gemm(a, w, acc, o.EPI_ADD)
+    assert torch.equal(acc, base + c)
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 32, 64), (3, 48, 96), (17, 1536, 3072), (70, 40, 72)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_swiglu(M, F, K, dtype):
+    a = rnd(M, K, dtype=dtype)
+    w = rnd(2 * F, K, dtype=dtype, seed=1, scale=0.2)
+    g = a.double().cpu() @ w[:F].double().cpu().T
+    u = a.double().cpu() @ w[F:].double().cpu().T
+    want = (g / (1 + torch.exp(-g))) * u
+    c = torch.empty(M, F, dtype=torch.float32, device=DEV)
+    ops().gemm(a, w, c, ops().EPI_SWIGLU)
+    assert (c.double().cpu() - want).abs().max() <= 2e-5 * math.sqrt(K) * want.abs().max()
+    # gate rows come first: with the halves swapped the result must differ
+    swapped = torch.cat([w[F:], w[:F]]).contiguous()
+    c2 = torch.empty_like(c)
+    ops().gemm(a, swapped, c2, ops().EPI_SWIGLU)
+    assert not torch.allclose(c, c2)
+
+
+def routed_setup(T, X, k, seed):
+    rng = random.Random(seed)
+    ids = torch.tensor([rng.sample(range(X), k) for _ in range(T)], dtype=torch.int32)
+    if T > 2:
+        ids[1, 0] = -1   # a slot without an expert
+    return ids
+
+
+@pytest.mark.parametrize("T,X,k,E,F", [(1, 8, 2, 64, 32), (5, 16, 4, 96, 48), (17, 24, 3, 72, 40), (40, 256, 8, 256, 128), (150, 6, 2, 64, 32)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_routed_products(T, X, k, E, F, dtype):
+    """moe_align, the two grouped products and the combine against a loop over pairs; experts without rows included."""
+    o = ops()
+    ids = routed_setup(T, X, k, T + X)
+    w_pairs = torch.rand(T, k, generator=torch.Generator().manual_seed(3))
+    h = rnd(T, E, dtype=dtype)
+    wgu = rnd(X, 2 * F, E, dtype=dtype, seed=1, scale=0.3)
+    wd = rnd(X, E, F, dtype=dtype, seed=2, scale=0.3)
+    ids_d, w_d = ids.to(DEV), w_pairs.to(DEV)
+    counts = torch.empty(X, dtype=torch.int32, device=DEV)
+    offsets = torch.empty(X + 1, dtype=torch.int32, device=DEV)
+    pairs = torch.full((T * k,), -7, dtype=torch.int32, device=DEV)
+    active = torch.full((X,), -1, dtype=torch.int32, device=DEV)
+    n_active = torch.empty(1, dtype=torch.int32, device=DEV)
+    o.moe_align(ids_d, X, counts, offsets, pairs, active, n_active)
+    flat = ids.flatten()
+    want_counts = torch.tensor([(flat == e).sum() for e in range(X)], dtype=torch.int32)
+    assert torch.equal(counts.cpu(), want_counts)
+    assert torch.equal(offsets.cpu(), torch.cat([torch.zeros(1, dtype=torch.int32), want_counts.cumsum(0).to(torch.int32)]))
+    want_pairs = torch.cat([torch.nonzero(flat == e).flatten() for e in range(X)]).to(torch.int32)
+    n_valid = int(want_counts.sum())
+    assert torch.equal(pairs.cpu()[:n_valid], want_pairs), "pairs are not grouped by expert in increasing pair order"
+    want_active = torch.nonzero(want_counts > 0).flatten().to(torch.int32)
+    assert int(n_active) == len(want_active) and torch.equal(active.cpu()[:len(want_active)], want_active)
+
+    act = torch.zeros(T * k, F, dtype=dtype, device=DEV)
+    o.grouped_gemm(h, wgu, act, offsets, pairs[:T * k], k, o.EPI_SWIGLU, active, n_active, token_rows=T)
+    y = torch.zeros(T * k, E, dtype=torch.float32, device=DEV)
+    o.grouped_gemm(act, wd, y, offsets, pairs, 1, o.EPI_STORE, active, n_active, token_rows=T)
+    x = rnd(T, E, seed=11)
+    x0 = x.clone()
+    o.moe_combine(x, y, ids_d, w_d, True)
+
+    hd, wgud, wdd = h.double().cpu(), wgu.double().cpu(), wd.double().cpu()
+    want = x0.double().cpu().clone()
+    act_want = torch.zeros(T * k, F, dtype=torch.float64)
+    for t in range(T):
+        acc = torch.zeros(E, dtype=torch.float64)
+        for j in range(k):
+            e = int(ids[t, j])
+            if e < 0:
+                continue
+            g = wgud[e, :F] @ hd[t]
+            u = wgud[e, F:] @ hd[t]
+            a = (g / (1 + torch.exp(-g))) * u
+            act_want[t * k + j] = a
+            a_in = act[t * k + j].double().cpu()   # the second product reads the stored (rounded) activation
+            acc = acc + float(w_pairs[t, j]) * (wdd[e] @ a_in)
+        want[t] += acc
+    tol = 2e-5 if dtype == torch.float32 else 1e-2
+    assert (act.double().cpu() - act_want).abs().max() <= tol * act_want.abs().max()
+    assert (x.double().cpu() - want).abs().max() <= 3e-5 * want.abs().max()
+    # the generic kernel gives the same rows (a row's bits depend on its own operands only; orders differ between kernels)
+    act_g = torch.zeros_like(act)
+    o.grouped_gemm(h, wgu, act_g, offsets, pairs, k, o.EPI_SWIGLU, force_generic=True)
+    assert (act_g.double().cpu() - act_want).abs().max() <= tol * act_want.abs().max()
+
+
+# ---------------------------------------------------------------------------
+def attention_case(T_lens, Hq, Hkv, D, R, page, dtype, window=0, shuffle_seed=0, norm=True, planned=True, second_single=False):
+    """Runs qknorm_rope_kvwrite + paged_attention for sequences of the given lengths, each cut into two steps, with
+    shuffled page tables, and returns (got, want) attention outputs in float64."""
+    o = ops()
+    eps = 1e-5
+    qw, kw = Hq * D, Hkv * D
+    n_seq = len(T_lens)
+    n_pages = sum(-(-L // page) for L in T_lens) + 3
+    order = list(range(n_pages))
+    random.Random(shuffle_seed).shuffle(order)
+    tables, at = [], 0
+    for L in T_lens:
+        nb = -(-L // page)
+        tables.append(order[at:at + nb])
+        at += nb
+    width = max(len(t) for t in tables)
+    table_t = torch.full((n_seq, width), -1, dtype=torch.int32)
+    for i, t in enumerate(tables):
+        table_t[i, :len(t)] = torch.tensor(t)
+    k_cache = torch.zeros(n_pages, Hkv, page, D, dtype=dtype, device=DEV)
+    v_cache = torch.zeros(n_pages, Hkv, D, page, dtype=dtype, device=DEV)
+    max_pos = max(T_lens)
+    cos, sin = plain_model.rope_tables(list(range(max_pos)), R, 10000.0) if R else (torch.zeros(max_pos, 0), torch.zeros(max_pos, 0))
+    cos_sin = torch.cat([cos, sin], dim=1).float().to(DEV).contiguous()
+    q_norm = (1 + 0.1 * rnd(qw, seed=3)) if norm else None
+    k_norm = (1 + 0.1 * rnd(kw, seed=4)) if norm else None
+    qkv_all = [rnd(L, qw + 2 * kw, seed=20 + i) for i, L in enumerate(T_lens)]
+    got = [None] * n_seq
+    # two steps: the first half of every sequence, then the rest (the second reads pages the first wrote)
+    for part in range(2):
+        rows, pos, ent = [], [], []
+        counts, contexts = [], []
+        for i, L in enumerate(T_lens):
+            a, b = (0, L // 2) if part == 0 else (L // 2, L)
+            if second_single:   # all but the last row first, then the last row alone (a decode row deep in its context)
+                a, b = (0, L - 1) if part == 0 else (L - 1, L)
+            rows.append(qkv_all[i][a:b])
+            pos += list(range(a, b))
+            ent += [i] * (b - a)
+            counts.append(b - a)
+            contexts.append(b)
+        qkv = torch.cat(rows).contiguous()
+        Tn = qkv.shape[0]
+        if Tn == 0:
+            continue
+        pos_t = torch.tensor(pos, dtype=torch.int32, device=DEV)
+        ent_t = torch.tensor(ent, dtype=torch.int32, device=DEV)
+        q = torch.empty(Tn, qw, dtype=dtype, device=DEV)
+        o.qknorm_rope_kvwrite(qkv, q_norm, k_norm, cos_sin, pos_t, ent_t, table_t.to(DEV), q, k_cache, v_cache, eps, Hq, Hkv, D, R,
+                              o.QKNORM_PROJECTION if norm else o.QKNORM_NONE)
+        out = torch.empty(Tn, qw, dtype=dtype, device=DEV)
+        plan = None
+        if planned and all(counts):
+            plan = o.attention_plan(counts, contexts, Hq, Hkv, DEV)
+        o.paged_attention(q, k_cache, v_cache, pos_t, ent_t, table_t.to(DEV), out, 1.0 / math.sqrt(D), Hq, window, plan=plan)
+        row = 0
+        for i, L in enumerate(T_lens):
+            a, b = (0, L // 2) if part == 0 else (L // 2, L)
+            if second_single:
+                a, b = (0, L - 1) if part == 0 else (L - 1, L)
+            piece = out[row:row + b - a].double().cpu()
+            got[i] = piece if got[i] is None else torch.cat([got[i], piece])
+            row += b - a
+    want = []
+    rt = None if dtype == torch.float32 else torch.bfloat16
+    for i, L in enumerate(T_lens):
+        x = qkv_all[i].double().cpu()
+        qq, kk, vv = x[:, :qw], x[:, qw:qw + kw], x[:, qw + kw:]
+        if norm:
+            qq = plain_model.rms_norm(qq, q_norm.double().cpu(), eps)
+            kk = plain_model.rms_norm(kk, k_norm.double().cpu(), eps)
+        c, s = cos[:L], sin[:L]
+        qq = plain_model.apply_partial_rope(qq.view(L, Hq, D), c, s, R)
+        kk = plain_model.apply_partial_rope(kk.view(L, Hkv, D), c, s, R)
+        qq, kk, vv = (plain_model._rounded(t, rt) for t in (qq, kk, vv.view(L, Hkv, D)))
+        want.append(plain_model.causal_attention(qq, kk, vv, window or None).reshape(L, qw))
+    return got, want
+
+
+@pytest.mark.parametrize("lens,Hq,Hkv,D,R,page", [((1, 2, 5), 4, 2, 16, 8, 4), ((37, 70), 6, 1, 24, 24, 8), ((130,), 8, 2, 64, 32, 16),
+                                                  ((200, 3), 12, 2, 128, 64, 16), ((33,), 2, 2, 48, 0, 16)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_with_rope_and_pages(lens, Hq, Hkv, D, R, page, dtype):
+    got, want = attention_case(lens, Hq, Hkv, D, R, page, dtype)
+    tol = 2e-5 if dtype == torch.float32 else 1.2e-2
+    for g, w in zip(got, want):
+        assert (g - w).abs().max() <= tol * w.abs().max()
+
+
+@pytest.mark.parametrize("lens,Hq,Hkv,D", [((1500,), 12, 2, 128), ((700, 1290, 33), 8, 8, 64), ((2100,), 40, 2, 48)])
+def test_attention_split_context(lens, Hq, Hkv, D):
+    """A decode row deep in a long context: the matrix-core kernel splits the keys over several items and merges them."""
+    o = ops()
+    got, want = attention_case(lens, Hq, Hkv, D, D // 2, 16, torch.bfloat16, second_single=True)
+    plan = o.attention_plan([1] * len(lens), list(lens), Hq, Hkv, DEV)
+    assert plan.n_merges > 0, "the context was not split"
+    for g, w in zip(got, want):
+        assert (g - w).abs().max() <= 1.2e-2 * w.abs().max()
+    universal, _ = attention_case(lens, Hq, Hkv, D, D // 2, 16, torch.bfloat16, second_single=True, planned=False)
+    for g, u in zip(got, universal):
+        assert (g - u).abs().max() <= 1.2e-2 * u.abs().max()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_window(dtype):
+    got, want = attention_case((90, 21), 4, 2, 32, 16, 8, dtype, window=17)
+    full, _ = attention_case((90, 21), 4, 2, 32, 16, 8, dtype, window=0)
+    tol = 2e-5 if dtype == torch.float32 else 1.2e-2
+    for g, w, f in zip(got, want, full):
+        assert (g - w).abs().max() <= tol * w.abs().max()
+        assert torch.equal(g[:17], f[:17]), "rows inside the window differ from full attention"
+        if len(g) > 40:
+            assert not torch.allclose(g[40:], f[40:]), "rows past the window equal full attention"
+
+
+def test_attention_finds_a_far_key():
+    """One key among hundreds is made to stand out: query and that key are scaled so its score dominates, and the
+    output must be that key's value, across page edges and whatever the table's order."""
+    o = ops()
+    Hq, Hkv, D, page, L = 4, 2, 32, 16, 333
+    for dtype in (torch.float32, torch.bfloat16):
+        for far in (0, 15, 16, 17, 200, 331):
+            n_pages = -(-L // page)
+            order = list(range(n_pages))
+            random.Random(far).shuffle(order)
+            table = torch.tensor([order], dtype=torch.int32, device=DEV)
+            k_cache = rnd(n_pages, Hkv, page, D, dtype=dtype, scale=0.1)
+            v_cache = rnd(n_pages, Hkv, D, page, dtype=dtype, seed=2)
+            q = rnd(1, Hq * D, dtype=dtype, scale=0.1, seed=3)
+            direction = torch.ones(D, device=DEV)
+            pg, sl = order[far // page], far % page
+            k_cache[pg, :, sl, :] = (6.0 * direction).to(dtype)
+            q[:] = (6.0 * direction).repeat(Hq).to(dtype)
+            out = torch.empty(1, Hq * D, dtype=dtype, device=DEV)
+            pos = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
+            ent = torch.zeros(1, dtype=torch.int32, device=DEV)
+            plan = o.attention_plan([1], [L], Hq, Hkv, DEV) if dtype == torch.bfloat16 else None
+            o.paged_attention(q, k_cache, v_cache, pos, ent, table, out, 1.0 / math.sqrt(D), Hq, plan=plan)
+            for h in range(Hq):
+                want = v_cache[pg, h // (Hq // Hkv), :, sl].float()
+                assert (out[0, h * D:(h + 1) * D].float() - want).abs().max() < 1e-2, f"key {far} was not found ({dtype})"
+
+
+# ---------------------------------------------------------------------------
+def test_route_topk_vectors():
+    """Levels with ties, infinities and a NaN; k in {1, 8, 24}; bias on/off; normalize on/off.  The method (not the
+    data) follows /root/reference/tests/minimax_ops.cpp:74-139: ids equal a stable sort by float(s)+bias descending,
+    weights close to s/sum*scale, a row with a non-finite key gives no expert, a row alone equals the row in a batch."""
+    o = ops()
+    X = 24
+    g = torch.Generator().manual_seed(5)
+    z = torch.randn(9, X, generator=g) * 2
+    z[1, 3] = z[1, 7] = z[1, 11] = 0.5          # ties
+    z[2] = 0.25                                  # all equal
+    z[3, 5] = float("inf")                       # sigmoid(inf) = 1, finite key
+    z[4, 2] = float("-inf")                      # sigmoid(-inf) = 0, finite key
+    z[5, 9] = float("nan")                       # non-finite key: no expert
+    bias = torch.randn(X, generator=g) * 0.3
+    for k in (1, 8, 24):
+        for use_bias in (False, True):
+            for normalize in (False, True):
+                ids = torch.empty(9, k, dtype=torch.int32, device=DEV)
+                w = torch.empty(9, k, dtype=torch.float32, device=DEV)
+                o.route_topk(z.to(DEV), bias.to(DEV) if use_bias else None, ids, w, k, o.SCORE_SIGMOID, normalize, 2.5)
+                s32 = 1.0 / (1.0 + torch.exp(-z))    # float32 scores as the kernel forms them
+                key = s32 + bias if use_bias else s32
+                for r in range(9):
+                    if not torch.isfinite(key[r]).all():
+                        assert (ids[r] == -1).all() and (w[r] == 0).all()
+                        continue
+                    order = sorted(range(X), key=lambda e: (-float(key[r, e]), e))[:k]
+                    assert ids[r].tolist() == order, f"row {r}, k {k}: picks {ids[r].tolist()} != {order}"
+                    chosen = s32[r, order].double()
+                    want = (chosen / chosen.sum() if normalize else chosen) * 2.5
+                    assert (w[r].double().cpu() - want).abs().max() <= (k + 8) * 2.0 ** -24 * want.abs().max()
+                # a row alone gives the bits it gives in the batch
+                ids1 = torch.empty(1, k, dtype=torch.int32, device=DEV)
+                w1 = torch.empty(1, k, dtype=torch.float32, device=DEV)
+                o.route_topk(z[6:7].to(DEV), bias.to(DEV) if use_bias else None, ids1, w1, k, o.SCORE_SIGMOID, normalize, 2.5)
+                assert torch.equal(ids1[0], ids[6]) and torch.equal(w1[0], w[6])
+
+
+def test_route_matches_plain_and_invariants():
+    o = ops()
+    T, X, k = 13, 40, 5
+    z = rnd(T, X, scale=1.5)
+    bias = 0.2 * rnd(X, seed=2)
+    ids = torch.empty(T, k, dtype=torch.int32, device=DEV)
+    w = torch.empty(T, k, dtype=torch.float32, device=DEV)
+    o.route_topk(z, bias, ids, w, k, o.SCORE_SIGMOID, True, 1.7)
+    pids, pw = plain_model.route(z.double().cpu(), bias.double().cpu(), k, True, 1.7)
+    assert torch.equal(ids.long().cpu(), pids)
+    assert (w.double().cpu() - pw).abs().max() < 1e-6
+    assert (w.sum(1) - 1.7).abs().max() < 1e-5            # normalized weights sum to the scale
+    # adding one constant to every bias changes nothing
+    ids2, w2 = torch.empty_like(ids), torch.empty_like(w)
+    o.route_topk(z, bias + 0.5, ids2, w2, k, o.SCORE_SIGMOID, True, 1.7)
+    assert torch.equal(ids2, ids) and torch.equal(w2, w)
+    # a huge bias forces an expert in, but its weight stays its unbiased score
+    big = bias.clone()
+    big[7] = 100.0
+    o.route_topk(z, big, ids2, w2, k, o.SCORE_SIGMOID, False, 1.0)
+    assert (ids2[:, 0] == 7).all()
+    assert (w2[:, 0].cpu() - torch.sigmoid(z[:, 7]).cpu()).abs().max() < 1e-6
+
+
+# ---------------------------------------------------------------------------
+def test_argmax_rows_vectors():
+    """Vectors the reference's own sampler test holds (/root/reference/tests/sampler.cpp:95-98) and the NaN rules."""
+    o = ops()
+    cases = [([0.5, 2.0, -1.0, 1.5], 1), ([-2.0, -0.5, -1.0], 1), ([1.0, 3.0, 0.0, 3.0], 1), ([3.0, 3.0, 3.0], 0),
+             ([float("nan"), 5.0, 1.0], 0), ([1.0, float("nan"), 5.0], 2), ([float("-inf")] * 3, 0)]
+    for row, want in cases:
+        s = torch.tensor([row], dtype=torch.float32, device=DEV)
+        out = torch.empty(1, dtype=torch.int32, device=DEV)
+        o.argmax_rows(s, out)
+        assert int(out) == want, (row, int(out))
+    V = 200064
+    s = rnd(3, V)
+    s[1, 77] = s[1, 150000] = 9.0
+    out = torch.empty(3, dtype=torch.int32, device=DEV)
+    o.argmax_rows(s, out)
+    assert out.tolist() == [int(s[0].argmax()), 77, int(s[2].argmax())]
+    skip = torch.tensor([int(out[0]), -1, -1], dtype=torch.int32, device=DEV)
+    out2 = torch.empty_like(out)
+    o.argmax_rows(s, out2, skip)
+    masked = s[0].clone()
+    masked[int(out[0])] = float("-inf")
+    assert int(out2[0]) == int(masked.argmax()) and out2[1:].tolist() == out[1:].tolist()
+
+
+@pytest.mark.parametrize("V", [320, 5000, 200064])
+def test_samplers_match_reference_draw_for_draw(V):
+    """Every draw equals a slow transcription of the reference's sampler fed the same uniform numbers."""
+    o = ops()
+    from llmx_amd.sampling import XorShift64
+    rows = 6
+    logits = rnd(rows, V, scale=2.0, seed=V)
+    settings = [dict(temp=0.8, top_k=0, top_p=1.0, min_p=0.0), dict(temp=1.3, top_k=0, top_p=1.0, min_p=0.05),
+                dict(temp=0.8, top_k=40, top_p=0.95, min_p=0.0), dict(temp=2.0, top_k=7, top_p=1.0, min_p=0.0),
+                dict(temp=1.0, top_k=300, top_p=0.5, min_p=0.1), dict(temp=0.5, top_k=1, top_p=0.3, min_p=0.0)]
+    rng = XorShift64(1234)
+    host = logits.cpu()
+    for draw in range(25):
+        units = [rng.unit() for _ in range(rows)]
+        unit = torch.tensor(units, dtype=torch.float32, device=DEV)
+        f = lambda key: torch.tensor([s[key] for s in settings], dtype=torch.float32, device=DEV)
+        out_all = torch.empty(rows, dtype=torch.int32, device=DEV)
+        out_top = torch.empty(rows, dtype=torch.int32, device=DEV)
+        o.sample_all(logits, f("temp"), unit, out_all, f("min_p"))
+        o.sample_topk(logits, f("temp"), torch.tensor([s["top_k"] for s in settings], dtype=torch.int32, device=DEV), f("top_p"),
+                      f("min_p"), unit, out_top)
+        for r, s in enumerate(settings):
+            want = sampler_reference.sample(host[r].tolist(), s["temp"], s["top_k"], s["top_p"], s["min_p"], units[r])
+            got = int(out_all[r]) if (s["top_k"] == 0 and s["top_p"] >= 1.0) else int(out_top[r])
+            assert got == want, f"draw {draw}, row {r} ({s}): device {got}, reference {want}"
+
+
+def test_sampling_frequencies():
+    """Empirical frequencies of 10,000 draws lie within 3 sigma of the softmax (method of sampler.cpp:41-53,128-150)."""
+    o = ops()
+    from llmx_amd.sampling import XorShift64
+    row = [0.2, 1.5, -0.3, 1.1, 0.9, -1.0, 1.3, 0.0]
+    n = 10000
+    rng = XorShift64(99)
+    logits = torch.tensor([row] * n, dtype=torch.float32, device=DEV)
+    unit = torch.tensor([rng.unit() for _ in range(n)], dtype=torch.float32, device=DEV)
+    for temp, top_k, kept in ((1.0, 0, range(8)), (2.0, 3, (1, 6, 3))):
+        out = torch.empty(n, dtype=torch.int32, device=DEV)
+        t = torch.full((n,), temp, device=DEV)
+        if top_k:
+            o.sample_topk(logits, t, torch.full((n,), top_k, dtype=torch.int32, device=DEV), torch.ones(n, device=DEV),
+                          torch.zeros(n, device=DEV), unit, out)
+        else:
+            o.sample_all(logits, t, unit, out)
+        w = torch.tensor([math.exp(row[i] / temp) if i in kept else 0.0 for i in range(8)], dtype=torch.float64)
+        p = w / w.sum()
+        counts = torch.bincount(out.long().cpu(), minlength=8).double()
+        sigma = torch.sqrt(n * p * (1 - p))
+        assert ((counts - n * p).abs() <= 3 * sigma + 1e-9).all(), (counts.tolist(), (n * p).tolist())
+
+
+def test_penalties():
+    """The reference's penalty cases (/root/reference/tests/sampler.cpp:101-113): a seen positive leader is divided, a
+    negative one multiplied, once however often it was seen."""
+    o = ops()
+
+    def greedy(row, penalty, seen, presence=0.0, frequency=0.0):
+        s = torch.tensor([row], dtype=torch.float32, device=DEV)
+        if seen:
+            from collections import Counter
+            c = Counter(seen)
+            i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+            f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=DEV)
+            o.penalize(s, i32([0] * len(c)), i32(list(c)), i32(list(c.values())), f32([penalty]), f32([presence]), f32([frequency]))
+        out = torch.empty(1, dtype=torch.int32, device=DEV)
+        o.argmax_rows(s, out)
+        return int(out), s[0].tolist()
+
+    assert greedy([3.0, 1.6, 0.0], 2.0, [0])[0] == 1
+    assert greedy([3.0, 1.4, 0.0], 2.0, [0])[0] == 0
+    assert greedy([-1.0, -1.9, -3.0], 2.0, [0])[0] == 1
+    assert greedy([-1.0, -2.1, -3.0], 2.0, [0])[0] == 0
+    assert greedy([3.0, 1.4, 0.0], 2.0, [0, 0, 0])[0] == 0
+    assert greedy([3.0, 1.6, 0.0], 1.0, [0])[0] == 0
+    assert greedy([3.0, 1.6, 0.0], 2.0, [])[0] == 0
+    _, row = greedy([3.0, 1.0, 0.0], 1.0, [0, 0, 1], presence=0.5, frequency=0.25)
+    assert row == [3.0 - 0.5 - 0.5, 1.0 - 0.5 - 0.25, 0.0]
+
+
+def test_fill_random_matches_host():
+    from llmx_amd.parts.spec import TensorSpec
+    from llmx_amd.weights import RandomInit, host_values
+    from llmx_amd.weights.device_init import fill_random
+    init = RandomInit(seed=3, std=0.05, norm_std=0.1, bias_range=0.2)
+    for spec in (TensorSpec("a.weight", (37, 53), "matrix"), TensorSpec("n.weight", (100,), "norm"), TensorSpec("b.bias", (64,), "bias")):
+        want = host_values(spec, init)
+        t = torch.empty(spec.shape, dtype=torch.float32, device=DEV)
+        fill_random(t, spec, init)
+        assert (t.cpu() - want).abs().max() < 1e-5
+    assert abs(float(host_values(TensorSpec("a.weight", (400, 400), "matrix"), init).std()) - 0.05) < 1e-3
