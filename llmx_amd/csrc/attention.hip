@@ -26,49 +26,57 @@ struct QkvArgs {
     int page_tokens, max_blocks, write_kv;
 };
 
-// One block per row.  Norm over the whole projection: the sum of squares of the row's q (or k) values, strided per
-// thread, butterfly per wave, waves in order.  Then y = x * (r * w) and the NeoX rotation of pairs (i, i + R/2) of
-// each head: a' = fma(-b, sin, a*cos), b' = fma(a, sin, b*cos); dims [R, D) pass through.
+// Two blocks per row: one norms and rotates q, the other norms and rotates k and writes k and v to the row's page.
+// Norm over the whole projection: the sum of squares of the row's q (or k) values, strided per thread, butterfly per
+// wave, waves in order.  Then y = x * (r * w) and the NeoX rotation of pairs (i, i + R/2) of each head:
+// a' = fma(-b, sin, a*cos), b' = fma(a, sin, b*cos); dims [R, D) pass through.
+__device__ __forceinline__ float normed_rotated(const float* __restrict__ row, const float* __restrict__ weight, const float* __restrict__ cs,
+                                                int i, int D, int rotary_dim, bool normed, float r) {
+    const int d = i % D, half = rotary_dim / 2;
+    float x = row[i];
+    if (normed) x = x * (r * weight[i]);
+    if (d < rotary_dim) {
+        const int j = d < half ? d : d - half;
+        const int other = d < half ? i + half : i - half;
+        float y = row[other];
+        if (normed) y = y * (r * weight[other]);
+        const float c = cs[j], s = cs[half + j];
+        x = d < half ? fmaf(-y, s, x * c) : fmaf(y, s, x * c);
+    }
+    return x;
+}
+
 template <typename TQ, typename TKV>
 __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
     __shared__ float scratch[4];
     const int t = blockIdx.x;
-    const int D = a.head_dim, half = a.rotary_dim / 2;
+    const int D = a.head_dim;
     const int qw = a.n_heads * D, kw = a.n_kv_heads * D;
     const float* row = a.qkv + (size_t)t * (qw + 2 * kw);
     const int p = a.pos[t];
     const float* cs = a.cos_sin + (size_t)p * a.rotary_dim;
-
-    float rq = 1.0f, rk = 1.0f;
-    if (a.norm_mode == QKNORM_PROJECTION) {
-        float s = 0.0f;
-        for (int i = threadIdx.x; i < qw; i += 256) s = fmaf(row[i], row[i], s);
-        s = block_sum<4>(s, scratch);
-        rq = 1.0f / sqrtf(s / (float)qw + a.eps);
-        s = 0.0f;
-        for (int i = threadIdx.x; i < kw; i += 256) s = fmaf(row[qw + i], row[qw + i], s);
-        s = block_sum<4>(s, scratch);
-        rk = 1.0f / sqrtf(s / (float)kw + a.eps);
-    }
     const bool normed = a.norm_mode != QKNORM_NONE;
-
-    // q: every (head, dim) once; the rotated pair is recomputed by both of its threads
-    TQ* q_out = (TQ*)a.q_out + (size_t)t * qw;
-    for (int i = threadIdx.x; i < qw; i += 256) {
-        const int d = i % D;
-        float x = row[i];
-        if (normed) x = x * (rq * a.q_weight[i]);
-        if (d < a.rotary_dim) {
-            const int j = d < half ? d : d - half;
-            const int other = d < half ? i + half : i - half;
-            float y = row[other];
-            if (normed) y = y * (rq * a.q_weight[other]);
-            const float c = cs[j], s = cs[half + j];
-            x = d < half ? fmaf(-y, s, x * c) : fmaf(y, s, x * c);
+    if (blockIdx.y == 0) {
+        float r = 1.0f;
+        if (a.norm_mode == QKNORM_PROJECTION) {
+            float s = 0.0f;
+            for (int i = threadIdx.x; i < qw; i += 256) s = fmaf(row[i], row[i], s);
+            s = block_sum<4>(s, scratch);
+            r = 1.0f / sqrtf(s / (float)qw + a.eps);
         }
-        st(q_out + i, x);
+        TQ* q_out = (TQ*)a.q_out + (size_t)t * qw;
+        for (int i = threadIdx.x; i < qw; i += 256) st(q_out + i, normed_rotated(row, a.q_weight, cs, i, D, a.rotary_dim, normed, r));
+        return;
     }
     if (!a.write_kv) return;
+    const float* krow = row + qw;
+    float r = 1.0f;
+    if (a.norm_mode == QKNORM_PROJECTION) {
+        float s = 0.0f;
+        for (int i = threadIdx.x; i < kw; i += 256) s = fmaf(krow[i], krow[i], s);
+        s = block_sum<4>(s, scratch);
+        r = 1.0f / sqrtf(s / (float)kw + a.eps);
+    }
     const int e = a.row_entry[t];
     const int page = a.tables[(size_t)e * a.max_blocks + p / a.page_tokens];
     const int slot = p % a.page_tokens;
@@ -76,19 +84,9 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
     TKV* vc = (TKV*)a.v_cache;
     for (int i = threadIdx.x; i < kw; i += 256) {
         const int h = i / D, d = i % D;
-        float x = row[qw + i];
-        if (normed) x = x * (rk * a.k_weight[i]);
-        if (d < a.rotary_dim) {
-            const int j = d < half ? d : d - half;
-            const int other = d < half ? i + half : i - half;
-            float y = row[qw + other];
-            if (normed) y = y * (rk * a.k_weight[other]);
-            const float c = cs[j], s = cs[half + j];
-            x = d < half ? fmaf(-y, s, x * c) : fmaf(y, s, x * c);
-        }
         const size_t head_at = (size_t)page * a.n_kv_heads + h;
-        st(kc + (head_at * a.page_tokens + slot) * D + d, x);
-        st(vc + (head_at * D + d) * a.page_tokens + slot, row[qw + kw + i]);
+        st(kc + (head_at * a.page_tokens + slot) * D + d, normed_rotated(krow, a.k_weight, cs, i, D, a.rotary_dim, normed, r));
+        st(vc + (head_at * D + d) * a.page_tokens + slot, krow[kw + i]);
     }
 }
 
@@ -100,10 +98,11 @@ extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight,
     if (norm_mode != QKNORM_NONE && norm_mode != QKNORM_PROJECTION) return -2;
     QkvArgs a{qkv, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
               n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv};
+    const dim3 grid(rows, 2);
     if (dtype == LLMX_F32)
-        hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<float, float>), dim3(rows), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<float, float>), grid, dim3(256), 0, stream, a);
     else
-        hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<bf16_t, bf16_t>), dim3(rows), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, stream, a);
     return LLMX_CHECK_LAUNCH();
 }
 

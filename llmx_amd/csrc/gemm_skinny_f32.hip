@@ -1,0 +1,112 @@
+// True 32-bit weight-streaming product on the matrix cores: C[M,N] (+)= A[M,K] * W[N,K]^T, all float32
+// (v_mfma_f32_16x16x4_f32 multiplies and adds full float32 values; there is no reduced-precision mode in it).
+// Used for the router logits, which are always float32.  Same shape as the bfloat16 streaming kernel: KS waves share
+// one strip of 16 output features, each lane loads 16 bytes (4 consecutive k) of its row, which feed 4 products; rows
+// come in tiles of 16, up to 4 tiles held at once, more by walking W again.  An output's bits depend on K and KS only.
+#include "common.h"
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+struct SkinnyF32Args {
+    const float* A;
+    const float* W;
+    float* C;
+    int M, N, K, lda, ldc, add;
+};
+
+template <int KS, int MT>
+__global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args g) {
+    __shared__ float red[KS > 1 ? KS : 1][MT][256];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, kg = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int K = g.K;
+    const int steps_total = (K + 15) >> 4;
+    const int per = (steps_total + KS - 1) / KS;
+    const int s_begin = wave * per, s_end = min(steps_total, s_begin + per);
+    const float* wp = g.W + (size_t)min(n0 + r, g.N - 1) * K + kg * 4;
+
+    // blockIdx.y walks the rows in chunks of 16*MT, so many rows spread over the chip (each chunk reads the strip again, from L2)
+    for (int m0 = blockIdx.y * 16 * MT; m0 < g.M; m0 += gridDim.y * 16 * MT) {
+        const float* ap[MT];
+        bool a_in[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int m = m0 + t * 16 + r;
+            a_in[t] = m < g.M;
+            ap[t] = g.A + (size_t)(a_in[t] ? m : 0) * g.lda + kg * 4;
+        }
+        f32x4_t acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int s = s_begin; s < s_end; s += 2) {
+            f32x4_t wf[2], af[2][MT];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int k = (s + u) * 16 + kg * 4;
+                const bool in = (s + u) < s_end && k < K;   // K is a multiple of 4: a lane's 4 values are all in or all out
+                wf[u] = in ? *reinterpret_cast<const f32x4_t*>(wp + (size_t)(s + u) * 16) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    af[u][t] = (in && a_in[t]) ? *reinterpret_cast<const f32x4_t*>(ap[t] + (size_t)(s + u) * 16) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[u][i], af[u][t][i], acc[t], 0, 0, 0);
+        }
+        if (KS > 1) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4_t*>(&red[wave][t][lane * 4]) = acc[t];
+            __syncthreads();
+        }
+        if (wave == 0) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                f32x4_t v = acc[t];
+                if (KS > 1) {
+                    v = *reinterpret_cast<f32x4_t*>(&red[0][t][lane * 4]);
+#pragma unroll
+                    for (int w = 1; w < KS; ++w) {
+                        const f32x4_t o = *reinterpret_cast<f32x4_t*>(&red[w][t][lane * 4]);
+                        v = f32x4_t{v[0] + o[0], v[1] + o[1], v[2] + o[2], v[3] + o[3]};
+                    }
+                }
+                const int m = m0 + t * 16 + r;
+                if (m >= g.M) continue;
+                float* c = g.C + (size_t)m * g.ldc + n0 + 4 * kg;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (n0 + 4 * kg + i >= g.N) continue;
+                    c[i] = g.add ? c[i] + v[i] : v[i];
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// K a multiple of 4, rows 16-byte aligned.  ks: 1, 2, 4 or 8.
+extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, int M, int N, int K, int lda, int ldc, int add, int ks,
+                                    hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (K % 4) return -2;
+    SkinnyF32Args g{A, W, C, M, N, K, lda, ldc, add};
+    int chunks = (M + 63) / 64;
+    if (chunks > 1024) chunks = 1024;
+    const dim3 grid((N + 15) / 16, M <= 64 ? 1 : chunks);
+#define SKF_LAUNCH(KS, MT) hipLaunchKernelGGL((gemm_skinny_f32_kernel<KS, MT>), grid, dim3(64 * KS), 0, stream, g)
+#define SKF_MT(KS) do { if (M <= 16) SKF_LAUNCH(KS, 1); else if (M <= 32) SKF_LAUNCH(KS, 2); else SKF_LAUNCH(KS, 4); } while (0)
+    switch (ks) {
+        case 1: SKF_MT(1); break;
+        case 2: SKF_MT(2); break;
+        case 4: SKF_MT(4); break;
+        case 8: SKF_MT(8); break;
+        default: return -2;
+    }
+#undef SKF_MT
+#undef SKF_LAUNCH
+    return LLMX_CHECK_LAUNCH();
+}

@@ -1,0 +1,245 @@
+// LDS-tiled bf16 product for many rows (prompt portions): C[M,N] (+)= A[M,K] * W[N,K]^T on the matrix cores.
+//
+// A workgroup of 4 waves computes a 128 x 128 tile (each wave 64 x 64 as 2 x 2 products of 32x32x16); K is walked 64 at a
+// time: the next A and W tiles travel from global memory into registers while the current ones are multiplied out of LDS
+// (rows padded to 144 bytes so that the 16-byte operand reads of 8 consecutive rows fall into different banks).
+// Grouped form: blockIdx.y walks the (expert, row tile) pairs of the experts that have rows; A's rows are gathered
+// through the expert-sorted pair list and C's rows scattered to the pairs.  SwiGLU form: the tile's 128 weight rows
+// are 64 gate rows and the 64 up rows of the same features, and silu(gate) * up is stored.
+// An output element is one accumulator walked over k in steps of 16: its bits depend on K only.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+enum : int { TL_STORE = 0, TL_ADD = 1, TL_SWIGLU = 2 };
+
+#define TL_BM 128
+#define TL_BN 128
+#define TL_BK 64
+#define TL_LD 72  // padded row length in bf16 elements (144 bytes)
+
+struct TileArgs {
+    const bf16_t* A;
+    const bf16_t* W;
+    void* C;
+    int M, N, K;
+    int lda, ldc;
+    const int* group_offsets;  // grouped: [G+1]
+    const int* list;
+    int n_groups, a_div;
+    long w_group_stride;
+    int up_offset;
+    int m_tiles;  // dense: number of row tiles
+};
+
+template <int EPI, typename TC, bool GROUPED>
+__global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
+    __shared__ __attribute__((aligned(16))) bf16_t As[TL_BM * TL_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[TL_BN * TL_LD];
+    __shared__ int rows_a[TL_BM];
+    __shared__ int rows_c[TL_BM];
+    __shared__ int tile_info[2];
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    constexpr int FEATS = (EPI == TL_SWIGLU) ? 64 : 128;  // output features a workgroup covers
+    const int n0 = blockIdx.x * FEATS;
+    const bf16_t* W = g.W;
+    int row_begin, row_end;
+    if (GROUPED) {
+        // which (expert, row tile) this workgroup has: experts in order, each with ceil(rows / 128) tiles
+        if (tid == 0) {
+            int left = blockIdx.y, found = -1, tile = 0;
+            for (int e = 0; e < g.n_groups; ++e) {
+                const int tiles = (g.group_offsets[e + 1] - g.group_offsets[e] + TL_BM - 1) / TL_BM;
+                if (left < tiles) {
+                    found = e;
+                    tile = left;
+                    break;
+                }
+                left -= tiles;
+            }
+            tile_info[0] = found;
+            tile_info[1] = tile;
+        }
+        __syncthreads();
+        const int e = tile_info[0];
+        if (e < 0) return;
+        row_begin = g.group_offsets[e] + tile_info[1] * TL_BM;
+        row_end = min(g.group_offsets[e + 1], row_begin + TL_BM);
+        W += (size_t)e * g.w_group_stride;
+    } else {
+        row_begin = blockIdx.y * TL_BM;
+        row_end = min(g.M, row_begin + TL_BM);
+    }
+    if (tid < TL_BM) {
+        const int m = row_begin + tid;
+        int ra = -1, rc = -1;
+        if (m < row_end) {
+            if (GROUPED) {
+                const int p = g.list[m];
+                ra = p / g.a_div;
+                rc = p;
+            } else {
+                ra = rc = m;
+            }
+        }
+        rows_a[tid] = ra;
+        rows_c[tid] = rc;
+    }
+    __syncthreads();
+
+    // global -> register staging: 1024 chunks of 16 bytes per tile, 4 per thread; chunk c: row c/8, k offset (c%8)*8
+    const int K = g.K;
+    const bf16_t* a_src[4];
+    const bf16_t* w_src[4];
+    bool a_ok[4], w_ok[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = tid + 256 * i;
+        const int row = c >> 3, kc = (c & 7) * 8;
+        const int ra = rows_a[row];
+        a_ok[i] = ra >= 0;
+        a_src[i] = g.A + (size_t)(ra >= 0 ? ra : 0) * g.lda + kc;
+        int wr;
+        if (EPI == TL_SWIGLU) {
+            const int f = n0 + (row & 63);
+            w_ok[i] = f < g.N;
+            wr = (row < 64 ? 0 : g.up_offset) + min(f, g.N - 1);
+        } else {
+            const int f = n0 + row;
+            w_ok[i] = f < g.N;
+            wr = min(f, g.N - 1);
+        }
+        w_src[i] = W + (size_t)wr * K + kc;
+    }
+    u32x4_t a_reg[4], w_reg[4];
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int kc = ((tid + 256 * i) & 7) * 8;
+            const bool in = k0 + kc < K;
+            a_reg[i] = (in && a_ok[i]) ? *reinterpret_cast<const u32x4_t*>(a_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
+            w_reg[i] = (in && w_ok[i]) ? *reinterpret_cast<const u32x4_t*>(w_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
+        }
+    };
+    auto store_lds = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + 256 * i;
+            const int row = c >> 3, kc = (c & 7) * 8;
+            *reinterpret_cast<u32x4_t*>(&As[row * TL_LD + kc]) = a_reg[i];
+            *reinterpret_cast<u32x4_t*>(&Ws[row * TL_LD + kc]) = w_reg[i];
+        }
+    };
+
+    // wave (wm, wn): rows 64*wm .., and its two column tiles
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lr = lane & 31, lk = (lane >> 5) * 8;
+    int b_row[2];
+    if (EPI == TL_SWIGLU) {
+        b_row[0] = 32 * wn + lr;        // gate rows of features n0 + 32*wn + lr
+        b_row[1] = 64 + 32 * wn + lr;   // up rows of the same features
+    } else {
+        b_row[0] = 64 * wn + lr;
+        b_row[1] = 64 * wn + 32 + lr;
+    }
+    f32x16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    load_global(0);
+    store_lds();
+    __syncthreads();
+    for (int k0 = 0; k0 < K; k0 += TL_BK) {
+        const bool more = k0 + TL_BK < K;
+        if (more) load_global(k0 + TL_BK);
+#pragma unroll
+        for (int kk = 0; kk < TL_BK; kk += 16) {
+            bf16x8_t af[2], bf[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+                af[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[(64 * wm + 32 * i + lr) * TL_LD + kk + lk]));
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                bf[j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[b_row[j] * TL_LD + kk + lk]));
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+        if (more) {
+            store_lds();
+            __syncthreads();
+        }
+    }
+
+    // acc[i][j][v]: row 64*wm + 32*i + 8*(v/4) + 4*(lane/32) + v%4, column lane%32 of column tile j
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int row = 64 * wm + 32 * i + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+            const int rc = rows_c[row];
+            if (rc < 0) continue;
+            if (EPI == TL_SWIGLU) {
+                const int n = n0 + 32 * wn + lr;
+                if (n < g.N) {
+                    const float gt = acc[i][0][v], u = acc[i][1][v];
+                    st((TC*)g.C + (size_t)rc * g.ldc + n, (gt / (1.0f + expf(-gt))) * u);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int n = n0 + 64 * wn + 32 * j + lr;
+                    if (n >= g.N) continue;
+                    TC* c = (TC*)g.C + (size_t)rc * g.ldc + n;
+                    float x = acc[i][j][v];
+                    if (EPI == TL_ADD) x = ld(c) + x;
+                    st(c, x);
+                }
+            }
+        }
+}
+
+template <int EPI, typename TC>
+static void tile_launch(const TileArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
+    if (grouped)
+        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, true>), grid, dim3(256), 0, stream, g);
+    else
+        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, false>), grid, dim3(256), 0, stream, g);
+}
+
+// A and W bfloat16, K a multiple of 8.  n_groups == 0: dense over M rows.  n_groups > 0: grouped over the n_pairs = M
+// rows of `list`; `max_tiles` bounds the (expert, row tile) pairs (at most min(groups, pairs) + pairs / 128).
+extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi,
+                              int n_groups, int max_tiles, const int* group_offsets, const int* list, int a_div, long w_group_stride,
+                              int up_offset, hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (K % 8) return -2;
+    const bool grouped = n_groups > 0;
+    TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
+               w_group_stride, up_offset, (M + TL_BM - 1) / TL_BM};
+    const int feats = epi == TL_SWIGLU ? 64 : 128;
+    dim3 grid((N + feats - 1) / feats, grouped ? max_tiles : g.m_tiles, 1);
+    if (grid.y > 65535) return -2;
+    if (epi == TL_SWIGLU) {
+        if (c_dtype == LLMX_BF16) tile_launch<TL_SWIGLU, bf16_t>(g, grid, grouped, stream);
+        else tile_launch<TL_SWIGLU, float>(g, grid, grouped, stream);
+    } else if (epi == TL_ADD) {
+        if (c_dtype != LLMX_F32) return -2;
+        tile_launch<TL_ADD, float>(g, grid, grouped, stream);
+    } else if (epi == TL_STORE) {
+        if (c_dtype == LLMX_BF16) tile_launch<TL_STORE, bf16_t>(g, grid, grouped, stream);
+        else tile_launch<TL_STORE, float>(g, grid, grouped, stream);
+    } else {
+        return -2;
+    }
+    return LLMX_CHECK_LAUNCH();
+}

@@ -139,10 +139,48 @@ __global__ void __launch_bounds__(64) moe_place_kernel(const int* __restrict__ i
     }
 }
 
+// Few pairs (a decode step): one workgroup does it all.  Thread e owns expert e: it counts its pairs, the counts are
+// scanned in expert order, and it places its pairs in increasing pair order.
+#define ALIGN_SMALL_PAIRS 1024
+__global__ void __launch_bounds__(1024) moe_align_small_kernel(const int* __restrict__ ids, int n_pairs, int n_experts, int* __restrict__ counts,
+                                                              int* __restrict__ offsets, int* __restrict__ list, int* __restrict__ active,
+                                                              int* __restrict__ n_active) {
+    __shared__ int pair_expert[ALIGN_SMALL_PAIRS];
+    __shared__ int cnt[1024];
+    const int e = threadIdx.x;
+    for (int p = e; p < n_pairs; p += 1024) pair_expert[p] = ids[p];
+    __syncthreads();
+    int c = 0;
+    if (e < n_experts)
+        for (int p = 0; p < n_pairs; ++p) c += pair_expert[p] == e;
+    cnt[e] = c;
+    __syncthreads();
+    if (e >= n_experts) return;
+    int before = 0, active_before = 0;
+    for (int i = 0; i < e; ++i) {
+        before += cnt[i];
+        active_before += cnt[i] > 0;
+    }
+    counts[e] = c;
+    offsets[e] = before;
+    if (c > 0) active[active_before] = e;
+    if (e == n_experts - 1) {
+        offsets[n_experts] = before + c;
+        n_active[0] = active_before + (c > 0);
+    }
+    int at = before;
+    for (int p = 0; p < n_pairs && c > 0; ++p)
+        if (pair_expert[p] == e) list[at++] = p;
+}
+
 // counts [X], offsets [X+1], list [n_pairs], active [X], n_active [1]
 extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* counts, int* offsets, int* list, int* active, int* n_active,
                               hipStream_t stream) {
     if (n_pairs <= 0 || n_experts <= 0) return 0;
+    if (n_pairs <= ALIGN_SMALL_PAIRS && n_experts <= 1024) {
+        hipLaunchKernelGGL(moe_align_small_kernel, dim3(1), dim3(1024), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
+        return LLMX_CHECK_LAUNCH();
+    }
     hipLaunchKernelGGL(moe_count_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, counts);
     hipLaunchKernelGGL(moe_place_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
     return LLMX_CHECK_LAUNCH();

@@ -56,22 +56,23 @@ extern "C" int llmx_rmsnorm(const float* x, const int* pick, const float* w, flo
 
 // ---------------------------------------------------------------------------
 // Expert combine: x[t,:] += sum_j w[t,j] * y[t*k+j,:], j in slot order; a slot without an expert (id < 0) adds nothing.
-__global__ void moe_combine_kernel(float* __restrict__ x, const float* __restrict__ y, const int* __restrict__ ids,
-                                   const float* __restrict__ w, int k, int width, int accumulate) {
-    const int t = blockIdx.x;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        float s = 0.0f;
-        for (int j = 0; j < k; ++j)
-            if (ids[t * k + j] >= 0) s += w[t * k + j] * y[((size_t)t * k + j) * width + i];
-        float* o = x + (size_t)t * width + i;
-        *o = accumulate ? *o + s : s;
-    }
+// One thread per output element, so the k loads of an element are independent and in flight together.
+__global__ void __launch_bounds__(256) moe_combine_kernel(float* __restrict__ x, const float* __restrict__ y, const int* __restrict__ ids,
+                                                        const float* __restrict__ w, int k, int width, int accumulate) {
+    const int t = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= width) return;
+    float s = 0.0f;
+    for (int j = 0; j < k; ++j)
+        if (ids[t * k + j] >= 0) s += w[t * k + j] * y[((size_t)t * k + j) * width + i];
+    float* o = x + (size_t)t * width + i;
+    *o = accumulate ? *o + s : s;
 }
 
 extern "C" int llmx_moe_combine(float* x, const float* y, const int* ids, const float* w, int rows, int k, int width, int accumulate,
                                 hipStream_t stream) {
     if (rows <= 0) return 0;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(rows), dim3(256), 0, stream, x, y, ids, w, k, width, accumulate);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((width + 255) / 256, rows), dim3(256), 0, stream, x, y, ids, w, k, width, accumulate);
     return LLMX_CHECK_LAUNCH();
 }
 

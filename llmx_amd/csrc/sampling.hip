@@ -56,9 +56,69 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) argmax_rows_kernel(const float
     if (threadIdx.x == 0) out[r] = id;
 }
 
-extern "C" int llmx_argmax_rows(const float* scores, const int* skip, int* out, int rows, int n, hipStream_t stream) {
+// Wide rows in two stages: each block takes the leader of one slice of a row, then one wave per row merges the slices'
+// leaders in slice order (so ties still go to the lowest id) and applies the NaN-leader rule.
+#define ARGMAX_SLICE 8192
+__global__ void __launch_bounds__(256) argmax_slices_kernel(const float* __restrict__ scores, const int* __restrict__ skip,
+                                                           Leader* __restrict__ partial, int n, int n_slices) {
+    __shared__ Leader scratch[4];
+    const int r = blockIdx.y, sl = blockIdx.x;
+    const float* s = scores + (size_t)r * n;
+    const int sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
+    const int first = sk == 0 ? 1 : 0;
+    const int begin = max(first, sl * ARGMAX_SLICE), end = min(n, (sl + 1) * ARGMAX_SLICE);
+    Leader best{-INFINITY, -1};
+    for (int i = begin + threadIdx.x; i < end; i += 256) {
+        if (i == sk) continue;
+        const Leader c{s[i], i};
+        if (c.score == c.score && beats(c, best)) best = c;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        Leader other{__shfl_xor(best.score, o, 64), __shfl_xor(best.id, o, 64)};
+        if (beats(other, best)) best = other;
+    }
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x / 64] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        best = scratch[0];
+        for (int w = 1; w < 4; ++w)
+            if (beats(scratch[w], best)) best = scratch[w];
+        partial[(size_t)r * n_slices + sl] = best;
+    }
+}
+
+__global__ void __launch_bounds__(64) argmax_merge_kernel(const float* __restrict__ scores, const int* __restrict__ skip,
+                                                         const Leader* __restrict__ partial, int* __restrict__ out, int n, int n_slices) {
+    const int r = blockIdx.x;
+    Leader best{-INFINITY, -1};
+    for (int i = threadIdx.x; i < n_slices; i += 64) {
+        const Leader c = partial[(size_t)r * n_slices + i];
+        if (beats(c, best)) best = c;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        Leader other{__shfl_xor(best.score, o, 64), __shfl_xor(best.id, o, 64)};
+        if (beats(other, best)) best = other;
+    }
+    if (threadIdx.x == 0) {
+        const int sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
+        const int first = sk == 0 ? 1 : 0;
+        const float lead = scores[(size_t)r * n + first];
+        out[r] = (lead != lead || best.id < 0) ? first : best.id;
+    }
+}
+
+// `partial` holds rows * ceil(n / 8192) leaders (8 bytes each); it may be null for rows of at most 16384 scores.
+extern "C" int llmx_argmax_rows(const float* scores, const int* skip, int* out, void* partial, int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
-    hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, skip, out, n);
+    if (n <= 2 * ARGMAX_SLICE || !partial) {
+        hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, skip, out, n);
+        return LLMX_CHECK_LAUNCH();
+    }
+    const int n_slices = (n + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
+    hipLaunchKernelGGL(argmax_slices_kernel, dim3(n_slices, rows), dim3(256), 0, stream, scores, skip, (Leader*)partial, n, n_slices);
+    hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(64), 0, stream, scores, skip, (const Leader*)partial, out, n, n_slices);
     return LLMX_CHECK_LAUNCH();
 }
 

@@ -63,7 +63,9 @@ def _declare(h) -> None:
         "llmx_route_topk": [P, P, P, P, I, I, I, I, I, F, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P],
         "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P],
-        "llmx_argmax_rows": [P, P, P, I, I, P],
+        "llmx_argmax_rows": [P, P, P, P, I, I, P],
+        "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, P],
+        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
@@ -160,6 +162,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
                                       _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()),
                "gemm_skinny")
         return
+    if not force_generic and _skinny_ok(a, w, c, epilogue):
+        _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue, 0, 0, 0, 0, 1, 0,
+                                    N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm_tile")
+        return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm")
 
@@ -189,6 +195,12 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
                                       _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
                                       _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
                "grouped_gemm_skinny")
+        return
+    if not force_generic and _skinny_ok(a, w, c, epilogue):
+        _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue, G,
+                                    min(G, n_pairs) + n_pairs // 128, _dev(offsets, "offsets", torch.int32, (G + 1,)),
+                                    _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
+               "grouped_gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    n_pairs, N, K, K, K, N, epilogue, G, _dev(offsets, "offsets", torch.int32, (G + 1,)),
@@ -357,10 +369,42 @@ def fill_random(t: torch.Tensor, key: int, kind: int, a: float, b: float) -> Non
                                   _stream()), "fill_random")
 
 
+_SCRATCH: dict = {}
+
+
+def _scratch(name: str, count: int, dtype: torch.dtype, device) -> torch.Tensor:
+    """A cached device buffer of at least `count` elements (grown, never shrunk): storage the kernels need besides their operands."""
+    key = (name, dtype, str(device))
+    t = _SCRATCH.get(key)
+    if t is None or t.numel() < count:
+        t = torch.empty(max(count, 1), dtype=dtype, device=device)
+        _SCRATCH[key] = t
+    return t
+
+
 def argmax_rows(scores: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Tensor] = None) -> None:
     rows, n = scores.shape
+    partial = _scratch("argmax.partial", 2 * rows * (-(-n // 8192)), torch.int32, scores.device) if n > 16384 else None
     _check(lib().llmx_argmax_rows(_dev(scores, "scores", torch.float32), _dev(skip, "skip", torch.int32, (rows,)),
-                                  _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()), "argmax_rows")
+                                  _dev(out, "out", torch.int32, (rows,)), _dev(partial, "partial"), rows, n, _stream()), "argmax_rows")
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, add: bool = False) -> None:
+    """c[M,N] (+)= a[M,K] @ w[N,K]^T, everything float32, on the float32 matrix instruction (the router's product).
+    A row's bits depend on the shape of w only.  K a multiple of 4; otherwise the universal kernel runs."""
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or tuple(c.shape) != (M, N):
+        raise KernelError(f"gemm_f32 shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
+    if K % 4:
+        gemm(a, w, c, EPI_ADD if add else EPI_STORE, force_generic=True)
+        return
+    ks = 1
+    n_strips = -(-N // 16)
+    while ks < 8 and n_strips * ks < 1024 and (K // 16) // (ks * 2) >= 8:
+        ks *= 2
+    _check(lib().llmx_gemm_skinny_f32(_dev(a, "a", torch.float32), _dev(w, "w", torch.float32), _dev(c, "c", torch.float32), M, N, K, K, N,
+                                      1 if add else 0, ks, _stream()), "gemm_f32")
 
 
 def sample_all(scores: torch.Tensor, temp: torch.Tensor, unit: torch.Tensor, out: torch.Tensor, min_p: Optional[torch.Tensor] = None,

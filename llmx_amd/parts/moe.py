@@ -79,7 +79,7 @@ class RoutedExperts(FeedForward):
     def route(self, step, h32):
         T, X, k = step.rows, self.experts, self.top_k
         z = step.buf("experts.router_logits", (T, X), torch.float32)
-        ops.gemm(h32, self.w_router, z)
+        ops.gemm_f32(h32, self.w_router, z)
         ids = step.buf("experts.ids", (T, k), torch.int32)
         weights = step.buf("experts.weights", (T, k), torch.float32)
         ops.route_topk(z, self.bias, ids, weights, k, self.score, self.normalize, self.scale)

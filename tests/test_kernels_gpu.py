@@ -69,7 +69,8 @@ def test_rmsnorm(rows, width, eps):
 
 
 # ---------------------------------------------------------------------------
-GEMM_SHAPES = [(1, 16, 32), (2, 48, 96), (3, 100, 72), (17, 200, 3072), (64, 96, 192), (65, 130, 264), (8, 8192, 3072), (33, 3072, 6144)]
+GEMM_SHAPES = [(1, 16, 32), (2, 48, 96), (3, 100, 72), (17, 200, 3072), (64, 96, 192), (65, 130, 264), (8, 8192, 3072), (33, 3072, 6144),
+               (129, 72, 40), (300, 257, 136), (2048, 512, 3072)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
@@ -96,8 +97,8 @@ def test_gemm_generic(M, N, K, dtypes):
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
-def test_gemm_skinny_bf16(M, N, K):
-    """The matrix-core kernel for few rows (it is taken for bfloat16 operands, K a multiple of 8, at most 64 rows)."""
+def test_gemm_matrix_cores_bf16(M, N, K):
+    """The matrix-core kernels (bfloat16 operands, K a multiple of 8): weight streaming up to 64 rows, LDS tiles above."""
     o = ops()
     a = rnd(M, K, dtype=torch.bfloat16)
     w = rnd(N, K, dtype=torch.bfloat16, seed=1)
@@ -119,7 +120,32 @@ def test_gemm_skinny_bf16(M, N, K):
     assert torch.equal(acc, base + c)
 
 
-@pytest.mark.parametrize("M,F,K", [(1, 32, 64), (3, 48, 96), (17, 1536, 3072), (70, 40, 72)])
+@pytest.mark.parametrize("M,N,K", [(1, 8, 64), (3, 16, 96), (8, 256, 3072), (17, 24, 100), (70, 40, 72), (2048, 256, 3072), (5, 13, 30)])
+def test_gemm_f32_matrix_cores(M, N, K):
+    """The router's product: true float32 on the float32 matrix instruction; a row's bits do not depend on the batch."""
+    o = ops()
+    a = rnd(M, K)
+    w = rnd(N, K, seed=1)
+    want = a.double().cpu() @ w.double().cpu().T
+    c = torch.full((M, N), float("nan"), device=DEV)
+    o.gemm_f32(a, w, c)
+    assert (c.double().cpu() - want).abs().max() <= 2e-6 * math.sqrt(K) * want.abs().max()
+    c1 = torch.empty(1, N, device=DEV)
+    o.gemm_f32(a[M - 1:M].contiguous(), w, c1)
+    assert torch.equal(c1[0], c[M - 1])
+    # no reduced-precision mode: operands that differ only below bfloat16's and tf32's precision give different results
+    a2 = a.clone()
+    a2[0, 0] += a2[0, 0].abs() * 2.0 ** -20 + 2.0 ** -30
+    c2 = torch.empty_like(c)
+    o.gemm_f32(a2, w, c2)
+    big = torch.zeros(1, K, device=DEV); big[0, 0] = 1.0
+    wb = torch.zeros(N, K, device=DEV); wb[:, 0] = 1.0 + 2.0 ** -20
+    cb = torch.empty(1, N, device=DEV)
+    o.gemm_f32(big, wb, cb)
+    assert torch.equal(cb, torch.full((1, N), 1.0 + 2.0 ** -20, device=DEV)), "low mantissa bits of the operands were dropped"
+
+
+@pytest.mark.parametrize("M,F,K", [(1, 32, 64), (3, 48, 96), (17, 1536, 3072), (70, 40, 72), (200, 100, 264)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gemm_swiglu(M, F, K, dtype):
     a = rnd(M, K, dtype=dtype)
@@ -145,7 +171,8 @@ def routed_setup(T, X, k, seed):
     return ids
 
 
-@pytest.mark.parametrize("T,X,k,E,F", [(1, 8, 2, 64, 32), (5, 16, 4, 96, 48), (17, 24, 3, 72, 40), (40, 256, 8, 256, 128), (150, 6, 2, 64, 32)])
+@pytest.mark.parametrize("T,X,k,E,F", [(1, 8, 2, 64, 32), (5, 16, 4, 96, 48), (17, 24, 3, 72, 40), (40, 256, 8, 256, 128), (150, 6, 2, 64, 32),
+                                       (700, 5, 2, 136, 72)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_routed_products(T, X, k, E, F, dtype):
     """moe_align, the two grouped products and the combine against a loop over pairs; experts without rows included."""
