@@ -14,16 +14,22 @@ from .base import PositionEncoding, register
 
 
 def neox_table(positions: int, rotary_dim: int, theta: float) -> np.ndarray:
-    """[positions, rotary_dim] float32: cos of the rotary_dim/2 pairs, then sin, every step in float32."""
+    """[positions, rotary_dim] float32: cos of the rotary_dim/2 pairs, then sin.
+
+    Every value is what correctly rounded float32 functions give: the power, the cosine and the sine are computed in
+    float64 from their float32 arguments and rounded once (vectorised float32 routines lose bits in the range reduction
+    of large angles, and a position of 65,536 is a large angle); products and the division are float32.
+    """
     half = rotary_dim // 2
     if half == 0:
         return np.zeros((positions, 0), dtype=np.float32)
     i = np.arange(half, dtype=np.float32)
-    power = np.float32(2.0) * i / np.float32(rotary_dim)
-    freq = np.float32(1.0) / np.power(np.float32(theta), power, dtype=np.float32)
+    exponent = (np.float32(2.0) * i / np.float32(rotary_dim)).astype(np.float32)
+    power = np.power(np.float64(np.float32(theta)), exponent.astype(np.float64)).astype(np.float32)
+    freq = (np.float32(1.0) / power).astype(np.float32)
     pos = np.arange(positions, dtype=np.float32)[:, None]
-    angle = (pos * freq[None, :]).astype(np.float32)
-    return np.concatenate([np.cos(angle, dtype=np.float32), np.sin(angle, dtype=np.float32)], axis=1)
+    angle = (pos * freq[None, :]).astype(np.float32).astype(np.float64)
+    return np.concatenate([np.cos(angle), np.sin(angle)], axis=1).astype(np.float32)
 
 
 class PartialRotary(PositionEncoding):

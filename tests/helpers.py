@@ -26,7 +26,8 @@ TINY_B = dict(vocab_size=320, hidden_size=96, num_hidden_layers=3, num_attention
 INIT_B = RandomInit(seed=1, std=0.05, norm_std=0.1, bias_range=0.1, storage="bfloat16")
 PAGE_B = 8
 
-TINY = {"A": (TINY_A, INIT_A, PAGE_A), "B": (TINY_B, INIT_B, PAGE_B)}
+# "A16": configuration A on pages of 16 tokens, where bfloat16 attention runs on the matrix cores
+TINY = {"A": (TINY_A, INIT_A, PAGE_A), "B": (TINY_B, INIT_B, PAGE_B), "A16": (TINY_A, INIT_A, 16)}
 
 _TMP = tempfile.TemporaryDirectory(prefix="llmx_amd_tests_")
 
@@ -69,6 +70,20 @@ def routing_margin(name: str, tokens, rounded: bool = False) -> float:
         top = torch.sort(keys, dim=-1, descending=True).values
         margin = min(margin, float((top[:, k - 1] - top[:, k]).min()))
     return margin
+
+
+@lru_cache(maxsize=None)
+def row_margins(name: str, length: int, seed: int, rounded: bool):
+    """Per row, the smallest gap over the layers between the last pick's key and the best key left out."""
+    cfg, w = plain(name)
+    _, routing = plain_model.forward(cfg, w, tokens_for(name, length, seed), torch.float64, torch.bfloat16 if rounded else None,
+                                     return_routing=True)
+    k = cfg["num_experts_per_tok"]
+    margins = torch.full((length,), float("inf"), dtype=torch.float64)
+    for _, _, keys in routing:
+        top = torch.sort(keys, dim=-1, descending=True).values
+        margins = torch.minimum(margins, top[:, k - 1] - top[:, k])
+    return margins
 
 
 class RoutingRecorder:

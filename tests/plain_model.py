@@ -48,16 +48,19 @@ def rms_norm(x, weight, eps):
 
 
 def rope_tables(positions, rotary_dim, theta):
-    """cos, sin [len(positions), rotary_dim/2], float32 arithmetic as the reference fills its tables.
+    """cos, sin [len(positions), rotary_dim/2], float32 values in the reference's float32 arithmetic.
 
     src/model/rope.hpp:25-28 (reciprocal_power: 1.0f / powf(theta, 2.0f*i/dim)), :203-210 (cosf((float)pos * freq[i])).
+    powf, cosf and sinf are taken as correctly rounded: evaluated in float64 on their float32 arguments and rounded once.
     """
     half = rotary_dim // 2
     i = torch.arange(half, dtype=torch.float32)
-    freq = 1.0 / torch.pow(torch.tensor(theta, dtype=torch.float32), 2.0 * i / float(rotary_dim))
+    exponent = 2.0 * i / float(rotary_dim)                                             # float32
+    power = torch.pow(torch.tensor(theta, dtype=torch.float32).double(), exponent.double()).float()
+    freq = 1.0 / power                                                                 # float32
     pos = torch.as_tensor(positions, dtype=torch.float32)[:, None]
-    angle = pos * freq[None, :]
-    return torch.cos(angle), torch.sin(angle)
+    angle = (pos * freq[None, :]).double()                                             # the float32 product, widened
+    return torch.cos(angle).float(), torch.sin(angle).float()
 
 
 def apply_partial_rope(x, cos, sin, rotary_dim):

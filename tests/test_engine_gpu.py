@@ -26,7 +26,7 @@ F32_TOL = 2e-5
 # given the engine's picks, after checking that each pick's key is within rounding of the best k.
 BF16_TOL = 2e-2
 
-LENGTHS = {"A": (5, 17, 32, 75), "B": (1, 9, 23, 40, 67)}
+LENGTHS = {"A": (5, 17, 32, 75), "B": (1, 9, 23, 40, 67), "A16": (5, 17, 32, 75)}
 
 
 def make_engine(name, dtype, kv_tokens=1024, max_requests=8):
@@ -40,7 +40,7 @@ def watch(engine, name, dtype):
     return engine
 
 
-@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16")],
+@pytest.fixture(scope="module", params=[("A", "float32"), ("B", "float32"), ("A", "bfloat16"), ("B", "bfloat16"), ("A16", "bfloat16")],
                 ids=lambda p: f"{p[0]}-{p[1]}")
 def setup(request):
     name, dtype = request.param
@@ -89,7 +89,7 @@ def test_whole_alone(setup):
 
 def test_last_32_one_by_one(setup):
     name, dtype, engine = setup
-    length = 75 if name == "A" else 67
+    length = 67 if name == "B" else 75
     tokens = tokens_for(name, length, 0)
     whole = run_whole(engine, "w", tokens)
     cuts = [(0, length - 32)] + [(i, i + 1) for i in range(length - 32, length)]
@@ -101,7 +101,7 @@ def test_last_32_one_by_one(setup):
 
 def test_portions_of_changing_size(setup):
     name, dtype, engine = setup
-    length = 75 if name == "A" else 67
+    length = 67 if name == "B" else 75
     tokens = tokens_for(name, length, 0)
     whole = run_whole(engine, "w", tokens)
     got = run_cut(engine, "p", tokens, portions(length))
