@@ -37,6 +37,7 @@ def parse():
     ap.add_argument("--context", type=int, default=0, help="tokens each sequence holds at the last timed step (0: the configuration's)")
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--only-prefill", action="store_true", help="for profiling: measure the prefill alone and print its record")
     ap.add_argument("--context-fill", choices=["synthetic", "prefill"], default="synthetic",
                     help="how the context before the timed steps gets into the cache: random keys and values written "
                          "directly, or prompts run through the model")
@@ -147,6 +148,30 @@ def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch):
     return dt, distinct
 
 
+def run_prefill(engine, cfg, sampler_out, torch):
+    """One prompt of 2,048 tokens from an empty cache, in one step, to its first sampled token; best of two after a warm-up."""
+    from llmx_amd import ops
+    from llmx_amd.engine import StepEntry
+    T = PREFILL_TOKENS
+    times = []
+    for rep in range(3):   # the first is the warm-up
+        rid = f"p{rep}"
+        engine.add_request(rid)
+        ids = lcg_ids(T, cfg.vocab_size, 500 + rep)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = engine.step([StepEntry(rid, ids, [T - 1])])
+        ops.argmax_rows(logits, sampler_out[:1])
+        sampler_out[:1].tolist()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.end_request(rid)
+    t = min(times[1:])
+    flops = prefill_flops(cfg, T)
+    return {"value": round(T / t, 1), "tokens": T, "ms": round(t * 1e3, 3), "frac": round(flops / t / PEAK_FLOPS["bf16"], 5),
+            "tflop": round(flops / 1e12, 2)}
+
+
 def main():
     a = parse()
     a.warmup = max(1, a.warmup)
@@ -173,6 +198,9 @@ def main():
     setup_s = time.perf_counter() - t_setup
     sampler_out = torch.empty(max_batch, dtype=torch.int32, device=engine.device)
 
+    if a.only_prefill:
+        print(json.dumps({"prefill": run_prefill(engine, cfg, sampler_out, torch)}))
+        return
     dt, distinct = run_decode(engine, sampler_out, a.batch, context, a.steps, a.warmup, a.context_fill, torch)
     ms_per_step = dt / a.steps * 1e3
     value = a.batch * a.steps / dt
@@ -209,24 +237,7 @@ def main():
         result["points"] = pts
 
     if not a.no_prefill:
-        T = PREFILL_TOKENS
-        times = []
-        for rep in range(3):   # the first is the warm-up
-            rid = f"p{rep}"
-            engine.add_request(rid)
-            ids = lcg_ids(T, cfg.vocab_size, 500 + rep)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            logits = engine.step([StepEntry(rid, ids, [T - 1])])
-            ops.argmax_rows(logits, sampler_out[:1])
-            sampler_out[:1].tolist()
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-            engine.end_request(rid)
-        t = min(times[1:])
-        flops = prefill_flops(cfg, T)
-        result["prefill"] = {"value": round(T / t, 1), "tokens": T, "ms": round(t * 1e3, 3),
-                             "frac": round(flops / t / PEAK_FLOPS["bf16"], 5), "tflop": round(flops / 1e12, 2)}
+        result["prefill"] = run_prefill(engine, cfg, sampler_out, torch)
     print(json.dumps(result))
 
 

@@ -24,6 +24,7 @@ struct QkvArgs {
     float eps;
     int n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode;
     int page_tokens, max_blocks, write_kv;
+    int q_slices, k_slices;  // blocks that share a row's q (k) projection: each norms with the whole sum and writes its slice
 };
 
 // Two blocks per row: one norms and rotates q, the other norms and rotates k and writes k and v to the row's page.
@@ -56,16 +57,19 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
     const int p = a.pos[t];
     const float* cs = a.cos_sin + (size_t)p * a.rotary_dim;
     const bool normed = a.norm_mode != QKNORM_NONE;
-    if (blockIdx.y == 0) {
+    if ((int)blockIdx.y < a.q_slices) {
         float r = 1.0f;
         if (a.norm_mode == QKNORM_PROJECTION) {
+            // every block of the row forms the same sum in the same order
             float s = 0.0f;
             for (int i = threadIdx.x; i < qw; i += 256) s = fmaf(row[i], row[i], s);
             s = block_sum<4>(s, scratch);
             r = 1.0f / sqrtf(s / (float)qw + a.eps);
         }
+        const int per = (qw + a.q_slices - 1) / a.q_slices;
+        const int begin = blockIdx.y * per, end = min(qw, begin + per);
         TQ* q_out = (TQ*)a.q_out + (size_t)t * qw;
-        for (int i = threadIdx.x; i < qw; i += 256) st(q_out + i, normed_rotated(row, a.q_weight, cs, i, D, a.rotary_dim, normed, r));
+        for (int i = begin + threadIdx.x; i < end; i += 256) st(q_out + i, normed_rotated(row, a.q_weight, cs, i, D, a.rotary_dim, normed, r));
         return;
     }
     if (!a.write_kv) return;
@@ -82,7 +86,9 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
     const int slot = p % a.page_tokens;
     TKV* kc = (TKV*)a.k_cache;
     TKV* vc = (TKV*)a.v_cache;
-    for (int i = threadIdx.x; i < kw; i += 256) {
+    const int per = (kw + a.k_slices - 1) / a.k_slices;
+    const int begin = ((int)blockIdx.y - a.q_slices) * per, end = min(kw, begin + per);
+    for (int i = begin + threadIdx.x; i < end; i += 256) {
         const int h = i / D, d = i % D;
         const size_t head_at = (size_t)page * a.n_kv_heads + h;
         st(kc + (head_at * a.page_tokens + slot) * D + d, normed_rotated(krow, a.k_weight, cs, i, D, a.rotary_dim, normed, r));
@@ -96,9 +102,18 @@ extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight,
                                         int page_tokens, int max_blocks, int write_kv, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (norm_mode != QKNORM_NONE && norm_mode != QKNORM_PROJECTION) return -2;
+    // few rows: many blocks a row, so the chip is used; many rows: two blocks a row, so the sum is not formed over and over
+    const int qw = n_heads * head_dim, kw = n_kv_heads * head_dim;
+    int q_slices = 1, k_slices = 1;
+    if (rows <= 256) {
+        q_slices = (qw + 255) / 256;
+        k_slices = (kw + 255) / 256;
+        if (q_slices > 16) q_slices = 16;
+        if (k_slices > 4) k_slices = 4;
+    }
     QkvArgs a{qkv, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
-              n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv};
-    const dim3 grid(rows, 2);
+              n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, q_slices, k_slices};
+    const dim3 grid(rows, q_slices + k_slices);
     if (dtype == LLMX_F32)
         hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<float, float>), grid, dim3(256), 0, stream, a);
     else

@@ -80,49 +80,69 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
     for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
     float m = -INFINITY, l = 0.0f;
 
-    for (int j0 = key_begin; j0 < key_end; j0 += 32) {
-        // the two 16-key tiles of the step: where their pages are
+    // Software pipeline: while step i is multiplied, the keys of step i+1 and the page ids of step i+2 are on their way.
+    struct Where {
         size_t k_at[2], v_at[2];
-        bool tile_in[2];
+        bool in[2];
+    };
+    auto locate = [&](int j0, int page0, int page1) {
+        Where w;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int key0 = j0 + 16 * u;
-            tile_in[u] = key0 < key_end;
-            int page = tile_in[u] ? table[key0 / bt] : -1;
-            if (page < 0) tile_in[u] = false;
+            const int page = u == 0 ? page0 : page1;
+            w.in[u] = key0 < key_end && page >= 0;
             const int sub = key0 % bt;
             const size_t head_at = (size_t)(page < 0 ? 0 : page) * Hkv + kvh;
-            k_at[u] = (head_at * bt + sub) * D;
-            v_at[u] = head_at * D * bt + sub;
+            w.k_at[u] = (head_at * bt + sub) * D;
+            w.v_at[u] = head_at * D * bt + sub;
         }
-        // scores^T: lane holds keys 4g + i of each tile for its column
-        f32x4_t s_acc[2];
+        return w;
+    };
+    auto page_of = [&](int key0) { return key0 < key_end ? table[key0 / bt] : -1; };
+    auto load_keys = [&](const Where& w, bf16x8_t (&kf)[2][QS]) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            s_acc[u] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-            bf16x8_t kf[QS];
+        for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int s = 0; s < QS; ++s) {
                 u32x4_t v = {0u, 0u, 0u, 0u};
                 const int d = 32 * s + 8 * g;
-                if (tile_in[u] && d < D) v = *reinterpret_cast<const u32x4_t*>(a.k_cache + k_at[u] + (size_t)c * D + d);
-                kf[s] = __builtin_bit_cast(bf16x8_t, v);
+                if (w.in[u] && d < D) v = *reinterpret_cast<const u32x4_t*>(a.k_cache + w.k_at[u] + (size_t)c * D + d);
+                kf[u][s] = __builtin_bit_cast(bf16x8_t, v);
             }
-#pragma unroll
-            for (int s = 0; s < QS; ++s) s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s], qf[s], s_acc[u], 0, 0, 0);
-        }
-        // V^T fragments: lane (dim 16dt + c, keys 4g .. 4g+3 of each tile); loaded before the softmax so they are in flight
+    };
+    bf16x8_t kf[2][QS], kf_next[2][QS];
+    Where here = locate(key_begin, page_of(key_begin), page_of(key_begin + 16));
+    load_keys(here, kf);
+    int page_next0 = page_of(key_begin + 32), page_next1 = page_of(key_begin + 48);
+
+    for (int j0 = key_begin; j0 < key_end; j0 += 32) {
+        // V^T fragments of this step: lane (dim 16dt + c, keys 4g .. 4g+3 of each tile)
         bf16x8_t vf[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             u32x2_t v0 = {0u, 0u}, v1 = {0u, 0u};
             const int d = 16 * dt + c;
             if (d < D) {
-                if (tile_in[0]) v0 = *reinterpret_cast<const u32x2_t*>(a.v_cache + v_at[0] + (size_t)d * bt + 4 * g);
-                if (tile_in[1]) v1 = *reinterpret_cast<const u32x2_t*>(a.v_cache + v_at[1] + (size_t)d * bt + 4 * g);
+                if (here.in[0]) v0 = *reinterpret_cast<const u32x2_t*>(a.v_cache + here.v_at[0] + (size_t)d * bt + 4 * g);
+                if (here.in[1]) v1 = *reinterpret_cast<const u32x2_t*>(a.v_cache + here.v_at[1] + (size_t)d * bt + 4 * g);
             }
             const u32x4_t v = {v0[0], v0[1], v1[0], v1[1]};
             vf[dt] = __builtin_bit_cast(bf16x8_t, v);
+        }
+        // the next step's keys, and the page ids of the step after it
+        const Where next = locate(j0 + 32, page_next0, page_next1);
+        if (j0 + 32 < key_end) load_keys(next, kf_next);
+        page_next0 = page_of(j0 + 64);
+        page_next1 = page_of(j0 + 80);
+
+        // scores^T: lane holds keys 4g + i of each tile for its column
+        f32x4_t s_acc[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s_acc[u] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s = 0; s < QS; ++s) s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][s], qf[s], s_acc[u], 0, 0, 0);
         }
         // online softmax of the column over the step's 32 keys
         float sc[8];
@@ -132,7 +152,7 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int key = j0 + 16 * u + 4 * g + i;
-                const bool ok = tile_in[u] && col_ok && key <= p_col && key >= lo_col && key < key_end;
+                const bool ok = here.in[u] && col_ok && key <= p_col && key >= lo_col && key < key_end;
                 const float v = ok ? s_acc[u][i] * a.scale : -INFINITY;
                 sc[4 * u + i] = v;
                 step_max = fmaxf(step_max, v);
@@ -160,6 +180,11 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
             o[dt] = f32x4_t{o[dt][0] * alpha, o[dt][1] * alpha, o[dt][2] * alpha, o[dt][3] * alpha};
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
         }
+        here = next;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int s = 0; s < QS; ++s) kf[u][s] = kf_next[u][s];
     }
     if (!col_ok) return;
     // lane holds dims 16dt + 4g + i of its column
@@ -191,26 +216,43 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
 }
 
 // merge: one block per output (row, head).  merge item: {row, head, first_slot, n_splits, column}
-__global__ void attention_merge_kernel(const int* __restrict__ merges, const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                       bf16_t* __restrict__ out, int n_heads, int D) {
+// The splits' weights exp(m_s - max) are formed once in LDS; the sum of weights * sums runs in split order; every
+// thread then adds its dims over the splits in split order, eight loads in flight at a time.
+#define AM_MAX_SPLITS 512
+__global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restrict__ merges, const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_ml, bf16_t* __restrict__ out, int n_heads, int D) {
+    __shared__ float weight[AM_MAX_SPLITS];
+    __shared__ float sums[AM_MAX_SPLITS];
     const int* mi = merges + (size_t)blockIdx.x * AM_ITEM_INTS;
     const int t = mi[0], h = mi[1], first = mi[2], n = mi[3], c = mi[4];
-    float mx = -INFINITY;
-    for (int s = 0; s < n; ++s) mx = fmaxf(mx, part_ml[((size_t)(first + s) * 16 + c) * 2]);
-    float total = 0.0f;
-    for (int s = 0; s < n; ++s) {
+    for (int s = threadIdx.x; s < n; s += 128) {
         const size_t at = (size_t)(first + s) * 16 + c;
-        const float ms = part_ml[at * 2];
-        total += (ms == -INFINITY ? 0.0f : __expf(ms - mx)) * part_ml[at * 2 + 1];
+        weight[s] = part_ml[at * 2];        // the split's running max for now
+        sums[s] = part_ml[at * 2 + 1];
     }
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    __syncthreads();
+    float mx = -INFINITY;
+    for (int s = 0; s < n; ++s) mx = fmaxf(mx, weight[s]);
+    __syncthreads();
+    for (int s = threadIdx.x; s < n; s += 128) weight[s] = weight[s] == -INFINITY ? 0.0f : __expf(weight[s] - mx);
+    __syncthreads();
+    float total = 0.0f;
+    for (int s = 0; s < n; ++s) total += weight[s] * sums[s];
+    const float inv = 1.0f / total;
+    const float* base = part_o + ((size_t)first * 16 + c) * D;
+    const size_t stride = (size_t)16 * D;
+    for (int d = threadIdx.x; d < D; d += 128) {
         float acc = 0.0f;
-        for (int s = 0; s < n; ++s) {
-            const size_t at = (size_t)(first + s) * 16 + c;
-            const float ms = part_ml[at * 2];
-            acc += (ms == -INFINITY ? 0.0f : __expf(ms - mx)) * part_o[at * D + d];
+        int s = 0;
+        for (; s + 8 <= n; s += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = base[(size_t)(s + u) * stride + d];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += weight[s + u] * v[u];
         }
-        out[((size_t)t * n_heads + h) * D + d] = f32_to_bf16(acc / total);
+        for (; s < n; ++s) acc += weight[s] * base[(size_t)s * stride + d];
+        out[((size_t)t * n_heads + h) * D + d] = f32_to_bf16(acc * inv);
     }
 }
 

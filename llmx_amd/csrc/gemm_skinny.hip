@@ -40,9 +40,7 @@ __device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p, bool in) {
     return __builtin_bit_cast(bf16x8_t, v);
 }
 
-#define SK_UNROLL 4
-
-template <int KS, int MT, int EPI, typename TC, bool GROUPED>
+template <int KS, int MT, int EPI, typename TC, bool GROUPED, int SK_UNROLL>
 __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
     constexpr int NACC = (EPI == SK_SWIGLU) ? 2 : 1;
     __shared__ float red[KS > 1 ? KS : 1][MT * NACC][256];
@@ -171,9 +169,9 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
 template <int KS, int MT, int EPI, typename TC>
 static void launch_grouped(const SkinnyArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
     if (grouped)
-        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true>), grid, dim3(64 * KS), 0, stream, g);
+        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true, (MT == 1 && EPI != SK_SWIGLU) ? 8 : 4>), grid, dim3(64 * KS), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false>), grid, dim3(64 * KS), 0, stream, g);
+        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false, (MT == 1 && EPI != SK_SWIGLU) ? 8 : 4>), grid, dim3(64 * KS), 0, stream, g);
 }
 
 template <int KS, int MT>

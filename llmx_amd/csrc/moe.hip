@@ -185,3 +185,120 @@ extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* c
     hipLaunchKernelGGL(moe_place_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
     return LLMX_CHECK_LAUNCH();
 }
+
+// ---------------------------------------------------------------------------
+// A decode step's routing in one launch: top-k of every row (one wave a row, values in registers: at most 256 experts,
+// at most 64 picks), then the pairs grouped by expert as moe_align_small_kernel does.  Same formulas and the same
+// orders as route_topk_kernel, so the picks and weights are the same bits.
+__global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __restrict__ z, const float* __restrict__ bias,
+                                                               int* __restrict__ ids, float* __restrict__ weights, int rows, int n_experts,
+                                                               int k, int normalize, float scale, int* __restrict__ counts,
+                                                               int* __restrict__ offsets, int* __restrict__ list, int* __restrict__ active,
+                                                               int* __restrict__ n_active) {
+    __shared__ int pair_expert[ALIGN_SMALL_PAIRS];
+    __shared__ int cnt[1024];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    for (int r = wave; r < rows; r += 16) {
+        const float* row = z + (size_t)r * n_experts;
+        float s[4], b[4];
+        bool taken[4];
+        int finite = 1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = lane + 64 * i;
+            s[i] = 0.0f;
+            b[i] = -INFINITY;
+            taken[i] = true;
+            if (e < n_experts) {
+                s[i] = 1.0f / (1.0f + expf(-row[e]));
+                b[i] = bias ? s[i] + bias[e] : s[i];
+                taken[i] = false;
+                if (!isfinite(b[i])) finite = 0;
+            }
+        }
+        finite = __all(finite);
+        if (!finite) {
+            if (lane < k) {
+                ids[(size_t)r * k + lane] = -1;
+                weights[(size_t)r * k + lane] = 0.0f;
+                pair_expert[r * k + lane] = -1;
+            }
+            continue;
+        }
+        float mine = 0.0f;
+        int mine_id = -1;
+        for (int j = 0; j < k; ++j) {
+            float best = -INFINITY;
+            int at = 0x7fffffff;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (!taken[i] && b[i] > best) {
+                    best = b[i];
+                    at = lane + 64 * i;
+                }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ob = __shfl_xor(best, o, 64);
+                const int oa = __shfl_xor(at, o, 64);
+                if (ob > best || (ob == best && oa < at)) {
+                    best = ob;
+                    at = oa;
+                }
+            }
+            const int slot = at >> 6;
+            const float picked = slot == 0 ? s[0] : slot == 1 ? s[1] : slot == 2 ? s[2] : s[3];
+            const float score = __shfl(picked, at & 63, 64);
+            if (lane == (at & 63)) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (i == slot) taken[i] = true;
+            }
+            if (lane == j) {
+                mine = score;
+                mine_id = at;
+            }
+        }
+        float total = 0.0f;
+        for (int j = 0; j < k; ++j) total += __shfl(mine, j, 64);
+        if (lane < k) {
+            ids[(size_t)r * k + lane] = mine_id;
+            weights[(size_t)r * k + lane] = (normalize ? mine / total : mine) * scale;
+            pair_expert[r * k + lane] = mine_id;
+        }
+    }
+    __syncthreads();
+    const int n_pairs = rows * k;
+    const int e = tid;
+    int c = 0;
+    if (e < n_experts)
+        for (int p = 0; p < n_pairs; ++p) c += pair_expert[p] == e;
+    cnt[e] = c;
+    __syncthreads();
+    if (e >= n_experts) return;
+    int before = 0, active_before = 0;
+    for (int i = 0; i < e; ++i) {
+        before += cnt[i];
+        active_before += cnt[i] > 0;
+    }
+    counts[e] = c;
+    offsets[e] = before;
+    if (c > 0) active[active_before] = e;
+    if (e == n_experts - 1) {
+        offsets[n_experts] = before + c;
+        n_active[0] = active_before + (c > 0);
+    }
+    int at = before;
+    for (int p = 0; p < n_pairs && c > 0; ++p)
+        if (pair_expert[p] == e) list[at++] = p;
+}
+
+// Sigmoid scores only; rows * k <= 1024, at most 256 experts, at most 64 picks.  Returns -2 otherwise.
+extern "C" int llmx_route_topk_align(const float* z, const float* bias, int* ids, float* weights, int rows, int n_experts, int k,
+                                     int normalize, float scale, int* counts, int* offsets, int* list, int* active, int* n_active,
+                                     hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (rows * k > ALIGN_SMALL_PAIRS || n_experts > 256 || k > 64 || k > n_experts || k <= 0) return -2;
+    hipLaunchKernelGGL(route_topk_align_kernel, dim3(1), dim3(1024), 0, stream, z, bias, ids, weights, rows, n_experts, k, normalize, scale,
+                       counts, offsets, list, active, n_active);
+    return LLMX_CHECK_LAUNCH();
+}

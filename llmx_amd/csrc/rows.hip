@@ -21,23 +21,24 @@ extern "C" int llmx_embed_gather(const void* table, int table_dtype, const int* 
 }
 
 // ---------------------------------------------------------------------------
-// RMSNorm of f32 rows: s = sum x^2 (strided per thread, butterfly per wave, waves in order),
+// RMSNorm of f32 rows, one block of 1024 threads a row: s = sum x^2 (strided per thread, butterfly per wave, waves in order),
 // r = 1/sqrt(s/n + eps), y = x * (r * w).  Optional row gather on the input (the head reads only wanted rows).
 // Writes the result in the activation type and/or as f32 (the router reads unrounded rows).
+#define RMS_THREADS 1024
 template <typename TO>
-__global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ pick, const float* __restrict__ w,
-                                                    float eps, TO* __restrict__ out, float* __restrict__ out32, int n) {
-    __shared__ float scratch[4];
+__global__ void __launch_bounds__(RMS_THREADS) rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ pick, const float* __restrict__ w,
+                                                            float eps, TO* __restrict__ out, float* __restrict__ out32, int n) {
+    __shared__ float scratch[RMS_THREADS / 64];
     const int r = blockIdx.x;
     const float* row = x + (size_t)(pick ? pick[r] : r) * n;
     float s = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) {
+    for (int i = threadIdx.x; i < n; i += RMS_THREADS) {
         const float v = row[i];
         s = fmaf(v, v, s);
     }
-    s = block_sum<4>(s, scratch);
+    s = block_sum<RMS_THREADS / 64>(s, scratch);
     const float scale = 1.0f / sqrtf(s / (float)n + eps);
-    for (int i = threadIdx.x; i < n; i += 256) {
+    for (int i = threadIdx.x; i < n; i += RMS_THREADS) {
         const float y = row[i] * (scale * w[i]);
         if (out) st(out + (size_t)r * n + i, y);
         if (out32) out32[(size_t)r * n + i] = y;
@@ -48,9 +49,9 @@ extern "C" int llmx_rmsnorm(const float* x, const int* pick, const float* w, flo
                             int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (out_dtype == LLMX_F32)
-        hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(rows), dim3(256), 0, stream, x, pick, w, eps, (float*)out, out32, n);
+        hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (float*)out, out32, n);
     else
-        hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, x, pick, w, eps, (bf16_t*)out, out32, n);
+        hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (bf16_t*)out, out32, n);
     return LLMX_CHECK_LAUNCH();
 }
 

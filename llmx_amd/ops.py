@@ -62,6 +62,7 @@ def _declare(h) -> None:
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, P, P, I, I, I, I, I, F, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P],
+        "llmx_route_topk_align": [P, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
         "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
         "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, P],
@@ -137,11 +138,16 @@ SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream 
 SKINNY_MAX_GROUPED_ROWS = 128  # routed products of at most this many token rows do
 
 
+_KS_OVERRIDE = None   # set by tuning scripts only
+
+
 def _split_k(n_strips: int, K: int) -> int:
-    """Waves that share one 16-feature strip's K: enough strips*waves to fill the chip, at least 4 k-steps a wave.
+    """Waves that share one 16-feature strip's K: enough strips*waves to fill the chip, at least 12 k-steps a wave.
     A function of the product's shape only, so a row's bits do not depend on the batch."""
+    if _KS_OVERRIDE:
+        return _KS_OVERRIDE
     ks = 1
-    while ks < 8 and n_strips * ks < 2048 and (K // 32) // (ks * 2) >= 4:
+    while ks < 8 and n_strips * ks < 2048 and (K // 32) // (ks * 2) >= 12:
         ks *= 2
     return ks
 
@@ -247,8 +253,8 @@ class AttentionPlan:
 
 
 _PLAN_CACHE: dict = {}
-ATTENTION_TARGET_WAVES = 1024   # work items wanted before long contexts stop being split further
-ATTENTION_MIN_SPLIT_KEYS = 256  # a split covers at least this many keys
+ATTENTION_TARGET_WAVES = 2048   # work items wanted before long contexts stop being split further
+ATTENTION_MIN_SPLIT_KEYS = 128  # a split covers at least this many keys
 
 
 def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device) -> AttentionPlan:
@@ -262,7 +268,7 @@ def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device) 
     if single:
         base = len(single) * len(head_chunks)
         longest = max(contexts[i] for i in single)
-        n_splits = max(1, min(-(-ATTENTION_TARGET_WAVES // base), longest // ATTENTION_MIN_SPLIT_KEYS))
+        n_splits = max(1, min(-(-ATTENTION_TARGET_WAVES // base), longest // ATTENTION_MIN_SPLIT_KEYS, 512))
     key = (tuple(row_counts), n_heads, n_kv_heads, n_splits, str(device))
     plan = _PLAN_CACHE.get(key)
     if plan is not None:
@@ -349,6 +355,24 @@ def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: 
                                 _dev(offsets, "offsets", torch.int32, (n_experts + 1,)), _dev(pairs, "pairs", torch.int32, (n_pairs,)),
                                 _dev(active, "active", torch.int32, (n_experts,)), _dev(n_active, "n_active", torch.int32, (1,)),
                                 _stream()), "moe_align")
+
+
+def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
+                     normalize: bool, scale: float, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
+                     active: torch.Tensor, n_active: torch.Tensor) -> None:
+    """route_topk followed by moe_align; a step of few rows (rows * k <= 1024, sigmoid scores, at most 256 experts and 64
+    picks) does both in one launch, with the same bits."""
+    rows, n_experts = z.shape
+    if score == SCORE_SIGMOID and rows * k <= 1024 and n_experts <= 256 and k <= 64:
+        _check(lib().llmx_route_topk_align(
+            _dev(z, "z", torch.float32), _dev(bias, "bias", torch.float32, (n_experts,)), _dev(ids, "ids", torch.int32, (rows, k)),
+            _dev(weights, "weights", torch.float32, (rows, k)), rows, n_experts, k, 1 if normalize else 0, float(scale),
+            _dev(counts, "counts", torch.int32, (n_experts,)), _dev(offsets, "offsets", torch.int32, (n_experts + 1,)),
+            _dev(pairs, "pairs", torch.int32, (rows * k,)), _dev(active, "active", torch.int32, (n_experts,)),
+            _dev(n_active, "n_active", torch.int32, (1,)), _stream()), "route_topk_align")
+        return
+    route_topk(z, bias, ids, weights, k, score, normalize, scale)
+    moe_align(ids, n_experts, counts, offsets, pairs, active, n_active)
 
 
 def moe_combine(x: torch.Tensor, y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, accumulate: bool = True) -> None:

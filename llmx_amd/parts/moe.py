@@ -76,25 +76,19 @@ class RoutedExperts(FeedForward):
             self.w_gate_up = tensors[self.name("experts.gate_up_proj")]
             self.w_down = tensors[self.name("experts.down_proj")]
 
-    def route(self, step, h32):
+    def forward(self, step, h, out, accumulate, h32=None):
         T, X, k = step.rows, self.experts, self.top_k
         z = step.buf("experts.router_logits", (T, X), torch.float32)
         ops.gemm_f32(h32, self.w_router, z)
         ids = step.buf("experts.ids", (T, k), torch.int32)
         weights = step.buf("experts.weights", (T, k), torch.float32)
-        ops.route_topk(z, self.bias, ids, weights, k, self.score, self.normalize, self.scale)
-        step.observe("routing", logits=z, ids=ids, weights=weights)
-        return ids, weights
-
-    def forward(self, step, h, out, accumulate, h32=None):
-        T, X, k = step.rows, self.experts, self.top_k
-        ids, weights = self.route(step, h32)
         counts = step.buf("experts.counts", (X,), torch.int32)
         offsets = step.buf("experts.offsets", (X + 1,), torch.int32)
         pairs = step.buf("experts.pairs", (T * k,), torch.int32)
         active = step.buf("experts.active", (X,), torch.int32)
         n_active = step.buf("experts.n_active", (1,), torch.int32)
-        ops.moe_align(ids, X, counts, offsets, pairs, active, n_active)
+        ops.route_topk_align(z, self.bias, ids, weights, k, self.score, self.normalize, self.scale, counts, offsets, pairs, active, n_active)
+        step.observe("routing", logits=z, ids=ids, weights=weights)
         act = step.buf("experts.act", (T * k, self.intermediate), step.act_dtype)
         ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T)
         y = step.buf("experts.y", (T * k, self.hidden), torch.float32)

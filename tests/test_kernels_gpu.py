@@ -415,6 +415,33 @@ def test_route_topk_vectors():
                 assert torch.equal(ids1[0], ids[6]) and torch.equal(w1[0], w[6])
 
 
+@pytest.mark.parametrize("T,X,k", [(1, 8, 2), (8, 256, 8), (64, 256, 8), (13, 100, 7), (5, 16, 16), (40, 24, 24)])
+def test_fused_route_and_align_equals_the_two_kernels(T, X, k):
+    o = ops()
+    z = rnd(T, X, scale=1.5, seed=T)
+    if T > 2:
+        z[1, 3] = z[1, 0]                 # a tie
+        z[2, 1] = float("nan")            # a row without experts
+    bias = 0.2 * rnd(X, seed=2)
+    mk = lambda shape, dt: torch.full(shape, -9, dtype=dt, device=DEV)
+    for normalize in (True, False):
+        outs = []
+        for fused in (True, False):
+            ids, w = mk((T, k), torch.int32), mk((T, k), torch.float32)
+            counts, offsets, pairs = mk((X,), torch.int32), mk((X + 1,), torch.int32), mk((T * k,), torch.int32)
+            active, n_active = mk((X,), torch.int32), mk((1,), torch.int32)
+            if fused:
+                o.route_topk_align(z, bias, ids, w, k, o.SCORE_SIGMOID, normalize, 2.5, counts, offsets, pairs, active, n_active)
+            else:
+                o.route_topk(z, bias, ids, w, k, o.SCORE_SIGMOID, normalize, 2.5)
+                o.moe_align(ids, X, counts, offsets, pairs, active, n_active)
+            n = int(n_active)
+            valid = int(offsets[X])
+            outs.append((ids, w, counts, offsets, pairs[:valid], active[:n], n_active))
+        for a, b in zip(*outs):
+            assert torch.equal(a, b)
+
+
 def test_route_matches_plain_and_invariants():
     o = ops()
     T, X, k = 13, 40, 5
