@@ -88,7 +88,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
     }
 }
 
-// K a multiple of 4, rows 16-byte aligned.  ks: 1, 2, 4 or 8.
+// K a multiple of 4, rows 16-byte aligned.  ks: 1, 2, 4, 8 or 16.
 extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, int M, int N, int K, int lda, int ldc, int add, int ks,
                                     hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
@@ -104,6 +104,7 @@ extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, in
         case 2: SKF_MT(2); break;
         case 4: SKF_MT(4); break;
         case 8: SKF_MT(8); break;
+        case 16: SKF_MT(16); break;
         default: return -2;
     }
 #undef SKF_MT

@@ -98,13 +98,16 @@ extern "C" int llmx_route_topk(const float* z, const float* bias, int* ids, floa
 // ---------------------------------------------------------------------------
 // The pairs p = t*k + j of a step grouped by expert, each expert's pairs in increasing p (stable), without atomics:
 // pass 1 counts each expert's pairs, pass 2 derives each expert's offset from the counts and places its pairs.
-__global__ void __launch_bounds__(64) moe_count_kernel(const int* __restrict__ ids, int n_pairs, int* __restrict__ counts) {
-    const int e = blockIdx.x, lane = threadIdx.x;
+__global__ void __launch_bounds__(256) moe_count_kernel(const int* __restrict__ ids, int n_pairs, int* __restrict__ counts) {
+    __shared__ int part[4];
+    const int e = blockIdx.x, lane = threadIdx.x & 63;
     int c = 0;
-    for (int p = lane; p < n_pairs; p += 64) c += ids[p] == e;
+    for (int p = threadIdx.x; p < n_pairs; p += 256) c += ids[p] == e;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
-    if (lane == 0) counts[e] = c;
+    if (lane == 0) part[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) counts[e] = part[0] + part[1] + part[2] + part[3];
 }
 
 __global__ void __launch_bounds__(64) moe_place_kernel(const int* __restrict__ ids, int n_pairs, int n_experts, const int* __restrict__ counts,
@@ -129,48 +132,82 @@ __global__ void __launch_bounds__(64) moe_place_kernel(const int* __restrict__ i
             n_active[0] = active_before + (counts[e] > 0);
         }
     }
+    if (counts[e] == 0) return;
     int at = before;
-    for (int p0 = 0; p0 < n_pairs; p0 += 64) {
-        const int p = p0 + lane;
-        const bool mine = p < n_pairs && ids[p] == e;
-        const unsigned long long mask = __ballot(mine);
-        if (mine) list[at + __popcll(mask & ((1ull << lane) - 1ull))] = p;
-        at += __popcll(mask);
+    for (int p0 = 0; p0 < n_pairs; p0 += 256) {
+        // four loads in flight: pairs p0 + 64*i + lane, placed in pair order
+        int id[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int p = p0 + 64 * i + lane;
+            id[i] = p < n_pairs ? ids[p] : -2;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool mine = id[i] == e;
+            const unsigned long long mask = __ballot(mine);
+            if (mine) list[at + __popcll(mask & ((1ull << lane) - 1ull))] = p0 + 64 * i + lane;
+            at += __popcll(mask);
+        }
     }
 }
 
-// Few pairs (a decode step): one workgroup does it all.  Thread e owns expert e: it counts its pairs, the counts are
-// scanned in expert order, and it places its pairs in increasing pair order.
+// Few pairs (a decode step): one workgroup of 16 waves does it all.  The pairs' experts sit in LDS; wave w owns experts
+// w, w+16, ...: it counts an expert's pairs with ballots over the pairs 64 at a time, the counts are scanned in expert
+// order, and the same ballots place the expert's pairs in increasing pair order.
 #define ALIGN_SMALL_PAIRS 1024
+__device__ void align_in_block(const int* pair_expert, int n_pairs, int n_experts, int* cnt, int* offs, int* __restrict__ counts,
+                               int* __restrict__ offsets, int* __restrict__ list, int* __restrict__ active, int* __restrict__ n_active) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    for (int e = wave; e < n_experts; e += 16) {
+        int c = 0;
+        for (int p0 = 0; p0 < n_pairs; p0 += 64) {
+            const int p = p0 + lane;
+            c += __popcll(__ballot(p < n_pairs && pair_expert[p] == e));
+        }
+        if (lane == 0) cnt[e] = c;
+    }
+    __syncthreads();
+    if (tid < n_experts) {
+        const int e = tid;
+        int before = 0, active_before = 0;
+        for (int i = 0; i < e; ++i) {
+            before += cnt[i];
+            active_before += cnt[i] > 0;
+        }
+        const int c = cnt[e];
+        offs[e] = before;
+        counts[e] = c;
+        offsets[e] = before;
+        if (c > 0) active[active_before] = e;
+        if (e == n_experts - 1) {
+            offsets[n_experts] = before + c;
+            n_active[0] = active_before + (c > 0);
+        }
+    }
+    __syncthreads();
+    for (int e = wave; e < n_experts; e += 16) {
+        if (cnt[e] == 0) continue;
+        int at = offs[e];
+        for (int p0 = 0; p0 < n_pairs; p0 += 64) {
+            const int p = p0 + lane;
+            const bool mine = p < n_pairs && pair_expert[p] == e;
+            const unsigned long long mask = __ballot(mine);
+            if (mine) list[at + __popcll(mask & ((1ull << lane) - 1ull))] = p;
+            at += __popcll(mask);
+        }
+    }
+}
+
 __global__ void __launch_bounds__(1024) moe_align_small_kernel(const int* __restrict__ ids, int n_pairs, int n_experts, int* __restrict__ counts,
                                                               int* __restrict__ offsets, int* __restrict__ list, int* __restrict__ active,
                                                               int* __restrict__ n_active) {
     __shared__ int pair_expert[ALIGN_SMALL_PAIRS];
     __shared__ int cnt[1024];
-    const int e = threadIdx.x;
-    for (int p = e; p < n_pairs; p += 1024) pair_expert[p] = ids[p];
+    __shared__ int offs[1024];
+    for (int p = threadIdx.x; p < n_pairs; p += 1024) pair_expert[p] = ids[p];
     __syncthreads();
-    int c = 0;
-    if (e < n_experts)
-        for (int p = 0; p < n_pairs; ++p) c += pair_expert[p] == e;
-    cnt[e] = c;
-    __syncthreads();
-    if (e >= n_experts) return;
-    int before = 0, active_before = 0;
-    for (int i = 0; i < e; ++i) {
-        before += cnt[i];
-        active_before += cnt[i] > 0;
-    }
-    counts[e] = c;
-    offsets[e] = before;
-    if (c > 0) active[active_before] = e;
-    if (e == n_experts - 1) {
-        offsets[n_experts] = before + c;
-        n_active[0] = active_before + (c > 0);
-    }
-    int at = before;
-    for (int p = 0; p < n_pairs && c > 0; ++p)
-        if (pair_expert[p] == e) list[at++] = p;
+    align_in_block(pair_expert, n_pairs, n_experts, cnt, offs, counts, offsets, list, active, n_active);
 }
 
 // counts [X], offsets [X+1], list [n_pairs], active [X], n_active [1]
@@ -181,7 +218,7 @@ extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* c
         hipLaunchKernelGGL(moe_align_small_kernel, dim3(1), dim3(1024), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
         return LLMX_CHECK_LAUNCH();
     }
-    hipLaunchKernelGGL(moe_count_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, counts);
+    hipLaunchKernelGGL(moe_count_kernel, dim3(n_experts), dim3(256), 0, stream, ids, n_pairs, counts);
     hipLaunchKernelGGL(moe_place_kernel, dim3(n_experts), dim3(64), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
     return LLMX_CHECK_LAUNCH();
 }
@@ -197,6 +234,7 @@ __global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __r
                                                                int* __restrict__ n_active) {
     __shared__ int pair_expert[ALIGN_SMALL_PAIRS];
     __shared__ int cnt[1024];
+    __shared__ int offs[1024];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     for (int r = wave; r < rows; r += 16) {
         const float* row = z + (size_t)r * n_experts;
@@ -267,37 +305,15 @@ __global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __r
         }
     }
     __syncthreads();
-    const int n_pairs = rows * k;
-    const int e = tid;
-    int c = 0;
-    if (e < n_experts)
-        for (int p = 0; p < n_pairs; ++p) c += pair_expert[p] == e;
-    cnt[e] = c;
-    __syncthreads();
-    if (e >= n_experts) return;
-    int before = 0, active_before = 0;
-    for (int i = 0; i < e; ++i) {
-        before += cnt[i];
-        active_before += cnt[i] > 0;
-    }
-    counts[e] = c;
-    offsets[e] = before;
-    if (c > 0) active[active_before] = e;
-    if (e == n_experts - 1) {
-        offsets[n_experts] = before + c;
-        n_active[0] = active_before + (c > 0);
-    }
-    int at = before;
-    for (int p = 0; p < n_pairs && c > 0; ++p)
-        if (pair_expert[p] == e) list[at++] = p;
+    align_in_block(pair_expert, rows * k, n_experts, cnt, offs, counts, offsets, list, active, n_active);
 }
 
-// Sigmoid scores only; rows * k <= 1024, at most 256 experts, at most 64 picks.  Returns -2 otherwise.
+// Sigmoid scores only; at most 16 rows (a wave each), rows * k <= 1024, at most 256 experts and 64 picks.  Returns -2 otherwise.
 extern "C" int llmx_route_topk_align(const float* z, const float* bias, int* ids, float* weights, int rows, int n_experts, int k,
                                      int normalize, float scale, int* counts, int* offsets, int* list, int* active, int* n_active,
                                      hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (rows * k > ALIGN_SMALL_PAIRS || n_experts > 256 || k > 64 || k > n_experts || k <= 0) return -2;
+    if (rows > 16 || rows * k > ALIGN_SMALL_PAIRS || n_experts > 256 || k > 64 || k > n_experts || k <= 0) return -2;
     hipLaunchKernelGGL(route_topk_align_kernel, dim3(1), dim3(1024), 0, stream, z, bias, ids, weights, rows, n_experts, k, normalize, scale,
                        counts, offsets, list, active, n_active);
     return LLMX_CHECK_LAUNCH();

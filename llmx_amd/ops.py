@@ -360,10 +360,10 @@ def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: 
 def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
                      normalize: bool, scale: float, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
                      active: torch.Tensor, n_active: torch.Tensor) -> None:
-    """route_topk followed by moe_align; a step of few rows (rows * k <= 1024, sigmoid scores, at most 256 experts and 64
-    picks) does both in one launch, with the same bits."""
+    """route_topk followed by moe_align; a step of at most 16 rows (sigmoid scores, at most 256 experts and 64 picks) does
+    both in one launch, with the same bits."""
     rows, n_experts = z.shape
-    if score == SCORE_SIGMOID and rows * k <= 1024 and n_experts <= 256 and k <= 64:
+    if score == SCORE_SIGMOID and rows <= 16 and rows * k <= 1024 and n_experts <= 256 and k <= 64:
         _check(lib().llmx_route_topk_align(
             _dev(z, "z", torch.float32), _dev(bias, "bias", torch.float32, (n_experts,)), _dev(ids, "ids", torch.int32, (rows, k)),
             _dev(weights, "weights", torch.float32, (rows, k)), rows, n_experts, k, 1 if normalize else 0, float(scale),
@@ -425,7 +425,7 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, add: bool = Fals
         return
     ks = 1
     n_strips = -(-N // 16)
-    while ks < 8 and n_strips * ks < 1024 and (K // 16) // (ks * 2) >= 8:
+    while ks < 16 and n_strips * ks < 1024 and (K // 16) // (ks * 2) >= 8:   # from w's shape only: a row's bits must not depend on M
         ks *= 2
     _check(lib().llmx_gemm_skinny_f32(_dev(a, "a", torch.float32), _dev(w, "w", torch.float32), _dev(c, "c", torch.float32), M, N, K, K, N,
                                       1 if add else 0, ks, _stream()), "gemm_f32")

@@ -212,3 +212,54 @@ def test_refusals_leave_nothing_behind(setup):
         engine.step([])
     assert engine.cache.pages_in_use() == before and engine.length("r") == 0
     engine.end_request("r")
+
+
+# ---------------------------------------------------------------------------
+# One layer at the real layer widths (hidden 3072, 48 query / 8 KV heads of 128, rotary 64, theta 5e6, expert
+# intermediate 1536, top-8) with fewer experts and a small vocabulary, so that the plain implementation stays fast:
+# the products, the attention and the routing run at the K, N and head sizes of the real model.
+WIDE = dict(vocab_size=1000, hidden_size=3072, num_hidden_layers=1, num_attention_heads=48, num_key_value_heads=8, head_dim=128,
+            rotary_dim=64, rope_theta=5e6, rms_norm_eps=1e-6, num_local_experts=16, num_experts_per_tok=8, intermediate_size=1536,
+            routed_scaling_factor=1.0, norm_topk_prob=True, tie_word_embeddings=False, max_position_embeddings=4096)
+
+
+@pytest.fixture(scope="module")
+def wide_folder(tmp_path_factory):
+    from llmx_amd import MiniMaxM3Config, RandomInit
+    from llmx_amd.weights.folder import write_random_model
+    folder = tmp_path_factory.mktemp("wide")
+    write_random_model(folder, MiniMaxM3Config(**WIDE), RandomInit(seed=3, std=0.02, norm_std=0.05, bias_range=0.05))
+    return str(folder)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_real_layer_widths(wide_folder, dtype):
+    import plain_model
+    from llmx_amd.engine import Engine, StepEntry
+    import random
+    cfg, w = plain_model.load_folder(wide_folder)
+    rng = random.Random(5)
+    tokens = [rng.randrange(1000) for _ in range(150)]
+    engine = Engine.load(wide_folder, dtype=dtype, kv_tokens=512, page_tokens=16, max_requests=2)
+    recorder = RoutingRecorder(1)
+    engine.observer = recorder
+    engine.add_request("w")
+    whole = engine.step([StepEntry("w", tokens, list(range(150)))]).clone().cpu()
+    engine.end_request("w")
+    picks = recorder.of("w", 150)
+    rounded = torch.bfloat16 if dtype == "bfloat16" else None
+    want, routing = plain_model.forward(cfg, w, tokens, torch.float64, rounded, return_routing=True, picks=picks if rounded else None)
+    if not rounded:
+        assert torch.equal(routing[0][0], picks[0]), "the float32 router picked other experts than the plain router"
+    tol = 3e-5 if dtype == "float32" else BF16_TOL
+    assert float((whole.double() - want).abs().max()) <= tol * float(want.abs().max())
+    # in portions (70 rows take the tiled kernels, 2 and 13 the streaming ones) and token by token at the end
+    engine.add_request("p")
+    cuts = [(0, 70), (70, 72), (72, 85), (85, 140)] + [(i, i + 1) for i in range(140, 150)]
+    rows = torch.cat([engine.step([StepEntry("p", tokens[a:b], list(range(b - a)))]).clone() for a, b in cuts]).cpu()
+    engine.end_request("p")
+    if dtype == "float32":
+        assert torch.equal(rows, whole)
+    else:
+        want_p = plain_model.forward(cfg, w, tokens, torch.float64, rounded, picks=recorder.of("p", 150))
+        assert float((rows.double() - want_p).abs().max()) <= tol * float(want_p.abs().max())
