@@ -9,7 +9,11 @@
 //   out^T[dim][col]  += V^T_tile[16 dims x 32 keys] . P^T[32 keys x 16 cols]
 // The value pages are stored transposed ([dim][token]) so that V^T's rows are contiguous, and the 32 keys of a step are
 // assigned to the product's k-slots in the order the score accumulators already hold them: no data moves between lanes.
-// A long context is split over several items whose partial (max, sum, out) are merged in split order by a second kernel.
+// Keys are grouped in fixed segments of 128 (absolute positions): each segment gets its own online softmax from scratch,
+// and the segments' (max, sum, out) are folded in key order with one formula (fold_segment).  A long context of a
+// decoding row is split over several items that write their segments' partials, which a second kernel folds; a prompt
+// tile folds its segments in registers.  Either way a row's result is the same bits: it does not depend on how many
+// rows the step holds or on how the context was split.
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -20,10 +24,19 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 #define AM_MAX_D 256
 #define AM_ITEM_INTS 8
+#define AM_SEG 128  // keys in a segment
+
+// state (M, L, O) <- state folded with a segment's (m, l, o); one element of O at a time.  An empty segment changes nothing.
+__device__ __forceinline__ void fold_weights(float M, float m, float& a, float& b, float& Mn) {
+    Mn = fmaxf(M, m);
+    a = __expf(M - Mn);
+    b = __expf(m - Mn);
+}
 
 // item: {row0, n_rows, head0, n_heads, split, n_splits, slot, unused}
 //   columns c = 0 .. n_rows*n_heads-1: row = row0 + c / n_heads, head = head0 + c % n_heads
-//   slot < 0: the item writes the final output; otherwise partials go to part_*[(slot) * 16 + c]
+//   slot < 0: the item folds its segments itself and writes the final output; otherwise segment s of the row (counted
+//   from the row's first segment) goes to part_*[(slot + s) * 16 + c]
 struct AttnMfmaArgs {
     const bf16_t* q;        // [T, n_heads, D]
     const bf16_t* k_cache;  // [pages, kv_heads, page_tokens, D]
@@ -39,7 +52,8 @@ struct AttnMfmaArgs {
     int n_items, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
 };
 
-template <int DT>  // DT = head_dim / 16 rounded up
+// DT = head_dim / 16 rounded up.  PARTIAL: the items write their segments (slot >= 0); otherwise they fold them (slot < 0).
+template <int DT, bool PARTIAL>
 __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs a) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int item_no = blockIdx.x * 4 + wave;
@@ -58,12 +72,14 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
     const int* table = a.tables + (size_t)a.row_entry[row0] * a.max_blocks;
     const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
     const int lo_first = (a.window > 0 && p_first - a.window + 1 > 0) ? p_first - a.window + 1 : 0;
-    // the item's keys: [lo32, p_last], cut into n_splits runs of whole 32-key steps
-    const int lo32 = lo_first & ~31;
-    const int n_steps = (p_last + 1 - lo32 + 31) >> 5;
-    const int steps_per = (n_steps + n_splits - 1) / n_splits;
-    const int key_begin = lo32 + split * steps_per * 32;
-    const int key_end = min(p_last + 1, key_begin + steps_per * 32);
+    // the item's keys: the segments seg_first .. p_last / 128 of the row, cut into n_splits runs of whole segments
+    const int seg_first = lo_first / AM_SEG;
+    const int n_seg = p_last / AM_SEG - seg_first + 1;
+    const int segs_per = (n_seg + n_splits - 1) / n_splits;
+    const int my_seg0 = seg_first + split * segs_per;
+    const int my_seg1 = min(seg_first + n_seg, my_seg0 + segs_per);
+    const int key_begin = my_seg0 * AM_SEG;
+    const int key_end = min(p_last + 1, my_seg1 * AM_SEG);
 
     // Q^T fragments: lane (column c, dims 32s + 8g ..)
     constexpr int QS = (DT + 1) / 2;
@@ -75,10 +91,13 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
         if (col_ok && d < D) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + d);
         qf[s] = __builtin_bit_cast(bf16x8_t, v);
     }
-    f32x4_t o[DT];
+    f32x4_t o[DT], o_tot[PARTIAL ? 1 : DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    float m = -INFINITY, l = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < (PARTIAL ? 1 : DT); ++dt) o_tot[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float m = -INFINITY, l = 0.0f;           // the running segment
+    float m_tot = -INFINITY, l_tot = 0.0f;   // the segments folded so far (slot < 0)
 
     // Software pipeline: while step i is multiplied, the keys of step i+1 and the page ids of step i+2 are on their way.
     struct Where {
@@ -180,99 +199,132 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
             o[dt] = f32x4_t{o[dt][0] * alpha, o[dt][1] * alpha, o[dt][2] * alpha, o[dt][3] * alpha};
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
         }
+        if (((j0 + 32) % AM_SEG) == 0 || j0 + 32 >= key_end) {
+            // the segment ends: write it out, or fold it into the segments before it
+            if (PARTIAL) {
+                if (col_ok) {
+                    const size_t at = (size_t)(slot + j0 / AM_SEG - seg_first) * 16 + c;
+                    float* dst = a.part_o + at * D;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+                        if (16 * dt + 4 * g < D) *reinterpret_cast<f32x4_t*>(dst + 16 * dt + 4 * g) = o[dt];   // D is a multiple of 16
+                    if (g == 0) {
+                        a.part_ml[at * 2] = m;
+                        a.part_ml[at * 2 + 1] = l;
+                    }
+                }
+            } else if (m != -INFINITY) {
+                if (m_tot == -INFINITY) {
+                    m_tot = m;
+                    l_tot = l;
+#pragma unroll
+                    for (int dt = 0; dt < (PARTIAL ? 1 : DT); ++dt) o_tot[dt] = o[dt];
+                } else {
+                    float fa, fb, mn;
+                    fold_weights(m_tot, m, fa, fb, mn);
+                    l_tot = l_tot * fa + l * fb;
+#pragma unroll
+                    for (int dt = 0; dt < (PARTIAL ? 1 : DT); ++dt)
+                        o_tot[dt] = f32x4_t{o_tot[dt][0] * fa + o[dt][0] * fb, o_tot[dt][1] * fa + o[dt][1] * fb,
+                                            o_tot[dt][2] * fa + o[dt][2] * fb, o_tot[dt][3] * fa + o[dt][3] * fb};
+                    m_tot = mn;
+                }
+            }
+            m = -INFINITY;
+            l = 0.0f;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
         here = next;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int s = 0; s < QS; ++s) kf[u][s] = kf_next[u][s];
     }
-    if (!col_ok) return;
+    if (!col_ok || PARTIAL) return;
     // lane holds dims 16dt + 4g + i of its column
-    if (slot < 0) {
-        const float inv = 1.0f / l;
-        bf16_t* dst = a.out + ((size_t)t * a.n_heads + h) * D;
+    const float inv = 1.0f / l_tot;
+    bf16_t* dst = a.out + ((size_t)t * a.n_heads + h) * D;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < (PARTIAL ? 1 : DT); ++dt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int d = 16 * dt + 4 * g + i;
-                if (d < D) dst[d] = f32_to_bf16(o[dt][i] * inv);
-            }
-    } else {
-        const size_t at = (size_t)slot * 16 + c;
-        float* dst = a.part_o + at * D;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int d = 16 * dt + 4 * g + i;
-                if (d < D) dst[d] = o[dt][i];
-            }
-        if (g == 0) {
-            a.part_ml[at * 2] = m;
-            a.part_ml[at * 2 + 1] = l;
+        for (int i = 0; i < 4; ++i) {
+            const int d = 16 * dt + 4 * g + i;
+            if (d < D) dst[d] = f32_to_bf16(o_tot[dt][i] * inv);
         }
-    }
 }
 
-// merge: one block per output (row, head).  merge item: {row, head, first_slot, n_splits, column}
-// The splits' weights exp(m_s - max) are formed once in LDS; the sum of weights * sums runs in split order; every
-// thread then adds its dims over the splits in split order, eight loads in flight at a time.
-#define AM_MAX_SPLITS 512
-__global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restrict__ merges, const float* __restrict__ part_o,
-                                                            const float* __restrict__ part_ml, bf16_t* __restrict__ out, int n_heads, int D) {
-    __shared__ float weight[AM_MAX_SPLITS];
-    __shared__ float sums[AM_MAX_SPLITS];
+// merge: one block per output (row, head).  merge item: {row, head, first_slot, column}.  The row's segments are folded
+// in key order with the formula the attention kernel uses for a tile's segments; thread d owns dim d.
+__global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restrict__ merges, const int* __restrict__ pos,
+                                                            const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                            bf16_t* __restrict__ out, int n_heads, int D, int window) {
     const int* mi = merges + (size_t)blockIdx.x * AM_ITEM_INTS;
-    const int t = mi[0], h = mi[1], first = mi[2], n = mi[3], c = mi[4];
-    for (int s = threadIdx.x; s < n; s += 128) {
-        const size_t at = (size_t)(first + s) * 16 + c;
-        weight[s] = part_ml[at * 2];        // the split's running max for now
-        sums[s] = part_ml[at * 2 + 1];
-    }
-    __syncthreads();
-    float mx = -INFINITY;
-    for (int s = 0; s < n; ++s) mx = fmaxf(mx, weight[s]);
-    __syncthreads();
-    for (int s = threadIdx.x; s < n; s += 128) weight[s] = weight[s] == -INFINITY ? 0.0f : __expf(weight[s] - mx);
-    __syncthreads();
-    float total = 0.0f;
-    for (int s = 0; s < n; ++s) total += weight[s] * sums[s];
-    const float inv = 1.0f / total;
-    const float* base = part_o + ((size_t)first * 16 + c) * D;
-    const size_t stride = (size_t)16 * D;
+    const int t = mi[0], h = mi[1], first = mi[2], c = mi[3];
+    const int p = pos[t];
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int n_seg = p / AM_SEG - lo / AM_SEG + 1;
+    const float* base_o = part_o + ((size_t)first * 16 + c) * D;
+    const float* base_ml = part_ml + ((size_t)first * 16 + c) * 2;
+    const size_t stride_o = (size_t)16 * D, stride_ml = 32;
     for (int d = threadIdx.x; d < D; d += 128) {
-        float acc = 0.0f;
-        int s = 0;
-        for (; s + 8 <= n; s += 8) {
-            float v[8];
+        float M = -INFINITY, L = 0.0f, O = 0.0f;
+        for (int s0 = 0; s0 < n_seg; s0 += 8) {
+            float ov[8], mv[8], lv[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = base[(size_t)(s + u) * stride + d];
+            for (int u = 0; u < 8; ++u) {
+                const bool in = s0 + u < n_seg;
+                ov[u] = in ? base_o[(size_t)(s0 + u) * stride_o + d] : 0.0f;
+                mv[u] = in ? base_ml[(size_t)(s0 + u) * stride_ml] : -INFINITY;
+                lv[u] = in ? base_ml[(size_t)(s0 + u) * stride_ml + 1] : 0.0f;
+            }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) acc += weight[s + u] * v[u];
+            for (int u = 0; u < 8; ++u) {
+                if (mv[u] == -INFINITY) continue;
+                if (M == -INFINITY) {
+                    M = mv[u];
+                    L = lv[u];
+                    O = ov[u];
+                } else {
+                    float fa, fb, mn;
+                    fold_weights(M, mv[u], fa, fb, mn);
+                    L = L * fa + lv[u] * fb;
+                    O = O * fa + ov[u] * fb;
+                    M = mn;
+                }
+            }
         }
-        for (; s < n; ++s) acc += weight[s] * base[(size_t)s * stride + d];
-        out[((size_t)t * n_heads + h) * D + d] = f32_to_bf16(acc * inv);
+        out[((size_t)t * n_heads + h) * D + d] = f32_to_bf16(O * (1.0f / L));
     }
 }
 
+// `items` holds first the n_direct items that fold their segments themselves (slot < 0), then the n_partial items
+// that write them (slot >= 0).
 extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
-                                         const int* tables, const int* items, int n_items, const int* merges, int n_merges, void* out,
-                                         float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
+                                         const int* tables, const int* items, int n_direct, int n_partial, const int* merges, int n_merges,
+                                         void* out, float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
                                          int page_tokens, int max_blocks, int window, hipStream_t stream) {
-    if (n_items <= 0) return 0;
+    if (n_direct + n_partial <= 0) return 0;
     if (head_dim % 16 || head_dim > AM_MAX_D || page_tokens % 16 || n_heads % n_kv_heads) return -2;
     AttnMfmaArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pos, row_entry, tables, items, (bf16_t*)out, part_o,
-                   part_ml, scale, n_items, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
-    const dim3 grid((n_items + 3) / 4), block(256);
+                   part_ml, scale, n_direct, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
+    AttnMfmaArgs b = a;
+    b.items = items + (size_t)n_direct * AM_ITEM_INTS;
+    b.n_items = n_partial;
+    const dim3 block(256);
     switch (head_dim / 16) {
-#define AM_CASE(DT) case DT: hipLaunchKernelGGL(paged_attention_mfma_kernel<DT>, grid, block, 0, stream, a); break;
+#define AM_CASE(DT)                                                                                                          \
+    case DT:                                                                                                                 \
+        if (n_direct > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, false>), dim3((n_direct + 3) / 4), block, 0, stream, a);  \
+        if (n_partial > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, true>), dim3((n_partial + 3) / 4), block, 0, stream, b); \
+        break;
         AM_CASE(1) AM_CASE(2) AM_CASE(3) AM_CASE(4) AM_CASE(5) AM_CASE(6) AM_CASE(7) AM_CASE(8)
         AM_CASE(9) AM_CASE(10) AM_CASE(11) AM_CASE(12) AM_CASE(13) AM_CASE(14) AM_CASE(15) AM_CASE(16)
 #undef AM_CASE
         default: return -2;
     }
     if (n_merges > 0)
-        hipLaunchKernelGGL(attention_merge_kernel, dim3(n_merges), dim3(128), 0, stream, merges, part_o, part_ml, (bf16_t*)out, n_heads, head_dim);
+        hipLaunchKernelGGL(attention_merge_kernel, dim3(n_merges), dim3(128), 0, stream, merges, pos, part_o, part_ml, (bf16_t*)out, n_heads, head_dim,
+                           window);
     return LLMX_CHECK_LAUNCH();
 }

@@ -1,16 +1,20 @@
 // LDS-tiled bf16 product for many rows (prompt portions): C[M,N] (+)= A[M,K] * W[N,K]^T on the matrix cores.
 //
-// A workgroup of 4 waves computes a 128 x 128 tile (each wave 64 x 64 as 2 x 2 products of 32x32x16); K is walked 64 at a
-// time: the next A and W tiles travel from global memory into registers while the current ones are multiplied out of LDS
-// (rows padded to 144 bytes so that the 16-byte operand reads of 8 consecutive rows fall into different banks).
+// A workgroup of 4 waves computes 128 rows x 128 features (each wave 64 x 64 as 4 x 4 products of 16x16x32); K is walked
+// 64 at a time: the next A and W tiles travel from global memory into registers while the current ones are multiplied out
+// of LDS (rows padded to 144 bytes so that the 16-byte operand reads of 8 consecutive rows fall into different banks).
 // Grouped form: blockIdx.y walks the (expert, row tile) pairs of the experts that have rows; A's rows are gathered
 // through the expert-sorted pair list and C's rows scattered to the pairs.  SwiGLU form: the tile's 128 weight rows
 // are 64 gate rows and the 64 up rows of the same features, and silu(gate) * up is stored.
-// An output element is one accumulator walked over k in steps of 16: its bits depend on K only.
+//
+// The arithmetic of an output element is the weight-streaming kernel's, bit for bit: the same 16x16x32 instruction with
+// the weights as its A operand and the same k-slots, K cut into the same `ks` runs of 32-wide steps, each run summed
+// from zero in step order, the runs' sums added in run order.  So a row's result does not depend on whether its step
+// held few rows or many.
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 enum : int { TL_STORE = 0, TL_ADD = 1, TL_SWIGLU = 2 };
@@ -32,9 +36,10 @@ struct TileArgs {
     long w_group_stride;
     int up_offset;
     int m_tiles;  // dense: number of row tiles
+    int ks;       // runs K is cut into (the weight-streaming kernel's waves per strip for this shape)
 };
 
-template <int EPI, typename TC, bool GROUPED>
+template <int EPI, typename TC, bool GROUPED, bool SPLIT>
 __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     __shared__ __attribute__((aligned(16))) bf16_t As[TL_BM * TL_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Ws[TL_BN * TL_LD];
@@ -134,24 +139,26 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         }
     };
 
-    // wave (wm, wn): rows 64*wm .., and its two column tiles
+    // wave (wm, wn): rows 64*wm .. (4 tiles of 16 rows), features: 4 tiles of 16 weight rows
     const int wm = wave >> 1, wn = wave & 1;
-    const int lr = lane & 31, lk = (lane >> 5) * 8;
-    int b_row[2];
-    if (EPI == TL_SWIGLU) {
-        b_row[0] = 32 * wn + lr;        // gate rows of features n0 + 32*wn + lr
-        b_row[1] = 64 + 32 * wn + lr;   // up rows of the same features
-    } else {
-        b_row[0] = 64 * wn + lr;
-        b_row[1] = 64 * wn + 32 + lr;
+    const int lr = lane & 15, lk = (lane >> 4) * 8;
+    int w_row[4];  // LDS rows of the wave's 4 feature tiles
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+        if (EPI == TL_SWIGLU)
+            w_row[f] = (f < 2 ? 0 : 64) + 32 * wn + 16 * (f & 1) + lr;   // tiles 0,1: gate rows; tiles 2,3: the up rows of the same features
+        else
+            w_row[f] = 64 * wn + 16 * f + lr;
     }
-    f32x16_t acc[2][2];
+    f32x4_t acc[4][4], total[SPLIT ? 4 : 1][SPLIT ? 4 : 1];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int f = 0; f < 4; ++f)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        for (int t = 0; t < 4; ++t) acc[f][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    const int steps_total = (K + 31) >> 5;
+    const int per = (steps_total + g.ks - 1) / g.ks;   // 32-wide steps in a run
+    int until_fold = per;                                // steps left in the current run
+    bool first_run = true;
 
     load_global(0);
     store_lds();
@@ -160,18 +167,34 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         const bool more = k0 + TL_BK < K;
         if (more) load_global(k0 + TL_BK);
 #pragma unroll
-        for (int kk = 0; kk < TL_BK; kk += 16) {
-            bf16x8_t af[2], bf[2];
+        for (int kk = 0; kk < TL_BK; kk += 32) {
+            if (k0 + kk < K) {
+                if (SPLIT && until_fold == 0) {
+                    // a run of K ends: its sum joins the runs before it, in run order
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                af[i] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[(64 * wm + 32 * i + lr) * TL_LD + kk + lk]));
+                    for (int f = 0; f < 4; ++f)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                bf[j] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[b_row[j] * TL_LD + kk + lk]));
+                        for (int t = 0; t < 4; ++t) {
+                            if (first_run) total[f][t] = acc[f][t];
+                            else total[f][t] = f32x4_t{total[f][t][0] + acc[f][t][0], total[f][t][1] + acc[f][t][1],
+                                                       total[f][t][2] + acc[f][t][2], total[f][t][3] + acc[f][t][3]};
+                            acc[f][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                        }
+                    first_run = false;
+                    until_fold = per;
+                }
+                bf16x8_t wf[4], af[4];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+                for (int f = 0; f < 4; ++f) wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[w_row[f] * TL_LD + kk + lk]));
 #pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                for (int t = 0; t < 4; ++t)
+                    af[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[(64 * wm + 16 * t + lr) * TL_LD + kk + lk]));
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[t], acc[f][t], 0, 0, 0);
+                --until_fold;
+            }
         }
         __syncthreads();
         if (more) {
@@ -179,53 +202,70 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
             __syncthreads();
         }
     }
+    if (SPLIT && !first_run) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                acc[f][t] = f32x4_t{total[f][t][0] + acc[f][t][0], total[f][t][1] + acc[f][t][1], total[f][t][2] + acc[f][t][2],
+                                    total[f][t][3] + acc[f][t][3]};
+    }
 
-    // acc[i][j][v]: row 64*wm + 32*i + 8*(v/4) + 4*(lane/32) + v%4, column lane%32 of column tile j
+    // acc[f][t][i]: feature (tile f) 4*(lane/16) + i, row 64*wm + 16*t + lane%16
+    const int fq = 4 * (lane >> 4);
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int t = 0; t < 4; ++t) {
+        const int rc = rows_c[64 * wm + 16 * t + lr];
+        if (rc < 0) continue;
+        TC* crow = (TC*)g.C + (size_t)rc * g.ldc;
+        if (EPI == TL_SWIGLU) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int row = 64 * wm + 32 * i + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-            const int rc = rows_c[row];
-            if (rc < 0) continue;
-            if (EPI == TL_SWIGLU) {
-                const int n = n0 + 32 * wn + lr;
-                if (n < g.N) {
-                    const float gt = acc[i][0][v], u = acc[i][1][v];
-                    st((TC*)g.C + (size_t)rc * g.ldc + n, (gt / (1.0f + expf(-gt))) * u);
-                }
-            } else {
+            for (int f = 0; f < 2; ++f)
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int n = n0 + 64 * wn + 32 * j + lr;
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + 32 * wn + 16 * f + fq + i;
                     if (n >= g.N) continue;
-                    TC* c = (TC*)g.C + (size_t)rc * g.ldc + n;
-                    float x = acc[i][j][v];
-                    if (EPI == TL_ADD) x = ld(c) + x;
-                    st(c, x);
+                    const float gt = acc[f][t][i], u = acc[f + 2][t][i];
+                    st(crow + n, (gt / (1.0f + expf(-gt))) * u);
                 }
-            }
+        } else {
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + 64 * wn + 16 * f + fq + i;
+                    if (n >= g.N) continue;
+                    float x = acc[f][t][i];
+                    if (EPI == TL_ADD) x = ld(crow + n) + x;
+                    st(crow + n, x);
+                }
         }
+    }
 }
 
 template <int EPI, typename TC>
 static void tile_launch(const TileArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
-    if (grouped)
-        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, true>), grid, dim3(256), 0, stream, g);
-    else
-        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, false>), grid, dim3(256), 0, stream, g);
+    if (grouped) {
+        if (g.ks > 1) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, true, true>), grid, dim3(256), 0, stream, g);
+        else hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, true, false>), grid, dim3(256), 0, stream, g);
+    } else {
+        if (g.ks > 1) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, false, true>), grid, dim3(256), 0, stream, g);
+        else hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, false, false>), grid, dim3(256), 0, stream, g);
+    }
 }
 
 // A and W bfloat16, K a multiple of 8.  n_groups == 0: dense over M rows.  n_groups > 0: grouped over the n_pairs = M
 // rows of `list`; `max_tiles` bounds the (expert, row tile) pairs (at most min(groups, pairs) + pairs / 128).
-extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi,
+// ks: the runs K is cut into; the caller passes what the weight-streaming kernel uses for this N and K.
+extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                               int n_groups, int max_tiles, const int* group_offsets, const int* list, int a_div, long w_group_stride,
                               int up_offset, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
     TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
-               w_group_stride, up_offset, (M + TL_BM - 1) / TL_BM};
+               w_group_stride, up_offset, (M + TL_BM - 1) / TL_BM, ks};
+    if (ks != 1 && ks != 2 && ks != 4 && ks != 8) return -2;
     const int feats = epi == TL_SWIGLU ? 64 : 128;
     dim3 grid((N + feats - 1) / feats, grouped ? max_tiles : g.m_tiles, 1);
     if (grid.y > 65535) return -2;

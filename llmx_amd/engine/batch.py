@@ -74,13 +74,14 @@ class StepState:
     def tables(self, group: int) -> torch.Tensor:
         return self._tables[group]
 
-    def attention_plan(self, n_heads: int, n_kv_heads: int):
+    def attention_plan(self, n_heads: int, n_kv_heads: int, window: int = 0):
         """The matrix-core attention kernel's work items for this step's rows (shared by layers with the same heads)."""
-        key = (n_heads, n_kv_heads)
+        key = (n_heads, n_kv_heads, window)
         plan = self._plans.get(key)
         if plan is None:
             from .. import ops
-            plan = ops.attention_plan([e.n for e in self.entries], [e.past + e.n for e in self.entries], n_heads, n_kv_heads, self.device)
+            plan = ops.attention_plan([e.n for e in self.entries], [e.past + e.n for e in self.entries], n_heads, n_kv_heads, self.device,
+                                      window)
             self._plans[key] = plan
         return plan
 

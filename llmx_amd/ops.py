@@ -59,14 +59,14 @@ def _declare(h) -> None:
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
-        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
+        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, P, P, I, I, I, I, I, F, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
         "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
         "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, P],
-        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
+        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
@@ -169,8 +169,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
                "gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
-        _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue, 0, 0, 0, 0, 1, 0,
-                                    N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm_tile")
+        _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
+                                    _split_k(-(-N // 16), K), 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm")
@@ -203,8 +203,8 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
                "grouped_gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
-        _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue, G,
-                                    min(G, n_pairs) + n_pairs // 128, _dev(offsets, "offsets", torch.int32, (G + 1,)),
+        _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
+                                    _split_k(-(-N // 16), K), G, min(G, n_pairs) + n_pairs // 128, _dev(offsets, "offsets", torch.int32, (G + 1,)),
                                     _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
                "grouped_gemm_tile")
         return
@@ -245,6 +245,8 @@ class AttentionPlan:
 
     def __init__(self, items, merges, n_slots, device):
         import numpy as np
+        items = [i for i in items if i[6] < 0] + [i for i in items if i[6] >= 0]   # those that fold their segments first
+        self.n_direct = sum(1 for i in items if i[6] < 0)
         self.n_items = len(items)
         self.n_merges = len(merges)
         self.n_slots = n_slots
@@ -254,22 +256,27 @@ class AttentionPlan:
 
 _PLAN_CACHE: dict = {}
 ATTENTION_TARGET_WAVES = 2048   # work items wanted before long contexts stop being split further
-ATTENTION_MIN_SPLIT_KEYS = 128  # a split covers at least this many keys
+ATTENTION_SEGMENT = 128         # keys in a segment: the unit contexts are split in (the kernel's AM_SEG)
 
 
-def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device) -> AttentionPlan:
+def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, window: int = 0) -> AttentionPlan:
     """row_counts[i]: rows of entry i in the step (entries' rows are consecutive, in order); contexts[i]: tokens the
-    entry holds after the step.  Single-row entries become one item per KV head (columns = its query heads), split over
-    the context when there are few of them; longer entries become tiles of 16 rows of one head."""
+    entry holds after the step.  Single-row entries become items per KV head (columns = its query heads) that share out
+    the context's 128-key segments when there are few rows; longer entries become tiles of 16 rows of one head.
+    How the context is shared out changes no result: segments are folded in key order either way."""
     ratio = n_heads // n_kv_heads
     head_chunks = [(kvh * ratio + c0, min(16, ratio - c0)) for kvh in range(n_kv_heads) for c0 in range(0, ratio, 16)]
     single = [i for i, n in enumerate(row_counts) if n == 1]
-    n_splits = 1
+    n_splits, seg_cap = 1, 1
     if single:
         base = len(single) * len(head_chunks)
         longest = max(contexts[i] for i in single)
-        n_splits = max(1, min(-(-ATTENTION_TARGET_WAVES // base), longest // ATTENTION_MIN_SPLIT_KEYS, 512))
-    key = (tuple(row_counts), n_heads, n_kv_heads, n_splits, str(device))
+        if window > 0:
+            longest = min(longest, window + ATTENTION_SEGMENT)
+        seg_cap = -(-longest // ATTENTION_SEGMENT) + 1
+        seg_cap = -(-seg_cap // 8) * 8       # in steps of 8, so a growing context reuses a plan for 1,024 tokens
+        n_splits = max(1, min(-(-ATTENTION_TARGET_WAVES // base), seg_cap))
+    key = (tuple(row_counts), n_heads, n_kv_heads, n_splits, seg_cap, str(device))
     plan = _PLAN_CACHE.get(key)
     if plan is not None:
         return plan
@@ -291,10 +298,10 @@ def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device) 
                 items.append([row0s[i], 1, head0, nh, 0, 1, -1, 0])
                 continue
             for c in range(nh):
-                merges.append([row0s[i], head0 + c, slot, n_splits, c, 0, 0, 0])
+                merges.append([row0s[i], head0 + c, slot, c, 0, 0, 0, 0])
             for sp in range(n_splits):
                 items.append([row0s[i], 1, head0, nh, sp, n_splits, slot, 0])
-                slot += 1
+            slot += seg_cap
     plan = AttentionPlan(items, merges, slot, device)
     if len(_PLAN_CACHE) > 256:
         _PLAN_CACHE.clear()
@@ -327,7 +334,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 scratch = lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=q.device)
             part_o = scratch("attention.part_o", (plan.n_slots * 16, head_dim), torch.float32)
             part_ml = scratch("attention.part_ml", (plan.n_slots * 16, 2), torch.float32)
-        _check(lib().llmx_paged_attention_mfma(*common, _dev(plan.items, "items", torch.int32), plan.n_items,
+        _check(lib().llmx_paged_attention_mfma(*common, _dev(plan.items, "items", torch.int32), plan.n_direct, plan.n_items - plan.n_direct,
                                                _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
                                                _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale), n_heads, n_kv_heads,
                                                head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention_mfma")

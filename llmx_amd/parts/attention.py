@@ -82,7 +82,7 @@ class Attention(Mixer):
         o = step.buf("attention.out", (T, self.q_width), act)
         plan = None
         if ops.attention_mfma_ok(act, self.head_dim, cache.k.shape[2]):
-            plan = step.attention_plan(self.heads, self.kv_heads)
+            plan = step.attention_plan(self.heads, self.kv_heads, int(self.window or 0))
         ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
                             window=int(self.window or 0), plan=plan, scratch=step.buf)
         ops.gemm(o, self.wo, out, ops.EPI_ADD if accumulate else ops.EPI_STORE)

@@ -118,6 +118,12 @@ def test_gemm_matrix_cores_bf16(M, N, K):
     acc = base.clone()
     o.gemm(a, w, acc, o.EPI_ADD)
     assert torch.equal(acc, base + c)
+    if M > o.SKINNY_MAX_ROWS:
+        # the tiled kernel gives each row the bits the weight-streaming kernel gives it alone or among few rows
+        for rows in ([0], [M - 1], list(range(M - 17, M))):
+            few = torch.empty(len(rows), N, dtype=torch.float32, device=DEV)
+            o.gemm(a[rows].contiguous(), w, few)
+            assert torch.equal(few, c[rows]), "a row's bits depend on how many rows the product has"
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 8, 64), (3, 16, 96), (8, 256, 3072), (17, 24, 100), (70, 40, 72), (2048, 256, 3072), (5, 13, 30)])
@@ -161,6 +167,10 @@ def test_gemm_swiglu(M, F, K, dtype):
     c2 = torch.empty_like(c)
     ops().gemm(a, swapped, c2, ops().EPI_SWIGLU)
     assert not torch.allclose(c, c2)
+    if M > 1:
+        c1 = torch.empty(1, F, dtype=torch.float32, device=DEV)
+        ops().gemm(a[M - 1:M].contiguous(), w, c1, ops().EPI_SWIGLU)
+        assert torch.equal(c1[0], c[M - 1]), "a row's bits depend on how many rows the product has"
 
 
 def routed_setup(T, X, k, seed):
@@ -334,6 +344,40 @@ def test_attention_split_context(lens, Hq, Hkv, D):
     universal, _ = attention_case(lens, Hq, Hkv, D, D // 2, 16, torch.bfloat16, second_single=True, planned=False)
     for g, u in zip(got, universal):
         assert (g - u).abs().max() <= 1.2e-2 * u.abs().max()
+
+
+@pytest.mark.parametrize("L,Hq,Hkv,D,window", [(700, 12, 2, 128, 0), (131, 4, 4, 64, 0), (1000, 6, 1, 48, 0), (900, 8, 2, 64, 300)])
+def test_attention_row_is_the_same_bits_alone_or_in_a_tile(L, Hq, Hkv, D, window):
+    """The matrix-core kernel gives a row the same bits as a single decoded row (its context shared out over several
+    items, or not) and as one of 16 rows of a prompt tile."""
+    o = ops()
+    page = 16
+    n_pages = -(-L // page)
+    order = list(range(n_pages))
+    random.Random(L).shuffle(order)
+    table = torch.tensor([order], dtype=torch.int32, device=DEV)
+    k_cache = rnd(n_pages, Hkv, page, D, dtype=torch.bfloat16, scale=0.5)
+    v_cache = rnd(n_pages, Hkv, D, page, dtype=torch.bfloat16, seed=2)
+    n = 37
+    q = rnd(n, Hq * D, dtype=torch.bfloat16, seed=3)
+    pos = torch.arange(L - n, L, dtype=torch.int32, device=DEV)
+    ent = torch.zeros(n, dtype=torch.int32, device=DEV)
+    scale = 1.0 / math.sqrt(D)
+    tile = torch.empty_like(q)
+    o.paged_attention(q, k_cache, v_cache, pos, ent, table, tile, scale, Hq, window, plan=o.attention_plan([n], [L], Hq, Hkv, DEV, window))
+    for r in (0, 15, 16, n - 1):
+        ctx = L - n + r + 1
+        for target in (1, 100000):       # one item per KV head, or the context shared out over many
+            saved = o.ATTENTION_TARGET_WAVES
+            o.ATTENTION_TARGET_WAVES = target
+            try:
+                plan = o.attention_plan([1], [ctx], Hq, Hkv, DEV, window)
+            finally:
+                o.ATTENTION_TARGET_WAVES = saved
+            assert (plan.n_merges > 0) == (target > 1)
+            alone = torch.empty(1, Hq * D, dtype=torch.bfloat16, device=DEV)
+            o.paged_attention(q[r:r + 1].contiguous(), k_cache, v_cache, pos[r:r + 1].contiguous(), ent[:1], table, alone, scale, Hq, window, plan=plan)
+            assert torch.equal(alone[0], tile[r]), f"row {r} (context {ctx}, target {target}) differs from its bits in the tile"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

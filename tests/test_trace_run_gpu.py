@@ -2,7 +2,7 @@
 
 The same requests are replayed whole, with the last 32 tokens one by one, in portions of changing size, and mixed with
 other requests in a pool so small that pages are used again; float32 and bfloat16; all compared with the plain
-implementation (and, in float32, with each other bit for bit)."""
+implementation, and with each other bit for bit."""
 
 from __future__ import annotations
 
@@ -118,8 +118,7 @@ def test_replay_every_cutting(name, dtype, tmp_path):
         out = replay(name, dtype, cut_steps(rid, toks, cuts), tmp_path / label, max_tokens=128, extra=extra)
         got = np.concatenate([out[i] for i in range(len(cuts))])
         check(rid, got)
-        if dtype == "float32":
-            assert np.array_equal(got, golden[rid]), f"{label}: differs from the whole prompt in float32"
+        assert np.array_equal(got, golden[rid]), f"{label}: differs from the whole prompt in {dtype}"
     # 4. mixed, up to four live requests, in a pool of four requests' worth of pages
     steps, where = mixed_steps(requests)
     # the pool: the most tokens live requests hold at any time, each request's count rounded up to a multiple of 64
@@ -135,8 +134,7 @@ def test_replay_every_cutting(name, dtype, tmp_path):
     for rid in requests:
         got = np.concatenate([out[s][row:row + k] for s, row, k in where[rid]])
         check(rid, got)
-        if dtype == "float32":
-            assert np.array_equal(got, golden[rid]), f"{rid} in the mix differs from its run alone in float32"
+        assert np.array_equal(got, golden[rid]), f"{rid} in the mix differs from its run alone in {dtype}"
 
 
 def test_replay_default_page_and_empty_want(tmp_path):
@@ -160,8 +158,7 @@ def test_replay_default_page_and_empty_want(tmp_path):
         assert np.abs(out[3][0] - want[48]).max() <= tol * scale and np.abs(out[4][0] - want[49]).max() <= tol * scale
         assert np.abs(out[1][0] - want[6]).max() <= tol * scale                 # the prompt's first 7 tokens are x's first 7
         assert np.abs(out[2][1] - want[0]).max() <= tol * scale and np.abs(out[2][2] - want[6]).max() <= tol * scale
-        if dtype == "float32":
-            assert np.array_equal(out[1][0], out[2][2])                          # y's second life equals its first
+        assert np.array_equal(out[1][0], out[2][2])                              # y's second life equals its first
 
 
 def test_replay_refuses_bad_weights(tmp_path):
