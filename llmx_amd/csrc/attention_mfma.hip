@@ -15,6 +15,7 @@
 // tile folds its segments in registers.  Either way a row's result is the same bits: it does not depend on how many
 // rows the step holds or on how the context was split.
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
@@ -31,6 +32,79 @@ __device__ __forceinline__ void fold_weights(float M, float m, float& a, float& 
     Mn = fmaxf(M, m);
     a = __expf(M - Mn);
     b = __expf(m - Mn);
+}
+
+// One step of a column tile: 32 keys against the tile's 16 columns.  kf: the keys (two tiles of 16), vf: the values
+// transposed, qf: the columns' queries; ok: bit 4u+i says whether key 16u + 4g + i counts for this lane's column
+// (MASKED false: all 32 keys count for every column, and the selects fall away; the sums are the same).
+// Updates the running segment (o, m, l).  Every form of the kernel calls this, so a column's bits do not depend on the form.
+template <int DT, bool MASKED>
+__device__ __forceinline__ void attention_step(const bf16x8_t (&kf)[2][(DT + 1) / 2], const bf16x8_t (&vf)[DT], const bf16x8_t (&qf)[(DT + 1) / 2],
+                                               unsigned ok, float scale, f32x4_t (&o)[DT], float& m, float& l) {
+    constexpr int QS = (DT + 1) / 2;
+    // scores^T: lane holds keys 4g + i of each tile for its column
+    f32x4_t s_acc[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        s_acc[u] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int s = 0; s < QS; ++s) s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][s], qf[s], s_acc[u], 0, 0, 0);
+    }
+    // online softmax of the column over the step's 32 keys
+    float sc[8];
+    float step_max = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float v = (!MASKED || ((ok >> (4 * u + i)) & 1u)) ? s_acc[u][i] * scale : -INFINITY;
+            sc[4 * u + i] = v;
+            step_max = fmaxf(step_max, v);
+        }
+    step_max = fmaxf(step_max, __shfl_xor(step_max, 16, 64));
+    step_max = fmaxf(step_max, __shfl_xor(step_max, 32, 64));
+    const float m_new = fmaxf(m, step_max);
+    const float alpha = (MASKED && m_new == -INFINITY) ? 1.0f : __expf(m - m_new);   // m = -inf gives 0
+    float step_sum = 0.0f;
+    float pw[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        pw[i] = (MASKED && sc[i] == -INFINITY) ? 0.0f : __expf(sc[i] - m_new);
+        step_sum += pw[i];
+    }
+    step_sum += __shfl_xor(step_sum, 16, 64);
+    step_sum += __shfl_xor(step_sum, 32, 64);
+    l = l * alpha + step_sum;
+    m = m_new;
+    bf16x8_t pf;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) pf[i] = (__bf16)pw[i];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        o[dt] = f32x4_t{o[dt][0] * alpha, o[dt][1] * alpha, o[dt][2] * alpha, o[dt][3] * alpha};
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
+    }
+}
+
+// A finished segment (o, m, l) folded into the segments before it (o_tot, m_tot, l_tot); an empty segment changes nothing.
+template <int DT>
+__device__ __forceinline__ void fold_segment(const f32x4_t (&o)[DT], float m, float l, f32x4_t (&o_tot)[DT], float& m_tot, float& l_tot) {
+    if (m == -INFINITY) return;
+    if (m_tot == -INFINITY) {
+        m_tot = m;
+        l_tot = l;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o_tot[dt] = o[dt];
+        return;
+    }
+    float fa, fb, mn;
+    fold_weights(m_tot, m, fa, fb, mn);
+    l_tot = l_tot * fa + l * fb;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+        o_tot[dt] = f32x4_t{o_tot[dt][0] * fa + o[dt][0] * fb, o_tot[dt][1] * fa + o[dt][1] * fb,
+                            o_tot[dt][2] * fa + o[dt][2] * fb, o_tot[dt][3] * fa + o[dt][3] * fb};
+    m_tot = mn;
 }
 
 // item: {row0, n_rows, head0, n_heads, split, n_splits, slot, unused}
@@ -72,6 +146,7 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
     const int* table = a.tables + (size_t)a.row_entry[row0] * a.max_blocks;
     const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
     const int lo_first = (a.window > 0 && p_first - a.window + 1 > 0) ? p_first - a.window + 1 : 0;
+    const int lo_last = (a.window > 0 && p_last - a.window + 1 > 0) ? p_last - a.window + 1 : 0;
     // the item's keys: the segments seg_first .. p_last / 128 of the row, cut into n_splits runs of whole segments
     const int seg_first = lo_first / AM_SEG;
     const int n_seg = p_last / AM_SEG - seg_first + 1;
@@ -155,53 +230,22 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
         page_next0 = page_of(j0 + 64);
         page_next1 = page_of(j0 + 80);
 
-        // scores^T: lane holds keys 4g + i of each tile for its column
-        f32x4_t s_acc[2];
+        if (j0 + 31 <= p_first && j0 >= lo_last && here.in[0] && here.in[1]) {
+            attention_step<DT, false>(kf, vf, qf, 0xffu, a.scale, o, m, l);   // every key counts for every column
+        } else {
+            unsigned ok = 0u;
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            s_acc[u] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int s = 0; s < QS; ++s) s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][s], qf[s], s_acc[u], 0, 0, 0);
-        }
-        // online softmax of the column over the step's 32 keys
-        float sc[8];
-        float step_max = -INFINITY;
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int key = j0 + 16 * u + 4 * g + i;
-                const bool ok = here.in[u] && col_ok && key <= p_col && key >= lo_col && key < key_end;
-                const float v = ok ? s_acc[u][i] * a.scale : -INFINITY;
-                sc[4 * u + i] = v;
-                step_max = fmaxf(step_max, v);
-            }
-        step_max = fmaxf(step_max, __shfl_xor(step_max, 16, 64));
-        step_max = fmaxf(step_max, __shfl_xor(step_max, 32, 64));
-        const float m_new = fmaxf(m, step_max);
-        const float alpha = (m_new == -INFINITY) ? 1.0f : __expf(m - m_new);   // m = -inf gives 0
-        float step_sum = 0.0f;
-        float pw[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            pw[i] = (sc[i] == -INFINITY) ? 0.0f : __expf(sc[i] - m_new);
-            step_sum += pw[i];
-        }
-        step_sum += __shfl_xor(step_sum, 16, 64);
-        step_sum += __shfl_xor(step_sum, 32, 64);
-        l = l * alpha + step_sum;
-        m = m_new;
-        bf16x8_t pf;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) pf[i] = (__bf16)pw[i];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            o[dt] = f32x4_t{o[dt][0] * alpha, o[dt][1] * alpha, o[dt][2] * alpha, o[dt][3] * alpha};
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
+                for (int i = 0; i < 4; ++i) {
+                    const int key = j0 + 16 * u + 4 * g + i;
+                    if (here.in[u] && col_ok && key <= p_col && key >= lo_col && key < key_end) ok |= 1u << (4 * u + i);
+                }
+            attention_step<DT, true>(kf, vf, qf, ok, a.scale, o, m, l);
         }
         if (((j0 + 32) % AM_SEG) == 0 || j0 + 32 >= key_end) {
             // the segment ends: write it out, or fold it into the segments before it
-            if (PARTIAL) {
+            if constexpr (PARTIAL) {
                 if (col_ok) {
                     const size_t at = (size_t)(slot + j0 / AM_SEG - seg_first) * 16 + c;
                     float* dst = a.part_o + at * D;
@@ -213,22 +257,8 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
                         a.part_ml[at * 2 + 1] = l;
                     }
                 }
-            } else if (m != -INFINITY) {
-                if (m_tot == -INFINITY) {
-                    m_tot = m;
-                    l_tot = l;
-#pragma unroll
-                    for (int dt = 0; dt < (PARTIAL ? 1 : DT); ++dt) o_tot[dt] = o[dt];
-                } else {
-                    float fa, fb, mn;
-                    fold_weights(m_tot, m, fa, fb, mn);
-                    l_tot = l_tot * fa + l * fb;
-#pragma unroll
-                    for (int dt = 0; dt < (PARTIAL ? 1 : DT); ++dt)
-                        o_tot[dt] = f32x4_t{o_tot[dt][0] * fa + o[dt][0] * fb, o_tot[dt][1] * fa + o[dt][1] * fb,
-                                            o_tot[dt][2] * fa + o[dt][2] * fb, o_tot[dt][3] * fa + o[dt][3] * fb};
-                    m_tot = mn;
-                }
+            } else {
+                fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
             }
             m = -INFINITY;
             l = 0.0f;
@@ -252,6 +282,202 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
             const int d = 16 * dt + 4 * g + i;
             if (d < D) dst[d] = f32_to_bf16(o_tot[dt][i] * inv);
         }
+}
+
+// Prompt tiles that share their keys: a workgroup's 4 waves hold 4 items (tiles of up to 16 rows of one head each) of one
+// request and one KV head, for instance 4 of the query heads that read it.  The 32 keys and values of a step are
+// brought from the pages into LDS once by all 256 threads (double-buffered: the next step's are on their way while
+// this step is multiplied) and every wave takes its fragments from there, so each byte of the cache is read once for
+// 4 tiles.  A wave steps through its own range of keys only; per column the arithmetic is attention_step and
+// fold_segment as in the kernel above.  Items with n_rows == 0 fill up the last workgroup of a KV head.
+template <int DT>
+__global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_kernel(AttnMfmaArgs a) {
+    constexpr int QS = (DT + 1) / 2;
+    constexpr int DP = 16 * DT;          // head_dim (a multiple of 16)
+    constexpr int K_LD = DP + 8;         // bf16 elements a key's row takes in LDS
+    constexpr int V_LD = 36;             // bf16 elements a dim's row of 32 keys takes in LDS
+    constexpr int K_CHUNKS = 32 * DP / 8;   // 16-byte chunks of a step's keys
+    constexpr int V_CHUNKS = DP * 4;        // and of its values: dim d, tile u, half h -> 8 tokens
+    constexpr int K_ROUNDS = (K_CHUNKS + 255) / 256, V_ROUNDS = (V_CHUNKS + 255) / 256;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[2][32 * K_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[2][DP * V_LD];
+    __shared__ int ranges[4][2];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int* it = a.items + ((size_t)blockIdx.x * 4 + wave) * AM_ITEM_INTS;
+    const int row0 = __builtin_amdgcn_readfirstlane(it[0]), n_rows = __builtin_amdgcn_readfirstlane(it[1]);
+    const int h = __builtin_amdgcn_readfirstlane(it[2]);
+    const int lead_row = a.items[(size_t)blockIdx.x * 4 * AM_ITEM_INTS];   // the first item is never a filler
+    const int lead_head = a.items[(size_t)blockIdx.x * 4 * AM_ITEM_INTS + 2];
+    const int D = DP, bt = a.page_tokens, Hkv = a.n_kv_heads;
+    const int kvh = lead_head / (a.n_heads / Hkv);
+    const int* table = a.tables + (size_t)a.row_entry[lead_row] * a.max_blocks;
+    const int c = lane & 15, g = lane >> 4;
+    const bool col_ok = c < n_rows;
+    const int t = row0 + (col_ok ? c : 0);
+    int p_col = 0, lo_col = 0, key_begin = 0, key_end = 0, p_first = -1, lo_last = 0;
+    if (n_rows > 0) {
+        p_col = a.pos[t];
+        p_first = __builtin_amdgcn_readfirstlane(a.pos[row0]);
+        const int p_last = __builtin_amdgcn_readfirstlane(a.pos[row0 + n_rows - 1]);
+        lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
+        const int lo_first = (a.window > 0 && p_first - a.window + 1 > 0) ? p_first - a.window + 1 : 0;
+        lo_last = (a.window > 0 && p_last - a.window + 1 > 0) ? p_last - a.window + 1 : 0;
+        key_begin = (lo_first / AM_SEG) * AM_SEG;
+        key_end = p_last + 1;
+    }
+    if (lane == 0) {
+        ranges[wave][0] = n_rows > 0 ? key_begin : 0x7fffffff;
+        ranges[wave][1] = key_end;
+    }
+    __syncthreads();
+    const int block_begin = __builtin_amdgcn_readfirstlane(min(min(ranges[0][0], ranges[1][0]), min(ranges[2][0], ranges[3][0])));
+    const int block_end = __builtin_amdgcn_readfirstlane(max(max(ranges[0][1], ranges[1][1]), max(ranges[2][1], ranges[3][1])));
+
+    bf16x8_t qf[QS];
+#pragma unroll
+    for (int s = 0; s < QS; ++s) {
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        const int d = 32 * s + 8 * g;
+        if (col_ok && d < D) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + d);
+        qf[s] = __builtin_bit_cast(bf16x8_t, v);
+    }
+    f32x4_t o[DT], o_tot[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        o_tot[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    float m = -INFINITY, l = 0.0f, m_tot = -INFINITY, l_tot = 0.0f;
+
+    // Staging: the thread's chunks of a step go from the pages into registers, then into LDS.  What a chunk is (which
+    // key or dim, which of the step's two tiles) is fixed per thread; a step brings only the two tiles' base addresses.
+    int k_off[K_ROUNDS], k_lds[K_ROUNDS], v_off[V_ROUNDS], v_lds[V_ROUNDS];
+    bool k_second[K_ROUNDS], v_second[V_ROUNDS];
+#pragma unroll
+    for (int i = 0; i < K_ROUNDS; ++i) {
+        const int ch = tid + 256 * i;          // key ch / (DP/8) of the step, dims 8 * (ch % (DP/8)) ..
+        const int key = ch / (DP / 8), dc = ch % (DP / 8);
+        k_second[i] = key >= 16;
+        k_off[i] = (key & 15) * D + 8 * dc;
+        k_lds[i] = ch < K_CHUNKS ? key * K_LD + 8 * dc : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < V_ROUNDS; ++i) {
+        const int ch = tid + 256 * i;          // dim ch / 4, tile (ch / 2) % 2, tokens 8 * (ch % 2) .. of the tile
+        const int d = ch >> 2, u = (ch >> 1) & 1, half = ch & 1;
+        v_second[i] = u == 1;
+        v_off[i] = d * bt + 8 * half;
+        v_lds[i] = ch < V_CHUNKS ? d * V_LD + 16 * u + 8 * half : -1;
+    }
+    u32x4_t k_reg[K_ROUNDS], v_reg[V_ROUNDS];
+    auto page_of = [&](int key0) { return key0 < block_end ? __builtin_amdgcn_readfirstlane(table[key0 / bt]) : -1; };
+    auto fetch = [&](int j0, int page0, int page1) {
+        // the tiles' first key and first value in the cache (uniform)
+        const int sub0 = j0 % bt, sub1 = (j0 + 16) % bt;
+        const size_t head0 = (size_t)(page0 < 0 ? 0 : page0) * Hkv + kvh, head1 = (size_t)(page1 < 0 ? 0 : page1) * Hkv + kvh;
+        const bf16_t* kb0 = a.k_cache + (head0 * bt + sub0) * D;
+        const bf16_t* kb1 = a.k_cache + (head1 * bt + sub1) * D;
+        const bf16_t* vb0 = a.v_cache + head0 * D * bt + sub0;
+        const bf16_t* vb1 = a.v_cache + head1 * D * bt + sub1;
+        const bool in0 = page0 >= 0 && j0 < block_end, in1 = page1 >= 0 && j0 + 16 < block_end;
+#pragma unroll
+        for (int i = 0; i < K_ROUNDS; ++i) {
+            u32x4_t v = {0u, 0u, 0u, 0u};
+            if (k_lds[i] >= 0 && (k_second[i] ? in1 : in0)) v = *reinterpret_cast<const u32x4_t*>((k_second[i] ? kb1 : kb0) + k_off[i]);
+            k_reg[i] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < V_ROUNDS; ++i) {
+            u32x4_t v = {0u, 0u, 0u, 0u};
+            if (v_lds[i] >= 0 && (v_second[i] ? in1 : in0)) v = *reinterpret_cast<const u32x4_t*>((v_second[i] ? vb1 : vb0) + v_off[i]);
+            v_reg[i] = v;
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < K_ROUNDS; ++i)
+            if (k_lds[i] >= 0) *reinterpret_cast<u32x4_t*>(&Ks[buf][k_lds[i]]) = k_reg[i];
+#pragma unroll
+        for (int i = 0; i < V_ROUNDS; ++i)
+            if (v_lds[i] >= 0) {
+                u32x2_t* dst = reinterpret_cast<u32x2_t*>(&Vs[buf][v_lds[i]]);
+                dst[0] = u32x2_t{v_reg[i][0], v_reg[i][1]};
+                dst[1] = u32x2_t{v_reg[i][2], v_reg[i][3]};
+            }
+    };
+    const int k_at = c * K_LD + 8 * g, v_at = c * V_LD + 4 * g;   // where the lane's fragments start in a buffer
+    int page_next0, page_next1;
+    // one step from buffer `buf` (a constant where it is called, so that the LDS addresses are immediates)
+    auto step = [&](int j0, auto buf_c) {
+        constexpr int buf = decltype(buf_c)::value;
+        const bool more = j0 + 32 < block_end;
+        if (more) fetch(j0 + 32, page_next0, page_next1);
+        page_next0 = page_of(j0 + 64);
+        page_next1 = page_of(j0 + 80);
+        if (j0 >= key_begin && j0 < key_end) {
+            bf16x8_t kf[2][QS], vf[DT];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int s = 0; s < QS; ++s) {
+                    u32x4_t v = {0u, 0u, 0u, 0u};
+                    if (32 * s + 8 * g < DP) v = *reinterpret_cast<const u32x4_t*>(&Ks[buf][k_at + 16 * u * K_LD + 32 * s]);
+                    kf[u][s] = __builtin_bit_cast(bf16x8_t, v);
+                }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(&Vs[buf][v_at + 16 * dt * V_LD]);
+                const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(&Vs[buf][v_at + 16 * dt * V_LD + 16]);
+                const u32x4_t v = {v0[0], v0[1], v1[0], v1[1]};
+                vf[dt] = __builtin_bit_cast(bf16x8_t, v);
+            }
+            if (j0 + 31 <= p_first && j0 >= lo_last) {
+                attention_step<DT, false>(kf, vf, qf, 0xffu, a.scale, o, m, l);   // every key counts for every column
+            } else {
+                unsigned ok = 0u;
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = j0 + 16 * u + 4 * g + i;
+                        if (col_ok && key <= p_col && key >= lo_col && key < key_end) ok |= 1u << (4 * u + i);
+                    }
+                attention_step<DT, true>(kf, vf, qf, ok, a.scale, o, m, l);
+            }
+            if (((j0 + 32) % AM_SEG) == 0 || j0 + 32 >= key_end) {
+                fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
+                m = -INFINITY;
+                l = 0.0f;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+    };
+
+    if (block_begin >= block_end) return;
+    fetch(block_begin, page_of(block_begin), page_of(block_begin + 16));
+    page_next0 = page_of(block_begin + 32);
+    page_next1 = page_of(block_begin + 48);
+    stage(0);
+    __syncthreads();
+    for (int j0 = block_begin; j0 < block_end; j0 += 64) {
+        step(j0, std::integral_constant<int, 0>{});
+        if (j0 + 32 < block_end) step(j0 + 32, std::integral_constant<int, 1>{});
+    }
+    if (!col_ok) return;
+    const float inv = 1.0f / l_tot;
+    bf16_t* dst = a.out + ((size_t)t * a.n_heads + h) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const int d = 16 * dt + 4 * g;
+        const u32x2_t packed = {(uint32_t)f32_to_bf16(o_tot[dt][0] * inv) | ((uint32_t)f32_to_bf16(o_tot[dt][1] * inv) << 16),
+                                (uint32_t)f32_to_bf16(o_tot[dt][2] * inv) | ((uint32_t)f32_to_bf16(o_tot[dt][3] * inv) << 16)};
+        *reinterpret_cast<u32x2_t*>(dst + d) = packed;
+    }
 }
 
 // merge: one block per output (row, head).  merge item: {row, head, first_slot, column}.  The row's segments are folded
@@ -298,23 +524,30 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
     }
 }
 
-// `items` holds first the n_direct items that fold their segments themselves (slot < 0), then the n_partial items
-// that write them (slot >= 0).
+// `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 4: one workgroup each 4),
+// then the n_direct items that fold their segments themselves (slot < 0), then the n_partial items that write them
+// (slot >= 0).
 extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
-                                         const int* tables, const int* items, int n_direct, int n_partial, const int* merges, int n_merges,
+                                         const int* tables, const int* items, int n_shared, int n_direct, int n_partial, const int* merges,
+                                         int n_merges,
                                          void* out, float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
                                          int page_tokens, int max_blocks, int window, hipStream_t stream) {
-    if (n_direct + n_partial <= 0) return 0;
+    if (n_shared + n_direct + n_partial <= 0) return 0;
+    if (n_shared % 4) return -2;
     if (head_dim % 16 || head_dim > AM_MAX_D || page_tokens % 16 || n_heads % n_kv_heads) return -2;
     AttnMfmaArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pos, row_entry, tables, items, (bf16_t*)out, part_o,
                    part_ml, scale, n_direct, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
+    AttnMfmaArgs sh = a;
+    sh.n_items = n_shared;
+    a.items = items + (size_t)n_shared * AM_ITEM_INTS;
     AttnMfmaArgs b = a;
-    b.items = items + (size_t)n_direct * AM_ITEM_INTS;
+    b.items = a.items + (size_t)n_direct * AM_ITEM_INTS;
     b.n_items = n_partial;
     const dim3 block(256);
     switch (head_dim / 16) {
 #define AM_CASE(DT)                                                                                                          \
     case DT:                                                                                                                 \
+        if (n_shared > 0) hipLaunchKernelGGL((paged_attention_tiles_kernel<DT>), dim3(n_shared / 4), block, 0, stream, sh);             \
         if (n_direct > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, false>), dim3((n_direct + 3) / 4), block, 0, stream, a);  \
         if (n_partial > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, true>), dim3((n_partial + 3) / 4), block, 0, stream, b); \
         break;

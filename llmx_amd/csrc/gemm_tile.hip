@@ -1,6 +1,7 @@
 // LDS-tiled bf16 product for many rows (prompt portions): C[M,N] (+)= A[M,K] * W[N,K]^T on the matrix cores.
 //
-// A workgroup of 4 waves computes 128 rows x 128 features (each wave 64 x 64 as 4 x 4 products of 16x16x32); K is walked
+// A workgroup of 4 waves computes 64 rows x 128 features (each wave 32 rows x 64 features as 2 x 4 products of 16x16x32, so
+// that the accumulators of the current run of K and of the runs before it fit in registers twice over); K is walked
 // 64 at a time: the next A and W tiles travel from global memory into registers while the current ones are multiplied out
 // of LDS (rows padded to 144 bytes so that the 16-byte operand reads of 8 consecutive rows fall into different banks).
 // Grouped form: blockIdx.y walks the (expert, row tile) pairs of the experts that have rows; A's rows are gathered
@@ -19,7 +20,7 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 enum : int { TL_STORE = 0, TL_ADD = 1, TL_SWIGLU = 2 };
 
-#define TL_BM 128
+#define TL_BM 64
 #define TL_BN 128
 #define TL_BK 64
 #define TL_LD 72  // padded row length in bf16 elements (144 bytes)
@@ -46,6 +47,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     __shared__ int rows_a[TL_BM];
     __shared__ int rows_c[TL_BM];
     __shared__ int tile_info[2];
+    __shared__ int scan_waves[4];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     constexpr int FEATS = (EPI == TL_SWIGLU) ? 64 : 128;  // output features a workgroup covers
@@ -53,20 +55,33 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     const bf16_t* W = g.W;
     int row_begin, row_end;
     if (GROUPED) {
-        // which (expert, row tile) this workgroup has: experts in order, each with ceil(rows / 128) tiles
-        if (tid == 0) {
-            int left = blockIdx.y, found = -1, tile = 0;
-            for (int e = 0; e < g.n_groups; ++e) {
-                const int tiles = (g.group_offsets[e + 1] - g.group_offsets[e] + TL_BM - 1) / TL_BM;
-                if (left < tiles) {
-                    found = e;
-                    tile = left;
-                    break;
-                }
-                left -= tiles;
+        // which (expert, row tile) this workgroup has: experts in order, each with ceil(rows / 64) tiles
+        // found by all threads together: 256 experts a round, their tile counts scanned within waves and across them
+        if (tid == 0) tile_info[0] = -1;
+        int base = 0;
+        for (int e0 = 0; e0 < g.n_groups; e0 += 256) {
+            const int e = e0 + tid;
+            const int begin = e < g.n_groups ? g.group_offsets[e] : 0;
+            const int tiles = e < g.n_groups ? (g.group_offsets[e + 1] - begin + TL_BM - 1) / TL_BM : 0;
+            int incl = tiles;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int o = __shfl_up(incl, d, 64);
+                if (lane >= d) incl += o;
             }
-            tile_info[0] = found;
-            tile_info[1] = tile;
+            if (lane == 63) scan_waves[wave] = incl;
+            __syncthreads();
+            int before = base;
+            for (int w = 0; w < wave; ++w) before += scan_waves[w];
+            const int round_total = scan_waves[0] + scan_waves[1] + scan_waves[2] + scan_waves[3];
+            const int first = before + incl - tiles;
+            if ((int)blockIdx.y >= first && (int)blockIdx.y < first + tiles) {
+                tile_info[0] = e;
+                tile_info[1] = (int)blockIdx.y - first;
+            }
+            base += round_total;
+            __syncthreads();
+            if ((int)blockIdx.y < base) break;
         }
         __syncthreads();
         const int e = tile_info[0];
@@ -95,7 +110,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     }
     __syncthreads();
 
-    // global -> register staging: 1024 chunks of 16 bytes per tile, 4 per thread; chunk c: row c/8, k offset (c%8)*8
+    // global -> register staging in chunks of 16 bytes: W 1024 chunks (4 a thread), A 512 (2 a thread); chunk c: row c/8, k offset (c%8)*8
     const int K = g.K;
     const bf16_t* a_src[4];
     const bf16_t* w_src[4];
@@ -104,9 +119,13 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     for (int i = 0; i < 4; ++i) {
         const int c = tid + 256 * i;
         const int row = c >> 3, kc = (c & 7) * 8;
-        const int ra = rows_a[row];
-        a_ok[i] = ra >= 0;
-        a_src[i] = g.A + (size_t)(ra >= 0 ? ra : 0) * g.lda + kc;
+        a_ok[i] = false;
+        a_src[i] = g.A;
+        if (i < 2) {
+            const int ra = rows_a[row];
+            a_ok[i] = ra >= 0;
+            a_src[i] = g.A + (size_t)(ra >= 0 ? ra : 0) * g.lda + kc;
+        }
         int wr;
         if (EPI == TL_SWIGLU) {
             const int f = n0 + (row & 63);
@@ -125,7 +144,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         for (int i = 0; i < 4; ++i) {
             const int kc = ((tid + 256 * i) & 7) * 8;
             const bool in = k0 + kc < K;
-            a_reg[i] = (in && a_ok[i]) ? *reinterpret_cast<const u32x4_t*>(a_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
+            if (i < 2) a_reg[i] = (in && a_ok[i]) ? *reinterpret_cast<const u32x4_t*>(a_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
             w_reg[i] = (in && w_ok[i]) ? *reinterpret_cast<const u32x4_t*>(w_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
         }
     };
@@ -134,12 +153,12 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         for (int i = 0; i < 4; ++i) {
             const int c = tid + 256 * i;
             const int row = c >> 3, kc = (c & 7) * 8;
-            *reinterpret_cast<u32x4_t*>(&As[row * TL_LD + kc]) = a_reg[i];
+            if (i < 2) *reinterpret_cast<u32x4_t*>(&As[row * TL_LD + kc]) = a_reg[i];
             *reinterpret_cast<u32x4_t*>(&Ws[row * TL_LD + kc]) = w_reg[i];
         }
     };
 
-    // wave (wm, wn): rows 64*wm .. (4 tiles of 16 rows), features: 4 tiles of 16 weight rows
+    // wave (wm, wn): rows 32*wm .. (2 tiles of 16 rows), features: 4 tiles of 16 weight rows
     const int wm = wave >> 1, wn = wave & 1;
     const int lr = lane & 15, lk = (lane >> 4) * 8;
     int w_row[4];  // LDS rows of the wave's 4 feature tiles
@@ -150,11 +169,11 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         else
             w_row[f] = 64 * wn + 16 * f + lr;
     }
-    f32x4_t acc[4][4], total[SPLIT ? 4 : 1][SPLIT ? 4 : 1];
+    f32x4_t acc[4][2], total[SPLIT ? 4 : 1][SPLIT ? 2 : 1];
 #pragma unroll
     for (int f = 0; f < 4; ++f)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[f][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int t = 0; t < 2; ++t) acc[f][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
     const int steps_total = (K + 31) >> 5;
     const int per = (steps_total + g.ks - 1) / g.ks;   // 32-wide steps in a run
     int until_fold = per;                                // steps left in the current run
@@ -174,7 +193,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
 #pragma unroll
                     for (int f = 0; f < 4; ++f)
 #pragma unroll
-                        for (int t = 0; t < 4; ++t) {
+                        for (int t = 0; t < 2; ++t) {
                             if (first_run) total[f][t] = acc[f][t];
                             else total[f][t] = f32x4_t{total[f][t][0] + acc[f][t][0], total[f][t][1] + acc[f][t][1],
                                                        total[f][t][2] + acc[f][t][2], total[f][t][3] + acc[f][t][3]};
@@ -183,16 +202,16 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
                     first_run = false;
                     until_fold = per;
                 }
-                bf16x8_t wf[4], af[4];
+                bf16x8_t wf[4], af[2];
 #pragma unroll
                 for (int f = 0; f < 4; ++f) wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[w_row[f] * TL_LD + kk + lk]));
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    af[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[(64 * wm + 16 * t + lr) * TL_LD + kk + lk]));
+                for (int t = 0; t < 2; ++t)
+                    af[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[(32 * wm + 16 * t + lr) * TL_LD + kk + lk]));
 #pragma unroll
                 for (int f = 0; f < 4; ++f)
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[t], acc[f][t], 0, 0, 0);
+                    for (int t = 0; t < 2; ++t) acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[t], acc[f][t], 0, 0, 0);
                 --until_fold;
             }
         }
@@ -206,16 +225,16 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
 #pragma unroll
         for (int f = 0; f < 4; ++f)
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 2; ++t)
                 acc[f][t] = f32x4_t{total[f][t][0] + acc[f][t][0], total[f][t][1] + acc[f][t][1], total[f][t][2] + acc[f][t][2],
                                     total[f][t][3] + acc[f][t][3]};
     }
 
-    // acc[f][t][i]: feature (tile f) 4*(lane/16) + i, row 64*wm + 16*t + lane%16
+    // acc[f][t][i]: feature (tile f) 4*(lane/16) + i, row 32*wm + 16*t + lane%16
     const int fq = 4 * (lane >> 4);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        const int rc = rows_c[64 * wm + 16 * t + lr];
+    for (int t = 0; t < 2; ++t) {
+        const int rc = rows_c[32 * wm + 16 * t + lr];
         if (rc < 0) continue;
         TC* crow = (TC*)g.C + (size_t)rc * g.ldc;
         if (EPI == TL_SWIGLU) {
@@ -255,7 +274,7 @@ static void tile_launch(const TileArgs& g, dim3 grid, bool grouped, hipStream_t 
 }
 
 // A and W bfloat16, K a multiple of 8.  n_groups == 0: dense over M rows.  n_groups > 0: grouped over the n_pairs = M
-// rows of `list`; `max_tiles` bounds the (expert, row tile) pairs (at most min(groups, pairs) + pairs / 128).
+// rows of `list`; `max_tiles` bounds the (expert, row tile) pairs (at most min(groups, pairs) + pairs / 64).
 // ks: the runs K is cut into; the caller passes what the weight-streaming kernel uses for this N and K.
 extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                               int n_groups, int max_tiles, const int* group_offsets, const int* list, int a_div, long w_group_stride,

@@ -59,7 +59,7 @@ def _declare(h) -> None:
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
-        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
+        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, P, P, I, I, I, I, I, F, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
@@ -142,8 +142,9 @@ _KS_OVERRIDE = None   # set by tuning scripts only
 
 
 def _split_k(n_strips: int, K: int) -> int:
-    """Waves that share one 16-feature strip's K: enough strips*waves to fill the chip, at least 12 k-steps a wave.
-    A function of the product's shape only, so a row's bits do not depend on the batch."""
+    """Runs the products cut K into (waves that share one 16-feature strip in the weight-streaming kernel; run boundaries
+    in the tiled kernel): enough strips * runs to fill the chip, at least 12 steps of 32 a run.  A function of the
+    product's shape only, so a row's bits do not depend on the batch."""
     if _KS_OVERRIDE:
         return _KS_OVERRIDE
     ks = 1
@@ -204,7 +205,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
-                                    _split_k(-(-N // 16), K), G, min(G, n_pairs) + n_pairs // 128, _dev(offsets, "offsets", torch.int32, (G + 1,)),
+                                    _split_k(-(-N // 16), K), G, min(G, n_pairs) + n_pairs // 64, _dev(offsets, "offsets", torch.int32, (G + 1,)),
                                     _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
                "grouped_gemm_tile")
         return
@@ -243,10 +244,11 @@ class AttentionPlan:
     """Work items of the matrix-core attention kernel for one step's rows (they hold no positions, so a plan serves
     every step with the same rows per request) and the merge list of the items that were split over the context."""
 
-    def __init__(self, items, merges, n_slots, device):
+    def __init__(self, shared, items, merges, n_slots, device):
         import numpy as np
-        items = [i for i in items if i[6] < 0] + [i for i in items if i[6] >= 0]   # those that fold their segments first
+        self.n_shared = len(shared)          # prompt tiles, 4 to a workgroup that shares their keys
         self.n_direct = sum(1 for i in items if i[6] < 0)
+        items = shared + [i for i in items if i[6] < 0] + [i for i in items if i[6] >= 0]   # those that fold their segments first
         self.n_items = len(items)
         self.n_merges = len(merges)
         self.n_slots = n_slots
@@ -262,8 +264,9 @@ ATTENTION_SEGMENT = 128         # keys in a segment: the unit contexts are split
 def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, window: int = 0) -> AttentionPlan:
     """row_counts[i]: rows of entry i in the step (entries' rows are consecutive, in order); contexts[i]: tokens the
     entry holds after the step.  Single-row entries become items per KV head (columns = its query heads) that share out
-    the context's 128-key segments when there are few rows; longer entries become tiles of 16 rows of one head.
-    How the context is shared out changes no result: segments are folded in key order either way."""
+    the context's 128-key segments when there are few rows; longer entries become tiles of 16 rows of one head, 4 tiles
+    that read the same KV head to a workgroup.  How the context is shared out changes no result: segments are folded in
+    key order either way."""
     ratio = n_heads // n_kv_heads
     head_chunks = [(kvh * ratio + c0, min(16, ratio - c0)) for kvh in range(n_kv_heads) for c0 in range(0, ratio, 16)]
     single = [i for i, n in enumerate(row_counts) if n == 1]
@@ -280,18 +283,24 @@ def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, 
     plan = _PLAN_CACHE.get(key)
     if plan is not None:
         return plan
-    items, merges, slot = [], [], 0
+    shared, items, merges, slot = [], [], [], 0
     row0s, at = [], 0
     for n in row_counts:
         row0s.append(at)
         at += n
-    # tiles of long entries first, latest rows (longest key ranges) first
+    # tiles of long entries, latest rows (longest key ranges) first; a KV head's last workgroup is filled up with empty items
     for i, n in enumerate(row_counts):
         if n == 1:
             continue
-        for r0 in range(((n - 1) // 16) * 16, -1, -16):
-            for h in range(n_heads):
-                items.append([row0s[i] + r0, min(16, n - r0), h, 1, 0, 1, -1, 0])
+        per_head = []
+        for kvh in range(n_kv_heads):
+            tiles = [[row0s[i] + r0, min(16, n - r0), h, 1, 0, 1, -1, 0]
+                     for r0 in range(((n - 1) // 16) * 16, -1, -16) for h in range(kvh * ratio, (kvh + 1) * ratio)]
+            tiles += [[0, 0, 0, 1, 0, 1, -1, 0]] * (-len(tiles) % 4)
+            per_head.append(tiles)
+        for b in range(0, len(per_head[0]), 4):      # the KV heads' workgroups take turns, so long ranges start first
+            for tiles in per_head:
+                shared += tiles[b:b + 4]
     for i in single:
         for head0, nh in head_chunks:
             if n_splits == 1:
@@ -302,7 +311,7 @@ def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, 
             for sp in range(n_splits):
                 items.append([row0s[i], 1, head0, nh, sp, n_splits, slot, 0])
             slot += seg_cap
-    plan = AttentionPlan(items, merges, slot, device)
+    plan = AttentionPlan(shared, items, merges, slot, device)
     if len(_PLAN_CACHE) > 256:
         _PLAN_CACHE.clear()
     _PLAN_CACHE[key] = plan
@@ -334,7 +343,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 scratch = lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=q.device)
             part_o = scratch("attention.part_o", (plan.n_slots * 16, head_dim), torch.float32)
             part_ml = scratch("attention.part_ml", (plan.n_slots * 16, 2), torch.float32)
-        _check(lib().llmx_paged_attention_mfma(*common, _dev(plan.items, "items", torch.int32), plan.n_direct, plan.n_items - plan.n_direct,
+        _check(lib().llmx_paged_attention_mfma(*common, _dev(plan.items, "items", torch.int32), plan.n_shared, plan.n_direct,
+                                               plan.n_items - plan.n_shared - plan.n_direct,
                                                _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
                                                _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale), n_heads, n_kv_heads,
                                                head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention_mfma")
