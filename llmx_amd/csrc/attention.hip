@@ -61,9 +61,7 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
         float r = 1.0f;
         if (a.norm_mode == QKNORM_PROJECTION) {
             // every block of the row forms the same sum in the same order
-            float s = 0.0f;
-            for (int i = threadIdx.x; i < qw; i += 256) s = fmaf(row[i], row[i], s);
-            s = block_sum<4>(s, scratch);
+            const float s = block_sum<4>(strided_squares<256>(row, qw), scratch);
             r = 1.0f / sqrtf(s / (float)qw + a.eps);
         }
         const int per = (qw + a.q_slices - 1) / a.q_slices;
@@ -76,9 +74,7 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
     const float* krow = row + qw;
     float r = 1.0f;
     if (a.norm_mode == QKNORM_PROJECTION) {
-        float s = 0.0f;
-        for (int i = threadIdx.x; i < kw; i += 256) s = fmaf(krow[i], krow[i], s);
-        s = block_sum<4>(s, scratch);
+        const float s = block_sum<4>(strided_squares<256>(krow, kw), scratch);
         r = 1.0f / sqrtf(s / (float)kw + a.eps);
     }
     const int e = a.row_entry[t];

@@ -61,8 +61,7 @@ __device__ __forceinline__ void attention_step(const bf16x8_t (&kf)[2][(DT + 1) 
             sc[4 * u + i] = v;
             step_max = fmaxf(step_max, v);
         }
-    step_max = fmaxf(step_max, __shfl_xor(step_max, 16, 64));
-    step_max = fmaxf(step_max, __shfl_xor(step_max, 32, 64));
+    step_max = rows_max4(step_max);
     const float m_new = fmaxf(m, step_max);
     const float alpha = (MASKED && m_new == -INFINITY) ? 1.0f : __expf(m - m_new);   // m = -inf gives 0
     float step_sum = 0.0f;
@@ -72,8 +71,7 @@ __device__ __forceinline__ void attention_step(const bf16x8_t (&kf)[2][(DT + 1) 
         pw[i] = (MASKED && sc[i] == -INFINITY) ? 0.0f : __expf(sc[i] - m_new);
         step_sum += pw[i];
     }
-    step_sum += __shfl_xor(step_sum, 16, 64);
-    step_sum += __shfl_xor(step_sum, 32, 64);
+    step_sum = rows_sum4(step_sum);
     l = l * alpha + step_sum;
     m = m_new;
     bf16x8_t pf;

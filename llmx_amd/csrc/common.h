@@ -33,15 +33,95 @@ template <typename T> __device__ __forceinline__ float round_to(float v);
 template <> __device__ __forceinline__ float round_to<float>(float v) { return v; }
 template <> __device__ __forceinline__ float round_to<bf16_t>(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 
+// Lane exchange without LDS.  gfx950's row swaps give a lane the values of its partner rows (rows are 16 lanes):
+// rows_pair16: (even, odd) = the values that the even and the odd row of the lane's row pair hold in this column;
+// halves_pair32: (lo, hi) = the values of lane % 32 and lane % 32 + 32.  Both partners get the same (first, second), so
+// op(first, second) is the same bits on both.  The elements are copied out of the builtin's result before any cast.
+__device__ __forceinline__ void rows_pair16(uint32_t x, uint32_t& even, uint32_t& odd) {
+    const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    even = r0;
+    odd = r1;
+}
+__device__ __forceinline__ void halves_pair32(uint32_t x, uint32_t& lo, uint32_t& hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    const uint32_t r0 = r[0], r1 = r[1];
+    lo = r0;
+    hi = r1;
+}
+// The value of the lane `N` places round the lane's row of 16 (N = 8, 4, 2, 1): used as butterfly steps after which a
+// row's values repeat with period N, so that the rotation pairs the same lanes as lane ^ N would.
+template <int N>
+__device__ __forceinline__ uint32_t row_rotate(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x120 + N, 0xf, 0xf, false);
+}
+template <int N> __device__ __forceinline__ float row_rotate(float x) { return __uint_as_float(row_rotate<N>(__float_as_uint(x))); }
+
+// Sum and max over the 4 lanes l % 16, l % 16 + 16, +32, +48: (row0 + row1) + (row2 + row3).
+__device__ __forceinline__ float rows_sum4(float v) {
+    uint32_t a, b;
+    rows_pair16(__float_as_uint(v), a, b);
+    v = __uint_as_float(a) + __uint_as_float(b);
+    halves_pair32(__float_as_uint(v), a, b);
+    return __uint_as_float(a) + __uint_as_float(b);
+}
+__device__ __forceinline__ float rows_max4(float v) {
+    uint32_t a, b;
+    rows_pair16(__float_as_uint(v), a, b);
+    v = fmaxf(__uint_as_float(a), __uint_as_float(b));
+    halves_pair32(__float_as_uint(v), a, b);
+    return fmaxf(__uint_as_float(a), __uint_as_float(b));
+}
+
+// Butterfly over the wave: partners 32, 16, 8, 4, 2, 1 lanes apart, in this order; every lane ends with the same bits.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, LLMX_WAVE);
+    uint32_t a, b;
+    halves_pair32(__float_as_uint(v), a, b);
+    v = __uint_as_float(a) + __uint_as_float(b);
+    rows_pair16(__float_as_uint(v), a, b);
+    v = __uint_as_float(a) + __uint_as_float(b);
+    v += row_rotate<8>(v);
+    v += row_rotate<4>(v);
+    v += row_rotate<2>(v);
+    v += row_rotate<1>(v);
     return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, LLMX_WAVE));
+    uint32_t a, b;
+    halves_pair32(__float_as_uint(v), a, b);
+    v = fmaxf(__uint_as_float(a), __uint_as_float(b));
+    rows_pair16(__float_as_uint(v), a, b);
+    v = fmaxf(__uint_as_float(a), __uint_as_float(b));
+    v = fmaxf(v, row_rotate<8>(v));
+    v = fmaxf(v, row_rotate<4>(v));
+    v = fmaxf(v, row_rotate<2>(v));
+    v = fmaxf(v, row_rotate<1>(v));
     return v;
+}
+// The wave's best (largest value; among equals the lowest id): every lane ends with it.  Ids are distinct, so the
+// order of the comparisons does not matter.
+__device__ __forceinline__ void wave_best(float& best, int& at) {
+    auto take = [&](float ob, int oa) {
+        if (ob > best || (ob == best && oa < at)) {
+            best = ob;
+            at = oa;
+        }
+    };
+    take(row_rotate<8>(best), (int)row_rotate<8>((uint32_t)at));
+    take(row_rotate<4>(best), (int)row_rotate<4>((uint32_t)at));
+    take(row_rotate<2>(best), (int)row_rotate<2>((uint32_t)at));
+    take(row_rotate<1>(best), (int)row_rotate<1>((uint32_t)at));
+    uint32_t v0, v1, i0, i1;
+    rows_pair16(__float_as_uint(best), v0, v1);
+    rows_pair16((uint32_t)at, i0, i1);
+    best = __uint_as_float(v0);
+    at = (int)i0;
+    take(__uint_as_float(v1), (int)i1);
+    halves_pair32(__float_as_uint(best), v0, v1);
+    halves_pair32((uint32_t)at, i0, i1);
+    best = __uint_as_float(v0);
+    at = (int)i0;
+    take(__uint_as_float(v1), (int)i1);
 }
 __device__ __forceinline__ double wave_sum(double v) {
 #pragma unroll
@@ -61,6 +141,21 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 #pragma unroll
     for (int w = 1; w < NW; ++w) s += scratch[w];
     __syncthreads();
+    return s;
+}
+
+// The thread's share of a row's sum of squares: elements threadIdx.x, threadIdx.x + THREADS, ... added in this order
+// with fmaf; four loads are in flight at a time (an element past the end adds fmaf(0, 0, s) = s).
+template <int THREADS>
+__device__ __forceinline__ float strided_squares(const float* __restrict__ row, int n) {
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < n; i += 4 * THREADS) {
+        float v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = i + u * THREADS < n ? row[i + u * THREADS] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s = fmaf(v[u], v[u], s);
+    }
     return s;
 }
 

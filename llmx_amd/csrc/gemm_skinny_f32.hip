@@ -39,10 +39,12 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
         f32x4_t acc[MT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        for (int s = s_begin; s < s_end; s += 2) {
-            f32x4_t wf[2], af[2][MT];
+        // UN steps' loads are in flight together (few rows: the step is bound by latency, not by bytes)
+        constexpr int UN = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
+        for (int s = s_begin; s < s_end; s += UN) {
+            f32x4_t wf[UN], af[UN][MT];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < UN; ++u) {
                 const int k = (s + u) * 16 + kg * 4;
                 const bool in = (s + u) < s_end && k < K;   // K is a multiple of 4: a lane's 4 values are all in or all out
                 wf[u] = in ? *reinterpret_cast<const f32x4_t*>(wp + (size_t)(s + u) * 16) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
@@ -51,7 +53,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
                     af[u][t] = (in && a_in[t]) ? *reinterpret_cast<const f32x4_t*>(ap[t] + (size_t)(s + u) * 16) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
             }
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < UN; ++u)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
 #pragma unroll

@@ -63,15 +63,7 @@ __global__ void __launch_bounds__(64) route_topk_kernel(const float* __restrict_
                 at = e;
             }
         }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ob = __shfl_xor(best, o, 64);
-            const int oa = __shfl_xor(at, o, 64);
-            if (ob > best || (ob == best && oa < at)) {
-                best = ob;
-                at = oa;
-            }
-        }
+        wave_best(best, at);
         if (lane == 0) {
             ids[(size_t)r * k + j] = at;
             chosen[j] = s[at];
@@ -158,6 +150,7 @@ __global__ void __launch_bounds__(64) moe_place_kernel(const int* __restrict__ i
 #define ALIGN_SMALL_PAIRS 1024
 __device__ void align_in_block(const int* pair_expert, int n_pairs, int n_experts, int* cnt, int* offs, int* __restrict__ counts,
                                int* __restrict__ offsets, int* __restrict__ list, int* __restrict__ active, int* __restrict__ n_active) {
+    __shared__ int wave_total[16], wave_active[16];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     for (int e = wave; e < n_experts; e += 16) {
         int c = 0;
@@ -168,21 +161,38 @@ __device__ void align_in_block(const int* pair_expert, int n_pairs, int n_expert
         if (lane == 0) cnt[e] = c;
     }
     __syncthreads();
-    if (tid < n_experts) {
+    // exclusive scan of the counts (and of "has rows") over the experts: within each wave, then over the waves before it
+    {
         const int e = tid;
-        int before = 0, active_before = 0;
-        for (int i = 0; i < e; ++i) {
-            before += cnt[i];
-            active_before += cnt[i] > 0;
+        const int c = e < n_experts ? cnt[e] : 0;
+        int incl = c, incl_active = c > 0;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int o = __shfl_up(incl, d, 64), oa = __shfl_up(incl_active, d, 64);
+            if (lane >= d) {
+                incl += o;
+                incl_active += oa;
+            }
         }
-        const int c = cnt[e];
-        offs[e] = before;
-        counts[e] = c;
-        offsets[e] = before;
-        if (c > 0) active[active_before] = e;
-        if (e == n_experts - 1) {
-            offsets[n_experts] = before + c;
-            n_active[0] = active_before + (c > 0);
+        if (lane == 63) {
+            wave_total[wave] = incl;
+            wave_active[wave] = incl_active;
+        }
+        __syncthreads();
+        int before = incl - c, active_before = incl_active - (c > 0);
+        for (int w = 0; w < wave; ++w) {
+            before += wave_total[w];
+            active_before += wave_active[w];
+        }
+        if (e < n_experts) {
+            offs[e] = before;
+            counts[e] = c;
+            offsets[e] = before;
+            if (c > 0) active[active_before] = e;
+            if (e == n_experts - 1) {
+                offsets[n_experts] = before + c;
+                n_active[0] = active_before + (c > 0);
+            }
         }
     }
     __syncthreads();
@@ -274,18 +284,11 @@ __global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __r
                     best = b[i];
                     at = lane + 64 * i;
                 }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const float ob = __shfl_xor(best, o, 64);
-                const int oa = __shfl_xor(at, o, 64);
-                if (ob > best || (ob == best && oa < at)) {
-                    best = ob;
-                    at = oa;
-                }
-            }
+            wave_best(best, at);
+            at = __builtin_amdgcn_readfirstlane(at);
             const int slot = at >> 6;
             const float picked = slot == 0 ? s[0] : slot == 1 ? s[1] : slot == 2 ? s[2] : s[3];
-            const float score = __shfl(picked, at & 63, 64);
+            const float score = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(picked), at & 63));
             if (lane == (at & 63)) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
@@ -297,7 +300,7 @@ __global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __r
             }
         }
         float total = 0.0f;
-        for (int j = 0; j < k; ++j) total += __shfl(mine, j, 64);
+        for (int j = 0; j < k; ++j) total += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mine), j));
         if (lane < k) {
             ids[(size_t)r * k + lane] = mine_id;
             weights[(size_t)r * k + lane] = (normalize ? mine / total : mine) * scale;

@@ -31,12 +31,7 @@ __global__ void __launch_bounds__(RMS_THREADS) rmsnorm_kernel(const float* __res
     __shared__ float scratch[RMS_THREADS / 64];
     const int r = blockIdx.x;
     const float* row = x + (size_t)(pick ? pick[r] : r) * n;
-    float s = 0.0f;
-    for (int i = threadIdx.x; i < n; i += RMS_THREADS) {
-        const float v = row[i];
-        s = fmaf(v, v, s);
-    }
-    s = block_sum<RMS_THREADS / 64>(s, scratch);
+    const float s = block_sum<RMS_THREADS / 64>(strided_squares<RMS_THREADS>(row, n), scratch);
     const float scale = 1.0f / sqrtf(s / (float)n + eps);
     for (int i = threadIdx.x; i < n; i += RMS_THREADS) {
         const float y = row[i] * (scale * w[i]);
