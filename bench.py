@@ -112,6 +112,8 @@ def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch):
     if start < 1:
         raise SystemExit(f"bench: context {context} is shorter than the {steps + warmup} steps")
     rids = [f"b{batch}_{i}" for i in range(batch)]
+    torch.cuda.synchronize()
+    t_fill = time.perf_counter()
     for i, rid in enumerate(rids):
         engine.add_request(rid)
         if fill == "synthetic":
@@ -120,6 +122,8 @@ def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch):
             ids = lcg_ids(start, c.vocab_size, 100 + i)
             for s in range(0, start, PREFILL_TOKENS):
                 engine.step([StepEntry(rid, ids[s:s + PREFILL_TOKENS], [])])
+    torch.cuda.synchronize()
+    run_decode.fill_s = time.perf_counter() - t_fill
     last = [lcg_ids(1, c.vocab_size, 7 + i)[0] for i in range(batch)]
     out = sampler_out[:batch]
 
@@ -202,6 +206,7 @@ def main():
         print(json.dumps({"prefill": run_prefill(engine, cfg, sampler_out, torch)}))
         return
     dt, distinct = run_decode(engine, sampler_out, a.batch, context, a.steps, a.warmup, a.context_fill, torch)
+    fill_s = run_decode.fill_s
     ms_per_step = dt / a.steps * 1e3
     value = a.batch * a.steps / dt
     mean_context = context - a.steps / 2
@@ -226,6 +231,9 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "bytes_gb": round(need / 1e9, 2),
                      "distinct_experts_per_layer": round(distinct, 1)},
         "setup_s": round(setup_s, 1),
+        **({"context_fill": {"tokens": a.batch * (context - a.steps - a.warmup), "s": round(fill_s, 2),
+                             "tok_s": round(a.batch * (context - a.steps - a.warmup) / fill_s, 1), "portion": PREFILL_TOKENS}}
+           if a.context_fill == "prefill" else {}),
     }
 
     pts = {}

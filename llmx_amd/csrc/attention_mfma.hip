@@ -479,10 +479,20 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
 }
 
 // merge: one block per output (row, head).  merge item: {row, head, first_slot, column}.  The row's segments are folded
-// in key order with the formula the attention kernel uses for a tile's segments; thread d owns dim d.
+// in key order with the formula the attention kernel uses for a tile's segments.  The fold's weights depend on the
+// segments' maxima only, so they are formed for 512 segments at a time by all threads (a prefix maximum, then
+// fold_weights per segment); what is left of the chain is O = O * a + o * b per segment, with thread d owning dim d and
+// 32 segments' loads in flight.  Same operations on the same values as a sequential fold: the same bits.
+#define MERGE_CHUNK 512
+#define MERGE_DEPTH 32
+template <bool WIDE>   // WIDE: head_dim above 128, two dims a thread
 __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restrict__ merges, const int* __restrict__ pos,
                                                             const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                             bf16_t* __restrict__ out, int n_heads, int D, int window) {
+    __shared__ __attribute__((aligned(16))) float seg_a[MERGE_CHUNK], seg_b[MERGE_CHUNK], seg_l[MERGE_CHUNK];
+    __shared__ __attribute__((aligned(16))) int seg_code[MERGE_CHUNK];   // 0: empty segment, 1: the first one that is not (the state becomes it), 2: fold
+    __shared__ float wave_top[2];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int* mi = merges + (size_t)blockIdx.x * AM_ITEM_INTS;
     const int t = mi[0], h = mi[1], first = mi[2], c = mi[3];
     const int p = pos[t];
@@ -491,35 +501,105 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
     const float* base_o = part_o + ((size_t)first * 16 + c) * D;
     const float* base_ml = part_ml + ((size_t)first * 16 + c) * 2;
     const size_t stride_o = (size_t)16 * D, stride_ml = 32;
-    for (int d = threadIdx.x; d < D; d += 128) {
-        float M = -INFINITY, L = 0.0f, O = 0.0f;
-        for (int s0 = 0; s0 < n_seg; s0 += 8) {
-            float ov[8], mv[8], lv[8];
+    float M = -INFINITY, L = 0.0f;   // the same in every thread
+    float O[WIDE ? 2 : 1] = {};       // dims tid and tid + 128
+    // a round's values: segments first .. first + MERGE_DEPTH - 1 (one past the end is read from the last and never used)
+    const int d0 = tid < D ? tid : 0, d1 = tid + 128 < D ? tid + 128 : 0;
+    float ahead[WIDE ? 2 : 1][MERGE_DEPTH];
+    auto fetch = [&](int first_seg) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const bool in = s0 + u < n_seg;
-                ov[u] = in ? base_o[(size_t)(s0 + u) * stride_o + d] : 0.0f;
-                mv[u] = in ? base_ml[(size_t)(s0 + u) * stride_ml] : -INFINITY;
-                lv[u] = in ? base_ml[(size_t)(s0 + u) * stride_ml + 1] : 0.0f;
+        for (int u = 0; u < MERGE_DEPTH; ++u) {
+            const float* src = base_o + (size_t)min(first_seg + u, n_seg - 1) * stride_o;
+            ahead[0][u] = src[d0];
+            if constexpr (WIDE) ahead[1][u] = src[d1];
+        }
+    };
+    fetch(0);
+    for (int c0 = 0; c0 < n_seg; c0 += MERGE_CHUNK) {
+        // the thread's 4 segments of the chunk: maxima and sums
+        float mv[4], lv[4], before[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int sg = c0 + 4 * tid + u;
+            const bool in = sg < n_seg;
+            mv[u] = in ? base_ml[(size_t)sg * stride_ml] : -INFINITY;
+            lv[u] = in ? base_ml[(size_t)sg * stride_ml + 1] : 0.0f;
+        }
+        // the maximum of everything before each segment: earlier chunks, earlier threads, the thread's earlier segments
+        float mine = fmaxf(fmaxf(mv[0], mv[1]), fmaxf(mv[2], mv[3]));
+        float incl = mine;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const float o = __shfl_up(incl, d, 64);
+            if (lane >= d) incl = fmaxf(incl, o);
+        }
+        if (lane == 63) wave_top[wave] = incl;
+        float excl = __shfl_up(incl, 1, 64);
+        if (lane == 0) excl = -INFINITY;
+        __syncthreads();
+        if (wave == 1) excl = fmaxf(excl, wave_top[0]);
+        float run = fmaxf(M, excl);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            before[u] = run;
+            run = fmaxf(run, mv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int at = 4 * tid + u;
+            int code = 0;
+            float fa = 1.0f, fb = 0.0f;
+            if (mv[u] != -INFINITY) {
+                code = before[u] == -INFINITY ? 1 : 2;
+                if (code == 2) {
+                    float mn;
+                    fold_weights(before[u], mv[u], fa, fb, mn);
+                }
+            }
+            seg_code[at] = code;
+            seg_a[at] = fa;
+            seg_b[at] = fb;
+            seg_l[at] = lv[u];
+        }
+        M = fmaxf(M, fmaxf(wave_top[0], wave_top[1]));
+        __syncthreads();
+        const int n = min(MERGE_CHUNK, n_seg - c0);
+        for (int s0 = 0; s0 < n; s0 += MERGE_DEPTH) {
+            // the next round's values are asked for before this round's are folded
+            float ov[WIDE ? 2 : 1][MERGE_DEPTH];
+#pragma unroll
+            for (int u = 0; u < MERGE_DEPTH; ++u) {
+                ov[0][u] = ahead[0][u];
+                if constexpr (WIDE) ov[1][u] = ahead[1][u];
+            }
+            fetch(c0 + s0 + MERGE_DEPTH);
+            f32x4_t fa[MERGE_DEPTH / 4], fb[MERGE_DEPTH / 4], fl[MERGE_DEPTH / 4];
+            u32x4_t fc[MERGE_DEPTH / 4];
+#pragma unroll
+            for (int u = 0; u < MERGE_DEPTH / 4; ++u) {
+                fa[u] = *reinterpret_cast<const f32x4_t*>(&seg_a[s0 + 4 * u]);
+                fb[u] = *reinterpret_cast<const f32x4_t*>(&seg_b[s0 + 4 * u]);
+                fl[u] = *reinterpret_cast<const f32x4_t*>(&seg_l[s0 + 4 * u]);
+                fc[u] = *reinterpret_cast<const u32x4_t*>(&seg_code[s0 + 4 * u]);
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                if (mv[u] == -INFINITY) continue;
-                if (M == -INFINITY) {
-                    M = mv[u];
-                    L = lv[u];
-                    O = ov[u];
-                } else {
-                    float fa, fb, mn;
-                    fold_weights(M, mv[u], fa, fb, mn);
-                    L = L * fa + lv[u] * fb;
-                    O = O * fa + ov[u] * fb;
-                    M = mn;
+            for (int u = 0; u < MERGE_DEPTH; ++u) {
+                const uint32_t code = (s0 + u < n) ? fc[u / 4][u % 4] : 0u;
+                const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
+                const float l_fold = L * a + l * b, o0_fold = O[0] * a + ov[0][u] * b;
+                L = code == 2u ? l_fold : (code == 1u ? l : L);
+                O[0] = code == 2u ? o0_fold : (code == 1u ? ov[0][u] : O[0]);
+                if constexpr (WIDE) {
+                    const float o1_fold = O[1] * a + ov[1][u] * b;
+                    O[1] = code == 2u ? o1_fold : (code == 1u ? ov[1][u] : O[1]);
                 }
             }
         }
-        out[((size_t)t * n_heads + h) * D + d] = f32_to_bf16(O * (1.0f / L));
+        __syncthreads();
     }
+    const float inv = 1.0f / L;
+    if (tid < D) out[((size_t)t * n_heads + h) * D + tid] = f32_to_bf16(O[0] * inv);
+    if (WIDE && tid + 128 < D) out[((size_t)t * n_heads + h) * D + tid + 128] = f32_to_bf16(O[WIDE ? 1 : 0] * inv);
 }
 
 // `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 4: one workgroup each 4),
@@ -555,7 +635,11 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
         default: return -2;
     }
     if (n_merges > 0)
-        hipLaunchKernelGGL(attention_merge_kernel, dim3(n_merges), dim3(128), 0, stream, merges, pos, part_o, part_ml, (bf16_t*)out, n_heads, head_dim,
-                           window);
+        if (head_dim > 128)
+            hipLaunchKernelGGL(attention_merge_kernel<true>, dim3(n_merges), dim3(128), 0, stream, merges, pos, part_o, part_ml, (bf16_t*)out, n_heads,
+                               head_dim, window);
+        else
+            hipLaunchKernelGGL(attention_merge_kernel<false>, dim3(n_merges), dim3(128), 0, stream, merges, pos, part_o, part_ml, (bf16_t*)out, n_heads,
+                               head_dim, window);
     return LLMX_CHECK_LAUNCH();
 }

@@ -380,6 +380,47 @@ def test_attention_row_is_the_same_bits_alone_or_in_a_tile(L, Hq, Hkv, D, window
             assert torch.equal(alone[0], tile[r]), f"row {r} (context {ctx}, target {target}) differs from its bits in the tile"
 
 
+@pytest.mark.parametrize("L,Hq,Hkv,D", [(70000, 2, 1, 32), (66000, 4, 2, 160)])
+def test_attention_very_long_context(L, Hq, Hkv, D):
+    """A decoded row over more than 512 segments of keys (the merge works through them in several rounds): the same bits
+    whether the context is shared out or walked by one item per KV head, and the plain softmax's values."""
+    o = ops()
+    page = 16
+    n_pages = -(-L // page)
+    order = list(range(n_pages))
+    random.Random(L).shuffle(order)
+    table = torch.tensor([order], dtype=torch.int32, device=DEV)
+    k_cache = rnd(n_pages, Hkv, page, D, dtype=torch.bfloat16, scale=0.5)
+    v_cache = rnd(n_pages, Hkv, D, page, dtype=torch.bfloat16, seed=2)
+    q = rnd(1, Hq * D, dtype=torch.bfloat16, seed=3)
+    pos = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
+    ent = torch.zeros(1, dtype=torch.int32, device=DEV)
+    scale = 1.0 / math.sqrt(D)
+    outs = []
+    for target in (1, 100000):
+        saved = o.ATTENTION_TARGET_WAVES
+        o.ATTENTION_TARGET_WAVES = target
+        try:
+            plan = o.attention_plan([1], [L], Hq, Hkv, DEV)
+        finally:
+            o.ATTENTION_TARGET_WAVES = saved
+        assert (plan.n_merges > 0) == (target > 1)
+        out = torch.empty(1, Hq * D, dtype=torch.bfloat16, device=DEV)
+        o.paged_attention(q, k_cache, v_cache, pos, ent, table, out, scale, Hq, plan=plan)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1]), "shared out over items and walked by one item give different bits"
+    # keys and values in position order
+    order_t = torch.tensor(order, device=DEV)
+    keys = k_cache[order_t].permute(1, 0, 2, 3).reshape(Hkv, n_pages * page, D)[:, :L].double()
+    values = v_cache[order_t].permute(1, 0, 3, 2).reshape(Hkv, n_pages * page, D)[:, :L].double()
+    for h in range(Hq):
+        kv = h // (Hq // Hkv)
+        w = torch.softmax((keys[kv] @ q[0, h * D:(h + 1) * D].double()) * scale, dim=0)
+        want = w @ values[kv]
+        got = outs[1][0, h * D:(h + 1) * D].double()
+        assert (got - want).abs().max() <= 1.2e-2 * want.abs().max() + 2e-4
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_window(dtype):
     got, want = attention_case((90, 21), 4, 2, 32, 16, 8, dtype, window=17)
