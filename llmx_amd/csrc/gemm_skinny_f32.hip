@@ -12,6 +12,7 @@ struct SkinnyF32Args {
     const float* W;
     float* C;
     int M, N, K, lda, ldc, add;
+    long slice_stride;   // gridDim.z > 1: slice z of K's steps goes to C + z * slice_stride (the reader adds the slices in order)
 };
 
 template <int KS, int MT>
@@ -22,8 +23,11 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
     const int n0 = blockIdx.x * 16;
     const int K = g.K;
     const int steps_total = (K + 15) >> 4;
-    const int per = (steps_total + KS - 1) / KS;
-    const int s_begin = wave * per, s_end = min(steps_total, s_begin + per);
+    const int per_slice = (steps_total + gridDim.z - 1) / gridDim.z;
+    const int slice_begin = blockIdx.z * per_slice, slice_end = min(steps_total, slice_begin + per_slice);
+    const int per = (per_slice + KS - 1) / KS;
+    const int s_begin = min(slice_end, slice_begin + wave * per), s_end = min(slice_end, s_begin + per);
+    float* C = g.C + (size_t)blockIdx.z * g.slice_stride;
     const float* wp = g.W + (size_t)min(n0 + r, g.N - 1) * K + kg * 4;
 
     // blockIdx.y walks the rows in chunks of 16*MT, so many rows spread over the chip (each chunk reads the strip again, from L2)
@@ -78,7 +82,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
                 }
                 const int m = m0 + t * 16 + r;
                 if (m >= g.M) continue;
-                float* c = g.C + (size_t)m * g.ldc + n0 + 4 * kg;
+                float* c = C + (size_t)m * g.ldc + n0 + 4 * kg;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     if (n0 + 4 * kg + i >= g.N) continue;
@@ -90,15 +94,16 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
     }
 }
 
-// K a multiple of 4, rows 16-byte aligned.  ks: 1, 2, 4, 8 or 16.
+// K a multiple of 4, rows 16-byte aligned.  ks: 1, 2, 4, 8 or 16 waves share a strip's K.  slices > 1: K's steps are
+// cut into `slices` runs first, run z written to C + z * slice_stride (no add then); the caller adds the runs in order.
 extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, int M, int N, int K, int lda, int ldc, int add, int ks,
-                                    hipStream_t stream) {
+                                    int slices, long slice_stride, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    if (K % 4) return -2;
-    SkinnyF32Args g{A, W, C, M, N, K, lda, ldc, add};
+    if (K % 4 || slices < 1 || slices > 64 || (slices > 1 && add)) return -2;
+    SkinnyF32Args g{A, W, C, M, N, K, lda, ldc, add, slice_stride};
     int chunks = (M + 63) / 64;
     if (chunks > 1024) chunks = 1024;
-    const dim3 grid((N + 15) / 16, M <= 64 ? 1 : chunks);
+    const dim3 grid((N + 15) / 16, M <= 64 ? 1 : chunks, slices);
 #define SKF_LAUNCH(KS, MT) hipLaunchKernelGGL((gemm_skinny_f32_kernel<KS, MT>), grid, dim3(64 * KS), 0, stream, g)
 #define SKF_MT(KS) do { if (M <= 16) SKF_LAUNCH(KS, 1); else if (M <= 32) SKF_LAUNCH(KS, 2); else SKF_LAUNCH(KS, 4); } while (0)
     switch (ks) {

@@ -5,19 +5,40 @@ enum : int { SCORE_SIGMOID = 0, SCORE_SOFTMAX = 1 };
 
 #define ROUTE_MAX_EXPERTS 1024
 #define ROUTE_MAX_K 256
+#define ROUTE_MAX_SLICES 8
+
+// p[0] + p[stride] + ... (`slices` <= 8 terms, added in this order; the loads do not wait for each other)
+__device__ __forceinline__ float sum_slices(const float* __restrict__ p, int slices, long stride) {
+    float v[ROUTE_MAX_SLICES];
+#pragma unroll
+    for (int i = 0; i < ROUTE_MAX_SLICES; ++i) v[i] = i < slices ? p[(size_t)i * stride] : 0.0f;
+    float x = v[0];
+#pragma unroll
+    for (int i = 1; i < ROUTE_MAX_SLICES; ++i)
+        if (i < slices) x += v[i];
+    return x;
+}
 
 // One wave per row.  score s_e = sigmoid(z_e) (or softmax over the row); the pick key is b_e = s_e + bias_e; k times
 // the largest key not yet taken is picked, the lowest id on ties; the weight is the unbiased s_e, divided by the
 // picks' sum (added in pick order) when `normalize`, then times `scale`.  A row with a non-finite key gets ids -1 and
 // weights 0.  Ids and weights come out in pick order, best first.
-__global__ void __launch_bounds__(64) route_topk_kernel(const float* __restrict__ z, const float* __restrict__ bias, int* __restrict__ ids,
+// `parts` (optional): the logits arrive as `slices` partial sums [slices][rows][experts]; the row adds them in slice order
+// into z first.
+__global__ void __launch_bounds__(64) route_topk_kernel(float* __restrict__ z, const float* __restrict__ parts, int slices, long slice_stride,
+                                                       const float* __restrict__ bias, int* __restrict__ ids,
                                                        float* __restrict__ weights, int n_experts, int k, int score, int normalize,
                                                        float scale) {
     __shared__ float s[ROUTE_MAX_EXPERTS];
     __shared__ float b[ROUTE_MAX_EXPERTS];
     __shared__ float chosen[ROUTE_MAX_K];
     const int r = blockIdx.x, lane = threadIdx.x;
-    const float* row = z + (size_t)r * n_experts;
+    float* row = z + (size_t)r * n_experts;
+    if (parts) {
+        for (int e = lane; e < n_experts; e += 64) {   // the thread reads back only what it wrote
+            row[e] = sum_slices(parts + (size_t)r * n_experts + e, slices, slice_stride);
+        }
+    }
     float row_max = -INFINITY;
     if (score == SCORE_SOFTMAX) {
         for (int e = lane; e < n_experts; e += 64) row_max = fmaxf(row_max, row[e]);
@@ -79,11 +100,12 @@ __global__ void __launch_bounds__(64) route_topk_kernel(const float* __restrict_
     }
 }
 
-extern "C" int llmx_route_topk(const float* z, const float* bias, int* ids, float* weights, int rows, int n_experts, int k, int score,
-                               int normalize, float scale, hipStream_t stream) {
+extern "C" int llmx_route_topk(float* z, const float* parts, int slices, long slice_stride, const float* bias, int* ids, float* weights,
+                               int rows, int n_experts, int k, int score, int normalize, float scale, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (n_experts > ROUTE_MAX_EXPERTS || k > ROUTE_MAX_K || k > n_experts || k <= 0) return -2;
-    hipLaunchKernelGGL(route_topk_kernel, dim3(rows), dim3(64), 0, stream, z, bias, ids, weights, n_experts, k, score, normalize, scale);
+    if (n_experts > ROUTE_MAX_EXPERTS || k > ROUTE_MAX_K || k > n_experts || k <= 0 || (parts && (slices < 1 || slices > ROUTE_MAX_SLICES))) return -2;
+    hipLaunchKernelGGL(route_topk_kernel, dim3(rows), dim3(64), 0, stream, z, parts, slices, slice_stride, bias, ids, weights, n_experts, k, score,
+                       normalize, scale);
     return LLMX_CHECK_LAUNCH();
 }
 
@@ -144,22 +166,20 @@ __global__ void __launch_bounds__(64) moe_place_kernel(const int* __restrict__ i
     }
 }
 
-// Few pairs (a decode step): one workgroup of 16 waves does it all.  The pairs' experts sit in LDS; wave w owns experts
-// w, w+16, ...: it counts an expert's pairs with ballots over the pairs 64 at a time, the counts are scanned in expert
-// order, and the same ballots place the expert's pairs in increasing pair order.
+// Few pairs (a decode step): one workgroup of 1024 threads does it all.  The pairs' experts sit in LDS; thread p owns
+// pair p: the experts' counts come from LDS atomics (a count does not depend on their order), the offsets from a scan
+// over the experts, and a pair's place in its expert's run is the number of earlier pairs of that expert (counted by
+// the thread itself), so each expert's pairs stay in increasing pair order.
 #define ALIGN_SMALL_PAIRS 1024
 __device__ void align_in_block(const int* pair_expert, int n_pairs, int n_experts, int* cnt, int* offs, int* __restrict__ counts,
                                int* __restrict__ offsets, int* __restrict__ list, int* __restrict__ active, int* __restrict__ n_active) {
     __shared__ int wave_total[16], wave_active[16];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    for (int e = wave; e < n_experts; e += 16) {
-        int c = 0;
-        for (int p0 = 0; p0 < n_pairs; p0 += 64) {
-            const int p = p0 + lane;
-            c += __popcll(__ballot(p < n_pairs && pair_expert[p] == e));
-        }
-        if (lane == 0) cnt[e] = c;
-    }
+    if (tid < n_experts) cnt[tid] = 0;
+    __syncthreads();
+    int mine = tid < n_pairs ? pair_expert[tid] : -1;
+    if (mine >= n_experts) mine = -1;   // an id outside the experts belongs to no run
+    if (mine >= 0) atomicAdd(&cnt[mine], 1);
     __syncthreads();
     // exclusive scan of the counts (and of "has rows") over the experts: within each wave, then over the waves before it
     {
@@ -196,16 +216,10 @@ __device__ void align_in_block(const int* pair_expert, int n_pairs, int n_expert
         }
     }
     __syncthreads();
-    for (int e = wave; e < n_experts; e += 16) {
-        if (cnt[e] == 0) continue;
-        int at = offs[e];
-        for (int p0 = 0; p0 < n_pairs; p0 += 64) {
-            const int p = p0 + lane;
-            const bool mine = p < n_pairs && pair_expert[p] == e;
-            const unsigned long long mask = __ballot(mine);
-            if (mine) list[at + __popcll(mask & ((1ull << lane) - 1ull))] = p;
-            at += __popcll(mask);
-        }
+    if (mine >= 0) {
+        int rank = 0;
+        for (int q = 0; q < tid; ++q) rank += pair_expert[q] == mine;
+        list[offs[mine] + rank] = tid;
     }
 }
 
@@ -237,7 +251,8 @@ extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* c
 // A decode step's routing in one launch: top-k of every row (one wave a row, values in registers: at most 256 experts,
 // at most 64 picks), then the pairs grouped by expert as moe_align_small_kernel does.  Same formulas and the same
 // orders as route_topk_kernel, so the picks and weights are the same bits.
-__global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __restrict__ z, const float* __restrict__ bias,
+__global__ void __launch_bounds__(1024) route_topk_align_kernel(float* __restrict__ z, const float* __restrict__ parts, int slices,
+                                                               long slice_stride, const float* __restrict__ bias,
                                                                int* __restrict__ ids, float* __restrict__ weights, int rows, int n_experts,
                                                                int k, int normalize, float scale, int* __restrict__ counts,
                                                                int* __restrict__ offsets, int* __restrict__ list, int* __restrict__ active,
@@ -247,7 +262,7 @@ __global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __r
     __shared__ int offs[1024];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     for (int r = wave; r < rows; r += 16) {
-        const float* row = z + (size_t)r * n_experts;
+        float* row = z + (size_t)r * n_experts;
         float s[4], b[4];
         bool taken[4];
         int finite = 1;
@@ -258,7 +273,14 @@ __global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __r
             b[i] = -INFINITY;
             taken[i] = true;
             if (e < n_experts) {
-                s[i] = 1.0f / (1.0f + expf(-row[e]));
+                float x;
+                if (parts) {   // the slices' loads are in flight together; they are added in slice order
+                    x = sum_slices(parts + (size_t)r * n_experts + e, slices, slice_stride);
+                    row[e] = x;
+                } else {
+                    x = row[e];
+                }
+                s[i] = 1.0f / (1.0f + expf(-x));
                 b[i] = bias ? s[i] + bias[e] : s[i];
                 taken[i] = false;
                 if (!isfinite(b[i])) finite = 0;
@@ -312,12 +334,14 @@ __global__ void __launch_bounds__(1024) route_topk_align_kernel(const float* __r
 }
 
 // Sigmoid scores only; at most 16 rows (a wave each), rows * k <= 1024, at most 256 experts and 64 picks.  Returns -2 otherwise.
-extern "C" int llmx_route_topk_align(const float* z, const float* bias, int* ids, float* weights, int rows, int n_experts, int k,
-                                     int normalize, float scale, int* counts, int* offsets, int* list, int* active, int* n_active,
-                                     hipStream_t stream) {
+extern "C" int llmx_route_topk_align(float* z, const float* parts, int slices, long slice_stride, const float* bias, int* ids, float* weights,
+                                     int rows, int n_experts, int k, int normalize, float scale, int* counts, int* offsets, int* list,
+                                     int* active, int* n_active, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (rows > 16 || rows * k > ALIGN_SMALL_PAIRS || n_experts > 256 || k > 64 || k > n_experts || k <= 0) return -2;
-    hipLaunchKernelGGL(route_topk_align_kernel, dim3(1), dim3(1024), 0, stream, z, bias, ids, weights, rows, n_experts, k, normalize, scale,
+    if (parts && (slices < 1 || slices > ROUTE_MAX_SLICES)) return -2;
+    hipLaunchKernelGGL(route_topk_align_kernel, dim3(1), dim3(1024), 0, stream, z, parts, slices, slice_stride, bias, ids, weights, rows, n_experts, k,
+                       normalize, scale,
                        counts, offsets, list, active, n_active);
     return LLMX_CHECK_LAUNCH();
 }

@@ -60,12 +60,12 @@ def _declare(h) -> None:
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
-        "llmx_route_topk": [P, P, P, P, I, I, I, I, I, F, P],
+        "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P],
-        "llmx_route_topk_align": [P, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
+        "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
         "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
-        "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, P],
+        "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P],
         "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
@@ -353,12 +353,22 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                               head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention")
 
 
+def _parts_args(z: torch.Tensor, parts: Optional[torch.Tensor]):
+    if parts is None:
+        return None, 1, 0
+    if parts.dim() != 3 or tuple(parts.shape[1:]) != tuple(z.shape):
+        raise KernelError(f"router partial sums {tuple(parts.shape)} do not fit logits {tuple(z.shape)}")
+    return _dev(parts, "parts", torch.float32), parts.shape[0], z.numel()
+
+
 def route_topk(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
-               normalize: bool, scale: float) -> None:
+               normalize: bool, scale: float, parts: Optional[torch.Tensor] = None) -> None:
+    """`parts` [slices, rows, experts]: the logits arrive as partial sums (gemm_f32's `parts`); they are added in slice
+    order into z first."""
     rows, n_experts = z.shape
     if n_experts > 1024 or k > 256 or k > n_experts:
         raise KernelError(f"route_topk takes at most 1024 experts and 256 picks, not {n_experts} and {k}")
-    _check(lib().llmx_route_topk(_dev(z, "z", torch.float32), _dev(bias, "bias", torch.float32, (n_experts,)),
+    _check(lib().llmx_route_topk(_dev(z, "z", torch.float32), *_parts_args(z, parts), _dev(bias, "bias", torch.float32, (n_experts,)),
                                  _dev(ids, "ids", torch.int32, (rows, k)), _dev(weights, "weights", torch.float32, (rows, k)),
                                  rows, n_experts, k, score, 1 if normalize else 0, float(scale), _stream()), "route_topk")
 
@@ -376,19 +386,20 @@ def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: 
 
 def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
                      normalize: bool, scale: float, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
-                     active: torch.Tensor, n_active: torch.Tensor) -> None:
+                     active: torch.Tensor, n_active: torch.Tensor, parts: Optional[torch.Tensor] = None) -> None:
     """route_topk followed by moe_align; a step of at most 16 rows (sigmoid scores, at most 256 experts and 64 picks) does
     both in one launch, with the same bits."""
     rows, n_experts = z.shape
     if score == SCORE_SIGMOID and rows <= 16 and rows * k <= 1024 and n_experts <= 256 and k <= 64:
         _check(lib().llmx_route_topk_align(
-            _dev(z, "z", torch.float32), _dev(bias, "bias", torch.float32, (n_experts,)), _dev(ids, "ids", torch.int32, (rows, k)),
+            _dev(z, "z", torch.float32), *_parts_args(z, parts), _dev(bias, "bias", torch.float32, (n_experts,)),
+            _dev(ids, "ids", torch.int32, (rows, k)),
             _dev(weights, "weights", torch.float32, (rows, k)), rows, n_experts, k, 1 if normalize else 0, float(scale),
             _dev(counts, "counts", torch.int32, (n_experts,)), _dev(offsets, "offsets", torch.int32, (n_experts + 1,)),
             _dev(pairs, "pairs", torch.int32, (rows * k,)), _dev(active, "active", torch.int32, (n_experts,)),
             _dev(n_active, "n_active", torch.int32, (1,)), _stream()), "route_topk_align")
         return
-    route_topk(z, bias, ids, weights, k, score, normalize, scale)
+    route_topk(z, bias, ids, weights, k, score, normalize, scale, parts)
     moe_align(ids, n_experts, counts, offsets, pairs, active, n_active)
 
 
@@ -430,22 +441,43 @@ def argmax_rows(scores: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Te
                                   _dev(out, "out", torch.int32, (rows,)), _dev(partial, "partial"), rows, n, _stream()), "argmax_rows")
 
 
-def gemm_f32(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, add: bool = False) -> None:
+def gemm_f32_slices(N: int, K: int) -> int:
+    """Runs that gemm_f32 cuts K into when its caller takes partial sums (a function of the weight's shape only)."""
+    if K % 4:
+        return 1
+    n_strips, steps, s = -(-N // 16), K // 16, 1
+    while s < 8 and n_strips * s < 128 and steps // (s * 2) >= 12:
+        s *= 2
+    return s
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, add: bool = False, parts: Optional[torch.Tensor] = None) -> None:
     """c[M,N] (+)= a[M,K] @ w[N,K]^T, everything float32, on the float32 matrix instruction (the router's product).
-    A row's bits depend on the shape of w only.  K a multiple of 4; otherwise the universal kernel runs."""
+    A row's bits depend on the shape of w only.  K a multiple of 4; otherwise the universal kernel runs.
+    `parts` [gemm_f32_slices(N, K), M, N] with more than one slice: K's runs are written there instead of c, spread over
+    that many more workgroups, and the reader (route_topk) adds them in order."""
     M, K = a.shape
     N = w.shape[0]
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm_f32 shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
     if K % 4:
+        if parts is not None:
+            raise KernelError("gemm_f32: partial sums need K to be a multiple of 4")
         gemm(a, w, c, EPI_ADD if add else EPI_STORE, force_generic=True)
         return
+    slices = 1
+    if parts is not None:
+        slices = parts.shape[0]
+        if tuple(parts.shape) != (gemm_f32_slices(N, K), M, N) or add:
+            raise KernelError(f"gemm_f32: partial sums {tuple(parts.shape)} for {(M, N)} with add={add}")
     ks = 1
     n_strips = -(-N // 16)
-    while ks < 16 and n_strips * ks < 1024 and (K // 16) // (ks * 2) >= 8:   # from w's shape only: a row's bits must not depend on M
+    steps = (K // 16) // slices
+    while ks < 16 and n_strips * slices * ks < 1024 and steps // (ks * 2) >= (8 if slices == 1 else 3):   # from w's shape only
         ks *= 2
-    _check(lib().llmx_gemm_skinny_f32(_dev(a, "a", torch.float32), _dev(w, "w", torch.float32), _dev(c, "c", torch.float32), M, N, K, K, N,
-                                      1 if add else 0, ks, _stream()), "gemm_f32")
+    target = parts if parts is not None else c
+    _check(lib().llmx_gemm_skinny_f32(_dev(a, "a", torch.float32), _dev(w, "w", torch.float32), _dev(target, "c", torch.float32), M, N, K, K, N,
+                                      1 if add else 0, ks, slices, M * N, _stream()), "gemm_f32")
 
 
 def sample_all(scores: torch.Tensor, temp: torch.Tensor, unit: torch.Tensor, out: torch.Tensor, min_p: Optional[torch.Tensor] = None,

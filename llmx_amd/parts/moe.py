@@ -79,7 +79,9 @@ class RoutedExperts(FeedForward):
     def forward(self, step, h, out, accumulate, h32=None):
         T, X, k = step.rows, self.experts, self.top_k
         z = step.buf("experts.router_logits", (T, X), torch.float32)
-        ops.gemm_f32(h32, self.w_router, z)
+        slices = ops.gemm_f32_slices(X, h32.shape[1])
+        parts = step.buf("experts.router_parts", (slices, T, X), torch.float32) if slices > 1 else None
+        ops.gemm_f32(h32, self.w_router, z, parts=parts)
         ids = step.buf("experts.ids", (T, k), torch.int32)
         weights = step.buf("experts.weights", (T, k), torch.float32)
         counts = step.buf("experts.counts", (X,), torch.int32)
@@ -87,7 +89,8 @@ class RoutedExperts(FeedForward):
         pairs = step.buf("experts.pairs", (T * k,), torch.int32)
         active = step.buf("experts.active", (X,), torch.int32)
         n_active = step.buf("experts.n_active", (1,), torch.int32)
-        ops.route_topk_align(z, self.bias, ids, weights, k, self.score, self.normalize, self.scale, counts, offsets, pairs, active, n_active)
+        ops.route_topk_align(z, self.bias, ids, weights, k, self.score, self.normalize, self.scale, counts, offsets, pairs, active, n_active,
+                             parts=parts)
         step.observe("routing", logits=z, ids=ids, weights=weights)
         act = step.buf("experts.act", (T * k, self.intermediate), step.act_dtype)
         ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T)

@@ -527,6 +527,47 @@ def test_fused_route_and_align_equals_the_two_kernels(T, X, k):
             assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("M,N,K,k", [(1, 256, 3072, 8), (8, 256, 3072, 8), (64, 256, 3072, 8), (300, 256, 3072, 8), (5, 64, 1024, 3)])
+def test_router_logits_as_partial_sums(M, N, K, k):
+    """The router's product spread over more workgroups: K's runs are written as partial sums and the routing kernels add
+    them in run order.  The logits they leave are that sum exactly, the picks are those of routing the summed logits, and
+    a row's bits do not depend on the batch."""
+    o = ops()
+    slices = o.gemm_f32_slices(N, K)
+    assert slices > 1
+    a = rnd(M, K)
+    w = rnd(N, K, seed=1)
+    parts = torch.full((slices, M, N), float("nan"), device=DEV)
+    z = torch.full((M, N), float("nan"), device=DEV)
+    o.gemm_f32(a, w, z, parts=parts)
+    assert torch.isnan(z).all(), "with partial sums asked for the product must leave the logits alone"
+    want = parts[0].clone()
+    for sl in range(1, slices):
+        want = want + parts[sl]
+    ref = a.double().cpu() @ w.double().cpu().T
+    assert (want.double().cpu() - ref).abs().max() <= 2e-6 * math.sqrt(K) * ref.abs().max()
+    bias = 0.1 * rnd(N, seed=2)
+    mk = lambda shape, dt: torch.full(shape, -9, dtype=dt, device=DEV)
+    ids0, w0 = mk((M, k), torch.int32), mk((M, k), torch.float32)
+    o.route_topk(want.clone(), bias, ids0, w0, k, o.SCORE_SIGMOID, True, 2.0)
+    for fused in (True, False):
+        if fused and M > 16:
+            continue
+        z = torch.full((M, N), float("nan"), device=DEV)
+        ids, wt = mk((M, k), torch.int32), mk((M, k), torch.float32)
+        if fused:
+            counts, offsets, pairs = mk((N,), torch.int32), mk((N + 1,), torch.int32), mk((M * k,), torch.int32)
+            o.route_topk_align(z, bias, ids, wt, k, o.SCORE_SIGMOID, True, 2.0, counts, offsets, pairs, mk((N,), torch.int32), mk((1,), torch.int32),
+                               parts=parts)
+        else:
+            o.route_topk(z, bias, ids, wt, k, o.SCORE_SIGMOID, True, 2.0, parts=parts)
+        assert torch.equal(z, want) and torch.equal(ids, ids0) and torch.equal(wt, w0)
+    # the last row alone
+    p1 = torch.empty(slices, 1, N, device=DEV)
+    o.gemm_f32(a[M - 1:M].contiguous(), w, torch.empty(1, N, device=DEV), parts=p1)
+    assert torch.equal(p1[:, 0], parts[:, M - 1])
+
+
 def test_route_matches_plain_and_invariants():
     o = ops()
     T, X, k = 13, 40, 5
