@@ -80,7 +80,13 @@ def _declare(h) -> None:
         fn.restype = c_int
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The current HIP stream's handle (asked for at every launch, so through torch's raw accessor where it has one)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
