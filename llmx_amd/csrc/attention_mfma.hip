@@ -1,19 +1,20 @@
 // Paged attention on the matrix cores (bfloat16 cache, pages of a multiple of 16 tokens, head_dim a multiple of 16).
 //
-// One wave owns a work item: up to 16 columns that share one request and one KV head, over a range of keys.
-// A column is a (row, query head) pair: for decoding the 16 columns are the query heads that read one KV head
-// (each K/V byte is read once for all of them), for a prompt portion they are 16 consecutive rows of one head.
-// Keys are walked 32 at a time (two tiles of 16):
-//   scores^T[key][col] = K_tile[16 keys x D] . Q^T[D x 16 cols]        (A = K straight from the page, B = Q in registers)
-//   online softmax per column in float32 (columns live in lanes l%16, keys in lane groups l/16 and registers)
-//   out^T[dim][col]  += V^T_tile[16 dims x 32 keys] . P^T[32 keys x 16 cols]
-// The value pages are stored transposed ([dim][token]) so that V^T's rows are contiguous, and the 32 keys of a step are
-// assigned to the product's k-slots in the order the score accumulators already hold them: no data moves between lanes.
-// Keys are grouped in fixed segments of 128 (absolute positions): each segment gets its own online softmax from scratch,
-// and the segments' (max, sum, out) are folded in key order with one formula (fold_segment).  A long context of a
-// decoding row is split over several items that write their segments' partials, which a second kernel folds; a prompt
-// tile folds its segments in registers.  Either way a row's result is the same bits: it does not depend on how many
-// rows the step holds or on how the context was split.
+// A column is a (row, query head) pair; a wave works on a tile of up to 16 columns that share one request and one KV
+// head: for decoding the columns are the query heads that read one KV head (each K/V byte is read once for all of
+// them), for a prompt portion they are 16 consecutive rows of one head.
+//
+// Keys are grouped in fixed segments of 128 absolute positions.  Per column and segment:
+//   scores^T[key][col] = K_tile[16 keys x D] . Q^T[D x 16 cols]   (A = K, B = Q in registers), 8 tiles of 16 keys
+//   m = max of the segment's scores that count, p = exp(score - m), l = sum p       (float32, a fixed order)
+//   o^T[dim][col] = V^T[16 dims x 32 keys] . P^T[32 keys x 16 cols], 4 chunks of 32 keys added in key order
+// The value pages are stored transposed ([dim][token]) so that V^T's rows are contiguous, and a chunk's 32 keys are
+// assigned to the product's k-slots in the order the score accumulators hold them: no data moves between lanes
+// except the softmax's reductions over the 4 lanes of a column.
+// The segments' (m, l, o) are folded in key order with one formula (fold_segment).  A long context of a decoding row is
+// shared out over several items that write their segments' (m, l, o), which a second kernel folds; a prompt tile folds
+// its segments in registers.  Every form calls the same functions with the same values, so a column's result is the
+// same bits whatever the step holds and however the context was shared out.
 #include "common.h"
 #include <type_traits>
 
@@ -34,54 +35,62 @@ __device__ __forceinline__ void fold_weights(float M, float m, float& a, float& 
     b = __expf(m - Mn);
 }
 
-// One step of a column tile: 32 keys against the tile's 16 columns.  kf: the keys (two tiles of 16), vf: the values
-// transposed, qf: the columns' queries; ok: bit 4u+i says whether key 16u + 4g + i counts for this lane's column
-// (MASKED false: all 32 keys count for every column, and the selects fall away; the sums are the same).
-// Updates the running segment (o, m, l).  Every form of the kernel calls this, so a column's bits do not depend on the form.
-template <int DT, bool MASKED>
-__device__ __forceinline__ void attention_step(const bf16x8_t (&kf)[2][(DT + 1) / 2], const bf16x8_t (&vf)[DT], const bf16x8_t (&qf)[(DT + 1) / 2],
-                                               unsigned ok, float scale, f32x4_t (&o)[DT], float& m, float& l) {
+// Whether a lane's 8 dims 32s + 8g .. of fragment s lie inside the head (always, unless head_dim is an odd multiple of 16
+// and s is the last fragment).
+template <int DT>
+__device__ __forceinline__ bool frag_in(int s, int g) {
+    if (DT % 2 == 0 || s < DT / 2) return true;
+    return g < 2;
+}
+
+// Scores of one chunk (32 keys, two tiles of 16) against the tile's columns.  kf: the keys, qf: the columns' queries.
+// Lane (column c = l % 16, group g = l / 16) gets keys 16u + 4g + i of the chunk in s[u][i].
+template <int DT>
+__device__ __forceinline__ void chunk_scores(const bf16x8_t (&kf)[2][(DT + 1) / 2], const bf16x8_t (&qf)[(DT + 1) / 2], f32x4_t& s0, f32x4_t& s1) {
     constexpr int QS = (DT + 1) / 2;
-    // scores^T: lane holds keys 4g + i of each tile for its column
-    f32x4_t s_acc[2];
+    s0 = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    s1 = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        s_acc[u] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int s = 0; s < QS; ++s) s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][s], qf[s], s_acc[u], 0, 0, 0);
+    for (int s = 0; s < QS; ++s) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][s], qf[s], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][s], qf[s], s1, 0, 0, 0);
     }
-    // online softmax of the column over the step's 32 keys
-    float sc[8];
-    float step_max = -INFINITY;
+}
+
+// Softmax of a column over one segment.  s[2v + u][i]: the score of key 32v + 16u + 4g + i; ok bit 8v + 4u + i says
+// whether that key counts for the lane's column (MASKED false: all 128 count for every column and the selects fall
+// away; the sums are the same).  Gives the segment's maximum m, its sum l and the weights as the value product's
+// operands pf[v] (chunk v).  A column without a key that counts gets m = -inf, l = 0, weights 0.
+template <bool MASKED>
+__device__ __forceinline__ void segment_softmax(const f32x4_t (&s)[8], uint32_t ok, float scale, float& m, float& l, bf16x8_t (&pf)[4]) {
+    // the maximum of the raw scores (scale > 0 keeps the order); p = 2^(score * k - top * k), k = scale * log2(e), as one
+    // fused multiply-add and one exponential a score
+    float top = -INFINITY;
 #pragma unroll
-    for (int u = 0; u < 2; ++u)
+    for (int t = 0; t < 8; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float v = (!MASKED || ((ok >> (4 * u + i)) & 1u)) ? s_acc[u][i] * scale : -INFINITY;
-            sc[4 * u + i] = v;
-            step_max = fmaxf(step_max, v);
-        }
-    step_max = rows_max4(step_max);
-    const float m_new = fmaxf(m, step_max);
-    const float alpha = (MASKED && m_new == -INFINITY) ? 1.0f : __expf(m - m_new);   // m = -inf gives 0
-    float step_sum = 0.0f;
-    float pw[8];
+        for (int i = 0; i < 4; ++i)
+            if (!MASKED || ((ok >> (4 * t + i)) & 1u)) top = fmaxf(top, s[t][i]);
+    top = rows_max4(top);
+    m = top * scale;
+    const float k = scale * 1.44269504088896340736f;
+    const float shift = -(top * k);
+    float sum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        pw[i] = (MASKED && sc[i] == -INFINITY) ? 0.0f : __expf(sc[i] - m_new);
-        step_sum += pw[i];
+    for (int j = 0; j < 32; ++j) {
+        const bool counts = !MASKED || (((ok >> j) & 1u) && top != -INFINITY);
+        const float p = counts ? __builtin_amdgcn_exp2f(fmaf(s[j / 4][j % 4], k, shift)) : 0.0f;
+        sum += p;
+        pf[j / 8][j % 8] = (__bf16)p;
     }
-    step_sum = rows_sum4(step_sum);
-    l = l * alpha + step_sum;
-    m = m_new;
-    bf16x8_t pf;
+    l = rows_sum4(sum);
+}
+
+// o^T += V^T[dims x 32 keys] . P^T for one chunk
+template <int DT>
+__device__ __forceinline__ void chunk_values(const bf16x8_t (&vf)[DT], const bf16x8_t& pf, f32x4_t (&o)[DT]) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) pf[i] = (__bf16)pw[i];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        o[dt] = f32x4_t{o[dt][0] * alpha, o[dt][1] * alpha, o[dt][2] * alpha, o[dt][3] * alpha};
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
-    }
+    for (int dt = 0; dt < DT; ++dt) o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, o[dt], 0, 0, 0);
 }
 
 // A finished segment (o, m, l) folded into the segments before it (o_tot, m_tot, l_tot); an empty segment changes nothing.
@@ -105,6 +114,33 @@ __device__ __forceinline__ void fold_segment(const f32x4_t (&o)[DT], float m, fl
     m_tot = mn;
 }
 
+// The keys of a segment that count for a lane's column: key in [lo_col, p_col], below key_end; bit 8v + 4u + i for key
+// seg0 + 32v + 16u + 4g + i.
+__device__ __forceinline__ uint32_t segment_mask(int seg0, int g, bool col_ok, int lo_col, int p_col, int key_end) {
+    uint32_t ok = 0u;
+    if (!col_ok) return ok;
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = seg0 + 16 * t + 4 * g + i;
+            if (key <= p_col && key >= lo_col && key < key_end) ok |= 1u << (4 * t + i);
+        }
+    return ok;
+}
+
+// the column's output row: lane holds dims 16dt + 4g + i
+template <int DT>
+__device__ __forceinline__ void store_output(bf16_t* dst, int g, const f32x4_t (&o_tot)[DT], float l_tot) {
+    const float inv = 1.0f / l_tot;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const u32x2_t packed = {(uint32_t)f32_to_bf16(o_tot[dt][0] * inv) | ((uint32_t)f32_to_bf16(o_tot[dt][1] * inv) << 16),
+                                (uint32_t)f32_to_bf16(o_tot[dt][2] * inv) | ((uint32_t)f32_to_bf16(o_tot[dt][3] * inv) << 16)};
+        *reinterpret_cast<u32x2_t*>(dst + 16 * dt + 4 * g) = packed;
+    }
+}
+
 // item: {row0, n_rows, head0, n_heads, split, n_splits, slot, unused}
 //   columns c = 0 .. n_rows*n_heads-1: row = row0 + c / n_heads, head = head0 + c % n_heads
 //   slot < 0: the item folds its segments itself and writes the final output; otherwise segment s of the row (counted
@@ -119,20 +155,27 @@ struct AttnMfmaArgs {
     const int* items;
     bf16_t* out;            // [T, n_heads * D]
     float* part_o;          // [slots * 16, D]
-    float* part_ml;         // [slots * 16, 2]: running max, running sum
+    float* part_ml;         // [slots * 16, 2]: segment max, segment sum
     float scale;
     int n_items, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
 };
 
-// DT = head_dim / 16 rounded up.  PARTIAL: the items write their segments (slot >= 0); otherwise they fold them (slot < 0).
+// One wave per item, keys and values straight from the pages into the products' operands: the form for decoding rows,
+// where the cache is read once and nothing is shared between waves.  A chunk's loads are on their way while the chunk
+// before it is multiplied; the first values of a segment are asked for before its softmax.
+// DT = head_dim / 16.  PARTIAL: the items write their segments (slot >= 0); otherwise they fold them (slot < 0).
 template <int DT, bool PARTIAL>
-__global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs a) {
+__global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_attention_mfma_kernel(AttnMfmaArgs a) {
+    constexpr int QS = (DT + 1) / 2;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int item_no = blockIdx.x * 4 + wave;
     if (item_no >= a.n_items) return;
-    const int* it = a.items + (size_t)item_no * AM_ITEM_INTS;
-    const int row0 = it[0], n_rows = it[1], head0 = it[2], n_heads_item = it[3], split = it[4], n_splits = it[5], slot = it[6];
-    const int D = a.head_dim, bt = a.page_tokens, Hkv = a.n_kv_heads;
+    const int* it = a.items + (size_t)item_no * AM_ITEM_INTS;   // the same for the whole wave
+    const int row0 = __builtin_amdgcn_readfirstlane(it[0]), n_rows = __builtin_amdgcn_readfirstlane(it[1]);
+    const int head0 = __builtin_amdgcn_readfirstlane(it[2]), n_heads_item = __builtin_amdgcn_readfirstlane(it[3]);
+    const int split = __builtin_amdgcn_readfirstlane(it[4]), n_splits = __builtin_amdgcn_readfirstlane(it[5]);
+    const int slot = __builtin_amdgcn_readfirstlane(it[6]);
+    const int D = 16 * DT, bt = a.page_tokens, Hkv = a.n_kv_heads;
     const int c = lane & 15, g = lane >> 4;
     const int n_cols = n_rows * n_heads_item;
     const bool col_ok = c < n_cols;
@@ -140,8 +183,8 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
     const int h = head0 + (col_ok ? c % n_heads_item : 0);
     const int kvh = head0 / (a.n_heads / Hkv);
     const int p_col = a.pos[t];
-    const int p_first = a.pos[row0], p_last = a.pos[row0 + n_rows - 1];
-    const int* table = a.tables + (size_t)a.row_entry[row0] * a.max_blocks;
+    const int p_first = __builtin_amdgcn_readfirstlane(a.pos[row0]), p_last = __builtin_amdgcn_readfirstlane(a.pos[row0 + n_rows - 1]);
+    const int* table = a.tables + (size_t)__builtin_amdgcn_readfirstlane(a.row_entry[row0]) * a.max_blocks;
     const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
     const int lo_first = (a.window > 0 && p_first - a.window + 1 > 0) ? p_first - a.window + 1 : 0;
     const int lo_last = (a.window > 0 && p_last - a.window + 1 > 0) ? p_last - a.window + 1 : 0;
@@ -155,150 +198,149 @@ __global__ void __launch_bounds__(256) paged_attention_mfma_kernel(AttnMfmaArgs 
     const int key_end = min(p_last + 1, my_seg1 * AM_SEG);
 
     // Q^T fragments: lane (column c, dims 32s + 8g ..)
-    constexpr int QS = (DT + 1) / 2;
     bf16x8_t qf[QS];
 #pragma unroll
     for (int s = 0; s < QS; ++s) {
         u32x4_t v = {0u, 0u, 0u, 0u};
         const int d = 32 * s + 8 * g;
-        if (col_ok && d < D) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + d);
+        if (col_ok && frag_in<DT>(s, g)) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + d);
         qf[s] = __builtin_bit_cast(bf16x8_t, v);
     }
-    f32x4_t o[DT], o_tot[PARTIAL ? 1 : DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4_t o_tot[PARTIAL ? 1 : DT];
 #pragma unroll
     for (int dt = 0; dt < (PARTIAL ? 1 : DT); ++dt) o_tot[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    float m = -INFINITY, l = 0.0f;           // the running segment
     float m_tot = -INFINITY, l_tot = 0.0f;   // the segments folded so far (slot < 0)
 
-    // Software pipeline: while step i is multiplied, the keys of step i+1 and the page ids of step i+2 are on their way.
-    struct Where {
-        size_t k_at[2], v_at[2];
-        bool in[2];
+    // the pages of a segment's 8 tiles of 16 keys (-1: the tile holds no key of the item) and the tiles' places in them;
+    // a cursor steps from tile to tile, so that nothing is divided
+    int cur_blk = key_begin / bt, cur_sub = key_begin % bt, cur_key = key_begin;
+    auto locate = [&](int (&pages)[8], int (&subs)[8]) {
+#pragma unroll
+        for (int tl = 0; tl < 8; ++tl) {
+            pages[tl] = cur_key < key_end ? table[cur_blk] : -1;
+            subs[tl] = cur_sub;
+            cur_key += 16;
+            cur_sub += 16;
+            if (cur_sub >= bt) {
+                cur_sub = 0;
+                ++cur_blk;
+            }
+        }
     };
-    auto locate = [&](int j0, int page0, int page1) {
-        Where w;
+    // K fragments of chunk v of the segment: lane (key c of each tile, dims 32s + 8g ..)
+    auto load_keys = [&](const int (&pages)[8], const int (&subs)[8], int v, bf16x8_t (&kf)[2][QS]) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int key0 = j0 + 16 * u;
-            const int page = u == 0 ? page0 : page1;
-            w.in[u] = key0 < key_end && page >= 0;
-            const int sub = key0 % bt;
-            const size_t head_at = (size_t)(page < 0 ? 0 : page) * Hkv + kvh;
-            w.k_at[u] = (head_at * bt + sub) * D;
-            w.v_at[u] = head_at * D * bt + sub;
-        }
-        return w;
-    };
-    auto page_of = [&](int key0) { return key0 < key_end ? table[key0 / bt] : -1; };
-    auto load_keys = [&](const Where& w, bf16x8_t (&kf)[2][QS]) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
+            const int page = pages[2 * v + u];
+            const bf16_t* src = a.k_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * bt + subs[2 * v + u] + c) * D + 8 * g;
 #pragma unroll
             for (int s = 0; s < QS; ++s) {
-                u32x4_t v = {0u, 0u, 0u, 0u};
-                const int d = 32 * s + 8 * g;
-                if (w.in[u] && d < D) v = *reinterpret_cast<const u32x4_t*>(a.k_cache + w.k_at[u] + (size_t)c * D + d);
-                kf[u][s] = __builtin_bit_cast(bf16x8_t, v);
+                u32x4_t x = {0u, 0u, 0u, 0u};
+                if (page >= 0 && frag_in<DT>(s, g)) x = *reinterpret_cast<const u32x4_t*>(src + 32 * s);
+                kf[u][s] = __builtin_bit_cast(bf16x8_t, x);
             }
+        }
     };
-    bf16x8_t kf[2][QS], kf_next[2][QS];
-    Where here = locate(key_begin, page_of(key_begin), page_of(key_begin + 16));
-    load_keys(here, kf);
-    int page_next0 = page_of(key_begin + 32), page_next1 = page_of(key_begin + 48);
-
-    for (int j0 = key_begin; j0 < key_end; j0 += 32) {
-        // V^T fragments of this step: lane (dim 16dt + c, keys 4g .. 4g+3 of each tile)
-        bf16x8_t vf[DT];
+    // V^T fragments of chunk v: lane (dim 16dt + c, keys 4g .. 4g+3 of each tile)
+    auto load_values = [&](const int (&pages)[8], const int (&subs)[8], int v, bf16x8_t (&vf)[DT]) {
+        const int page0 = pages[2 * v], page1 = pages[2 * v + 1];
+        const bf16_t* src0 = a.v_cache + (((size_t)(page0 < 0 ? 0 : page0) * Hkv + kvh) * D + c) * bt + subs[2 * v] + 4 * g;
+        const bf16_t* src1 = a.v_cache + (((size_t)(page1 < 0 ? 0 : page1) * Hkv + kvh) * D + c) * bt + subs[2 * v + 1] + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             u32x2_t v0 = {0u, 0u}, v1 = {0u, 0u};
-            const int d = 16 * dt + c;
-            if (d < D) {
-                if (here.in[0]) v0 = *reinterpret_cast<const u32x2_t*>(a.v_cache + here.v_at[0] + (size_t)d * bt + 4 * g);
-                if (here.in[1]) v1 = *reinterpret_cast<const u32x2_t*>(a.v_cache + here.v_at[1] + (size_t)d * bt + 4 * g);
-            }
-            const u32x4_t v = {v0[0], v0[1], v1[0], v1[1]};
-            vf[dt] = __builtin_bit_cast(bf16x8_t, v);
+            if (page0 >= 0) v0 = *reinterpret_cast<const u32x2_t*>(src0 + (size_t)16 * dt * bt);
+            if (page1 >= 0) v1 = *reinterpret_cast<const u32x2_t*>(src1 + (size_t)16 * dt * bt);
+            const u32x4_t x = {v0[0], v0[1], v1[0], v1[1]};
+            vf[dt] = __builtin_bit_cast(bf16x8_t, x);
         }
-        // the next step's keys, and the page ids of the step after it
-        const Where next = locate(j0 + 32, page_next0, page_next1);
-        if (j0 + 32 < key_end) load_keys(next, kf_next);
-        page_next0 = page_of(j0 + 64);
-        page_next1 = page_of(j0 + 80);
+    };
 
-        if (j0 + 31 <= p_first && j0 >= lo_last && here.in[0] && here.in[1]) {
-            attention_step<DT, false>(kf, vf, qf, 0xffu, a.scale, o, m, l);   // every key counts for every column
-        } else {
-            unsigned ok = 0u;
+    if (key_begin >= key_end) return;
+    int pages[8], subs[8], pages_next[8], subs_next[8];
+    locate(pages, subs);
+    bf16x8_t kf[2][QS], kf_next[2][QS];
+    load_keys(pages, subs, 0, kf);
+    for (int seg0 = key_begin; seg0 < key_end; seg0 += AM_SEG) {
+        locate(pages_next, subs_next);   // the next segment's pages are looked up while this one is worked on
+        f32x4_t s[8];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            if (v < 3) load_keys(pages, subs, v + 1, kf_next);
+            else load_keys(pages_next, subs_next, 0, kf_next);
+            chunk_scores<DT>(kf, qf, s[2 * v], s[2 * v + 1]);
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = j0 + 16 * u + 4 * g + i;
-                    if (here.in[u] && col_ok && key <= p_col && key >= lo_col && key < key_end) ok |= 1u << (4 * u + i);
-                }
-            attention_step<DT, true>(kf, vf, qf, ok, a.scale, o, m, l);
+                for (int q = 0; q < QS; ++q) kf[u][q] = kf_next[u][q];
         }
-        if (((j0 + 32) % AM_SEG) == 0 || j0 + 32 >= key_end) {
-            // the segment ends: write it out, or fold it into the segments before it
-            if constexpr (PARTIAL) {
-                if (col_ok) {
-                    const size_t at = (size_t)(slot + j0 / AM_SEG - seg_first) * 16 + c;
-                    float* dst = a.part_o + at * D;
+        bf16x8_t vf[DT], vf_next[DT];
+        load_values(pages, subs, 0, vf);
+        float m, l;
+        bf16x8_t pf[4];
+        bool all_in = true;
 #pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
-                        if (16 * dt + 4 * g < D) *reinterpret_cast<f32x4_t*>(dst + 16 * dt + 4 * g) = o[dt];   // D is a multiple of 16
-                    if (g == 0) {
-                        a.part_ml[at * 2] = m;
-                        a.part_ml[at * 2 + 1] = l;
-                    }
-                }
-            } else {
-                fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
+        for (int tl = 0; tl < 8; ++tl) all_in = all_in && pages[tl] >= 0;
+        if (seg0 + AM_SEG - 1 <= p_first && seg0 >= lo_last && all_in) {
+            segment_softmax<false>(s, 0xffffffffu, a.scale, m, l, pf);   // every key counts for every column
+        } else {
+            uint32_t ok = segment_mask(seg0, g, col_ok, lo_col, p_col, key_end);
+#pragma unroll
+            for (int tl = 0; tl < 8; ++tl)
+                if (pages[tl] < 0) ok &= ~(0xfu << (4 * tl));
+            segment_softmax<true>(s, ok, a.scale, m, l, pf);
+        }
+        f32x4_t o[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            if (v < 3) load_values(pages, subs, v + 1, vf_next);
+            chunk_values<DT>(vf, pf[v], o);
+            if (v < 3) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) vf[dt] = vf_next[dt];
             }
-            m = -INFINITY;
-            l = 0.0f;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
         }
-        here = next;
+        if constexpr (PARTIAL) {
+            if (col_ok) {
+                const size_t at = (size_t)(slot + seg0 / AM_SEG - seg_first) * 16 + c;
+                float* dst = a.part_o + at * D;
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+                for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(dst + 16 * dt + 4 * g) = o[dt];
+                if (g == 0) {
+                    a.part_ml[at * 2] = m;
+                    a.part_ml[at * 2 + 1] = l;
+                }
+            }
+        } else {
+            fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
+        }
 #pragma unroll
-            for (int s = 0; s < QS; ++s) kf[u][s] = kf_next[u][s];
+        for (int tl = 0; tl < 8; ++tl) {
+            pages[tl] = pages_next[tl];
+            subs[tl] = subs_next[tl];
+        }
     }
-    if (!col_ok || PARTIAL) return;
-    // lane holds dims 16dt + 4g + i of its column
-    const float inv = 1.0f / l_tot;
-    bf16_t* dst = a.out + ((size_t)t * a.n_heads + h) * D;
-#pragma unroll
-    for (int dt = 0; dt < (PARTIAL ? 1 : DT); ++dt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int d = 16 * dt + 4 * g + i;
-            if (d < D) dst[d] = f32_to_bf16(o_tot[dt][i] * inv);
-        }
+    if constexpr (!PARTIAL) {
+        if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
+    }
 }
 
 // Prompt tiles that share their keys: a workgroup's 4 waves hold 4 items (tiles of up to 16 rows of one head each) of one
-// request and one KV head, for instance 4 of the query heads that read it.  The 32 keys and values of a step are
-// brought from the pages into LDS once by all 256 threads (double-buffered: the next step's are on their way while
-// this step is multiplied) and every wave takes its fragments from there, so each byte of the cache is read once for
-// 4 tiles.  A wave steps through its own range of keys only; per column the arithmetic is attention_step and
-// fold_segment as in the kernel above.  Items with n_rows == 0 fill up the last workgroup of a KV head.
+// request and one KV head, for instance 4 of the query heads that read it.  A segment's 128 keys and values are brought
+// from the pages into LDS once by all 256 threads and every wave takes its fragments from there, so each byte of the
+// cache is read once for 4 tiles.  The values of a segment travel while its scores are formed, the keys of the next
+// one while its values are multiplied; two barriers a segment.  A wave works on the segments of its own range only;
+// per column the arithmetic is that of the kernel above.  Items with n_rows == 0 fill up the last workgroup of a KV head.
 template <int DT>
 __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_kernel(AttnMfmaArgs a) {
     constexpr int QS = (DT + 1) / 2;
-    constexpr int DP = 16 * DT;          // head_dim (a multiple of 16)
-    constexpr int K_LD = DP + 8;         // bf16 elements a key's row takes in LDS
-    constexpr int V_LD = 36;             // bf16 elements a dim's row of 32 keys takes in LDS
-    constexpr int K_CHUNKS = 32 * DP / 8;   // 16-byte chunks of a step's keys
-    constexpr int V_CHUNKS = DP * 4;        // and of its values: dim d, tile u, half h -> 8 tokens
-    constexpr int K_ROUNDS = (K_CHUNKS + 255) / 256, V_ROUNDS = (V_CHUNKS + 255) / 256;
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[2][32 * K_LD];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[2][DP * V_LD];
+    constexpr int D = 16 * DT;
+    constexpr int K_LD = D + 8;              // bf16 elements a key's row takes in LDS
+    constexpr int V_LD = AM_SEG + 4;         // bf16 elements a dim's row of 128 keys takes in LDS: 66 words, so 16 dims' 8-byte reads miss each other's banks
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[AM_SEG * K_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * V_LD];
     __shared__ int ranges[4][2];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -308,7 +350,7 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
     const int h = __builtin_amdgcn_readfirstlane(it[2]);
     const int lead_row = a.items[(size_t)blockIdx.x * 4 * AM_ITEM_INTS];   // the first item is never a filler
     const int lead_head = a.items[(size_t)blockIdx.x * 4 * AM_ITEM_INTS + 2];
-    const int D = DP, bt = a.page_tokens, Hkv = a.n_kv_heads;
+    const int bt = a.page_tokens, Hkv = a.n_kv_heads;
     const int kvh = lead_head / (a.n_heads / Hkv);
     const int* table = a.tables + (size_t)a.row_entry[lead_row] * a.max_blocks;
     const int c = lane & 15, g = lane >> 4;
@@ -338,144 +380,146 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
     for (int s = 0; s < QS; ++s) {
         u32x4_t v = {0u, 0u, 0u, 0u};
         const int d = 32 * s + 8 * g;
-        if (col_ok && d < D) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + d);
+        if (col_ok && frag_in<DT>(s, g)) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + d);
         qf[s] = __builtin_bit_cast(bf16x8_t, v);
     }
-    f32x4_t o[DT], o_tot[DT];
+    f32x4_t o_tot[DT];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        o_tot[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-    float m = -INFINITY, l = 0.0f, m_tot = -INFINITY, l_tot = 0.0f;
+    for (int dt = 0; dt < DT; ++dt) o_tot[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_tot = -INFINITY, l_tot = 0.0f;
 
-    // Staging: the thread's chunks of a step go from the pages into registers, then into LDS.  What a chunk is (which
-    // key or dim, which of the step's two tiles) is fixed per thread; a step brings only the two tiles' base addresses.
-    int k_off[K_ROUNDS], k_lds[K_ROUNDS], v_off[V_ROUNDS], v_lds[V_ROUNDS];
-    bool k_second[K_ROUNDS], v_second[V_ROUNDS];
+    // Staging, tile by tile (a segment has 8 tiles of 16 keys, each inside one page).  A thread's 16-byte chunks of a
+    // tile: keys: chunk ch = tid + 256 r is key ch / (D/8) of the tile, dims 8 (ch % (D/8)) ..; values: chunk ch is dim
+    // ch / 2, tokens 8 (ch % 2) .. of the tile.  What a thread adds to a tile's base address never changes; the bases
+    // (page and place in the page) are the same for all threads and are kept by a cursor that steps from tile to tile.
+    constexpr int PER_TILE = (2 * D + 255) / 256;   // rounds a tile takes: 2 D chunks of keys (and of values)
+    constexpr int ROUNDS = 8 * PER_TILE;
+    u32x4_t stage[ROUNDS];
+    int k_off[PER_TILE], k_lds[PER_TILE], v_off[PER_TILE], v_lds[PER_TILE];
 #pragma unroll
-    for (int i = 0; i < K_ROUNDS; ++i) {
-        const int ch = tid + 256 * i;          // key ch / (DP/8) of the step, dims 8 * (ch % (DP/8)) ..
-        const int key = ch / (DP / 8), dc = ch % (DP / 8);
-        k_second[i] = key >= 16;
-        k_off[i] = (key & 15) * D + 8 * dc;
-        k_lds[i] = ch < K_CHUNKS ? key * K_LD + 8 * dc : -1;
+    for (int r = 0; r < PER_TILE; ++r) {
+        const int ch = tid + 256 * r;
+        const bool in = ch < 2 * D;
+        const int key = ch / (D / 8), dc = ch % (D / 8);
+        k_off[r] = key * D + 8 * dc;
+        k_lds[r] = in ? key * K_LD + 8 * dc : -1;
+        const int d = ch >> 1, half = ch & 1;
+        v_off[r] = d * bt + 8 * half;
+        v_lds[r] = in ? d * V_LD + 8 * half : -1;
     }
+    // the segment whose keys are fetched next: block-table index and place in the page of its first tile, and the
+    // pages and places of the 8 tiles of the segment whose keys were fetched last (its values are fetched later)
+    int next_blk = __builtin_amdgcn_readfirstlane(block_begin / bt), next_sub = __builtin_amdgcn_readfirstlane(block_begin % bt);
+    int pages[8], subs[8];
+    auto fetch_keys = [&](int seg0) {
 #pragma unroll
-    for (int i = 0; i < V_ROUNDS; ++i) {
-        const int ch = tid + 256 * i;          // dim ch / 4, tile (ch / 2) % 2, tokens 8 * (ch % 2) .. of the tile
-        const int d = ch >> 2, u = (ch >> 1) & 1, half = ch & 1;
-        v_second[i] = u == 1;
-        v_off[i] = d * bt + 8 * half;
-        v_lds[i] = ch < V_CHUNKS ? d * V_LD + 16 * u + 8 * half : -1;
-    }
-    u32x4_t k_reg[K_ROUNDS], v_reg[V_ROUNDS];
-    auto page_of = [&](int key0) { return key0 < block_end ? __builtin_amdgcn_readfirstlane(table[key0 / bt]) : -1; };
-    auto fetch = [&](int j0, int page0, int page1) {
-        // the tiles' first key and first value in the cache (uniform)
-        const int sub0 = j0 % bt, sub1 = (j0 + 16) % bt;
-        const size_t head0 = (size_t)(page0 < 0 ? 0 : page0) * Hkv + kvh, head1 = (size_t)(page1 < 0 ? 0 : page1) * Hkv + kvh;
-        const bf16_t* kb0 = a.k_cache + (head0 * bt + sub0) * D;
-        const bf16_t* kb1 = a.k_cache + (head1 * bt + sub1) * D;
-        const bf16_t* vb0 = a.v_cache + head0 * D * bt + sub0;
-        const bf16_t* vb1 = a.v_cache + head1 * D * bt + sub1;
-        const bool in0 = page0 >= 0 && j0 < block_end, in1 = page1 >= 0 && j0 + 16 < block_end;
+        for (int tl = 0; tl < 8; ++tl) {
+            const int page = seg0 + 16 * tl < block_end ? __builtin_amdgcn_readfirstlane(table[next_blk]) : -1;
+            pages[tl] = page;
+            subs[tl] = next_sub;
+            const bf16_t* base = a.k_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * bt + next_sub) * D;
 #pragma unroll
-        for (int i = 0; i < K_ROUNDS; ++i) {
-            u32x4_t v = {0u, 0u, 0u, 0u};
-            if (k_lds[i] >= 0 && (k_second[i] ? in1 : in0)) v = *reinterpret_cast<const u32x4_t*>((k_second[i] ? kb1 : kb0) + k_off[i]);
-            k_reg[i] = v;
-        }
-#pragma unroll
-        for (int i = 0; i < V_ROUNDS; ++i) {
-            u32x4_t v = {0u, 0u, 0u, 0u};
-            if (v_lds[i] >= 0 && (v_second[i] ? in1 : in0)) v = *reinterpret_cast<const u32x4_t*>((v_second[i] ? vb1 : vb0) + v_off[i]);
-            v_reg[i] = v;
-        }
-    };
-    auto stage = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < K_ROUNDS; ++i)
-            if (k_lds[i] >= 0) *reinterpret_cast<u32x4_t*>(&Ks[buf][k_lds[i]]) = k_reg[i];
-#pragma unroll
-        for (int i = 0; i < V_ROUNDS; ++i)
-            if (v_lds[i] >= 0) {
-                u32x2_t* dst = reinterpret_cast<u32x2_t*>(&Vs[buf][v_lds[i]]);
-                dst[0] = u32x2_t{v_reg[i][0], v_reg[i][1]};
-                dst[1] = u32x2_t{v_reg[i][2], v_reg[i][3]};
+            for (int r = 0; r < PER_TILE; ++r) {
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                if (page >= 0 && k_lds[r] >= 0) v = *reinterpret_cast<const u32x4_t*>(base + k_off[r]);
+                stage[tl * PER_TILE + r] = v;
             }
+            next_sub += 16;
+            if (next_sub >= bt) {
+                next_sub = 0;
+                ++next_blk;
+            }
+        }
     };
-    const int k_at = c * K_LD + 8 * g, v_at = c * V_LD + 4 * g;   // where the lane's fragments start in a buffer
-    int page_next0, page_next1;
-    // one step from buffer `buf` (a constant where it is called, so that the LDS addresses are immediates)
-    auto step = [&](int j0, auto buf_c) {
-        constexpr int buf = decltype(buf_c)::value;
-        const bool more = j0 + 32 < block_end;
-        if (more) fetch(j0 + 32, page_next0, page_next1);
-        page_next0 = page_of(j0 + 64);
-        page_next1 = page_of(j0 + 80);
-        if (j0 >= key_begin && j0 < key_end) {
-            bf16x8_t kf[2][QS], vf[DT];
+    auto stage_keys = [&]() {
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+        for (int tl = 0; tl < 8; ++tl)
 #pragma unroll
-                for (int s = 0; s < QS; ++s) {
-                    u32x4_t v = {0u, 0u, 0u, 0u};
-                    if (32 * s + 8 * g < DP) v = *reinterpret_cast<const u32x4_t*>(&Ks[buf][k_at + 16 * u * K_LD + 32 * s]);
-                    kf[u][s] = __builtin_bit_cast(bf16x8_t, v);
+            for (int r = 0; r < PER_TILE; ++r)
+                if (k_lds[r] >= 0) *reinterpret_cast<u32x4_t*>(&Ks[16 * tl * K_LD + k_lds[r]]) = stage[tl * PER_TILE + r];
+    };
+    auto fetch_values = [&]() {   // of the segment whose keys were fetched last
+#pragma unroll
+        for (int tl = 0; tl < 8; ++tl) {
+            const int page = pages[tl];
+            const bf16_t* base = a.v_cache + ((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * D * bt + subs[tl];
+#pragma unroll
+            for (int r = 0; r < PER_TILE; ++r) {
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                if (page >= 0 && v_lds[r] >= 0) v = *reinterpret_cast<const u32x4_t*>(base + v_off[r]);
+                stage[tl * PER_TILE + r] = v;
+            }
+        }
+    };
+    auto stage_values = [&]() {
+#pragma unroll
+        for (int tl = 0; tl < 8; ++tl)
+#pragma unroll
+            for (int r = 0; r < PER_TILE; ++r)
+                if (v_lds[r] >= 0) {
+                    u32x2_t* dst = reinterpret_cast<u32x2_t*>(&Vs[v_lds[r] + 16 * tl]);
+                    dst[0] = u32x2_t{stage[tl * PER_TILE + r][0], stage[tl * PER_TILE + r][1]};
+                    dst[1] = u32x2_t{stage[tl * PER_TILE + r][2], stage[tl * PER_TILE + r][3]};
                 }
+    };
+    const int k_at = c * K_LD + 8 * g, v_at = c * V_LD + 4 * g;   // where the lane's fragments start
+
+    if (block_begin >= block_end) return;
+    fetch_keys(block_begin);
+    stage_keys();
+    __syncthreads();
+    for (int seg0 = block_begin; seg0 < block_end; seg0 += AM_SEG) {
+        const bool mine = seg0 >= key_begin && seg0 < key_end;
+        fetch_values();
+        f32x4_t s[8];
+        if (mine) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(&Vs[buf][v_at + 16 * dt * V_LD]);
-                const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(&Vs[buf][v_at + 16 * dt * V_LD + 16]);
-                const u32x4_t v = {v0[0], v0[1], v1[0], v1[1]};
-                vf[dt] = __builtin_bit_cast(bf16x8_t, v);
-            }
-            if (j0 + 31 <= p_first && j0 >= lo_last) {
-                attention_step<DT, false>(kf, vf, qf, 0xffu, a.scale, o, m, l);   // every key counts for every column
-            } else {
-                unsigned ok = 0u;
+            for (int v = 0; v < 4; ++v) {
+                bf16x8_t kf[2][QS];
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int key = j0 + 16 * u + 4 * g + i;
-                        if (col_ok && key <= p_col && key >= lo_col && key < key_end) ok |= 1u << (4 * u + i);
+                    for (int q = 0; q < QS; ++q) {
+                        u32x4_t x = {0u, 0u, 0u, 0u};
+                        if (frag_in<DT>(q, g)) x = *reinterpret_cast<const u32x4_t*>(&Ks[k_at + (32 * v + 16 * u) * K_LD + 32 * q]);
+                        kf[u][q] = __builtin_bit_cast(bf16x8_t, x);
                     }
-                attention_step<DT, true>(kf, vf, qf, ok, a.scale, o, m, l);
-            }
-            if (((j0 + 32) % AM_SEG) == 0 || j0 + 32 >= key_end) {
-                fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
-                m = -INFINITY;
-                l = 0.0f;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                chunk_scores<DT>(kf, qf, s[2 * v], s[2 * v + 1]);
             }
         }
-        if (more) stage(buf ^ 1);
-        __syncthreads();
-    };
-
-    if (block_begin >= block_end) return;
-    fetch(block_begin, page_of(block_begin), page_of(block_begin + 16));
-    page_next0 = page_of(block_begin + 32);
-    page_next1 = page_of(block_begin + 48);
-    stage(0);
-    __syncthreads();
-    for (int j0 = block_begin; j0 < block_end; j0 += 64) {
-        step(j0, std::integral_constant<int, 0>{});
-        if (j0 + 32 < block_end) step(j0 + 32, std::integral_constant<int, 1>{});
-    }
-    if (!col_ok) return;
-    const float inv = 1.0f / l_tot;
-    bf16_t* dst = a.out + ((size_t)t * a.n_heads + h) * D;
+        stage_values();
+        __syncthreads();                       // the values are in LDS; nobody reads this segment's keys any more
+        const bool more = seg0 + AM_SEG < block_end;
+        if (more) fetch_keys(seg0 + AM_SEG);
+        if (mine) {
+            float m, l;
+            bf16x8_t pf[4];
+            if (seg0 + AM_SEG - 1 <= p_first && seg0 >= lo_last) {
+                segment_softmax<false>(s, 0xffffffffu, a.scale, m, l, pf);   // every key counts for every column
+            } else {
+                segment_softmax<true>(s, segment_mask(seg0, g, col_ok, lo_col, p_col, key_end), a.scale, m, l, pf);
+            }
+            f32x4_t o[DT];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        const int d = 16 * dt + 4 * g;
-        const u32x2_t packed = {(uint32_t)f32_to_bf16(o_tot[dt][0] * inv) | ((uint32_t)f32_to_bf16(o_tot[dt][1] * inv) << 16),
-                                (uint32_t)f32_to_bf16(o_tot[dt][2] * inv) | ((uint32_t)f32_to_bf16(o_tot[dt][3] * inv) << 16)};
-        *reinterpret_cast<u32x2_t*>(dst + d) = packed;
+            for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                bf16x8_t vf[DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(&Vs[v_at + 16 * dt * V_LD + 32 * v]);
+                    const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(&Vs[v_at + 16 * dt * V_LD + 32 * v + 16]);
+                    const u32x4_t x = {v0[0], v0[1], v1[0], v1[1]};
+                    vf[dt] = __builtin_bit_cast(bf16x8_t, x);
+                }
+                chunk_values<DT>(vf, pf[v], o);
+            }
+            fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
+        }
+        if (more) stage_keys();
+        __syncthreads();                       // the next keys are in LDS; nobody reads this segment's values any more
     }
+    if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
 }
 
 // merge: one block per output (row, head).  merge item: {row, head, first_slot, column}.  The row's segments are folded
