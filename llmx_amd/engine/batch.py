@@ -36,6 +36,7 @@ class Workspace:
     def __init__(self, device: torch.device):
         self.device = device
         self._store: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self.generation = 0     # counts allocations: addresses handed out before a change may be stale
 
     def get(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         count = 1
@@ -46,6 +47,7 @@ class Workspace:
         if flat is None or flat.numel() < count:
             flat = torch.empty(max(count, 1), dtype=dtype, device=self.device)
             self._store[key] = flat
+            self.generation += 1
         return flat[:count].view(*shape)
 
     def bytes(self) -> int:
@@ -85,6 +87,10 @@ class StepState:
             self._plans[key] = plan
         return plan
 
+    def plan_requests(self):
+        """The (heads, kv heads, window) attention plans were asked for in this step."""
+        return list(self._plans.keys())
+
     def observe(self, kind: str, **tensors) -> None:
         """Shows intermediate tensors (a router's picks, for instance) to the engine's observer, when one is set."""
         if self.observer is not None:
@@ -99,6 +105,7 @@ class RowPlanUploader:
         self._host = None
         self._dev = None
         self._done = None
+        self.generation = 0     # counts allocations of the device buffer
 
     def upload(self, arrays: List[np.ndarray]) -> List[torch.Tensor]:
         total = sum(a.size for a in arrays)
@@ -107,6 +114,7 @@ class RowPlanUploader:
             self._host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
             self._dev = torch.empty(cap, dtype=torch.int32, device=self.device)
             self._done = None
+            self.generation += 1
         if self._done is not None:
             self._done.synchronize()  # the previous copy has left the pinned buffer
         host = self._host.numpy()
@@ -117,6 +125,11 @@ class RowPlanUploader:
             views.append(self._dev[at:at + a.size].view(*a.shape))
             at += a.size
         self._dev[:total].copy_(self._host[:total], non_blocking=True)
+        self.mark()
+        return views
+
+    def mark(self) -> None:
+        """Everything enqueued so far (the copy, kernels that read the device buffer) must end before the pinned buffer
+        and the device buffer are written again."""
         self._done = torch.cuda.Event()
         self._done.record()
-        return views

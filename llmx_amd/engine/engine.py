@@ -43,11 +43,26 @@ def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
     raise ValueError(f"dtype {dtype!r} is not float32 or bfloat16")
 
 
+class _StepGraph:
+    """A recorded decode step: the graph, where its logits appear, and what must not have moved since."""
+
+    def __init__(self, graph, logits, plans, workspace_generation, uploader_generation):
+        self.graph = graph
+        self.logits = logits
+        self.plans = plans      # kept alive: the graph's kernels read their work items
+        self.generations = (workspace_generation, uploader_generation)
+
+    def stale(self, engine: "Engine") -> bool:
+        return self.generations != (engine._workspace.generation, engine._uploader.generation)
+
+
 class Engine:
     def __init__(self, config, spec: ModelSpec, dtype: Union[str, torch.dtype] = "bfloat16", *, kv_tokens: int,
-                 page_tokens: int = 16, max_requests: int = 8, device: Union[str, torch.device] = "cuda:0", weights=None):
+                 page_tokens: int = 16, max_requests: int = 8, device: Union[str, torch.device] = "cuda:0", weights=None,
+                 graphs: bool = True):
         """`weights(engine)` returns the device tensors by name; it runs before the cache is allocated, so weights that
-        do not fit the model are refused before anything large exists."""
+        do not fit the model are refused before anything large exists.  `graphs`: steps of single decoded tokens are
+        replayed as HIP graphs once their shape has been seen twice (see `_run`)."""
         if not torch.cuda.is_available():
             raise RuntimeError("llmx_amd runs on a GPU only: no GPU is visible and there is no CPU path")
         ops.lib()  # fail now, loudly, when the kernel library is missing
@@ -74,6 +89,12 @@ class Engine:
         #: /root/reference/src/model/arch/blocks.hpp:118-138); None in serving
         self.observer = None
         self._make_cache()
+        self.graphs = bool(graphs) and all(getattr(p, "graph_safe", False) for p in self.model.parts()) \
+            and all(getattr(b, "graph_safe", False) for b in self.model.blocks)
+        self._graphs: Dict[tuple, "_StepGraph"] = {}
+        self._graph_seen: Dict[tuple, int] = {}
+        self._plan_requests: set = set()      # the (heads, kv heads, window) the mixers ask attention plans for
+        self.graph_replays = 0                # steps that ran as a replay (for tests and measurement)
 
     # -- construction -----------------------------------------------------------
     @classmethod
@@ -243,7 +264,7 @@ class Engine:
         for g in range(len(self.cache.groups)):
             tables = [self.cache.table(e.request, g) for e in entries]
             width = max(1, max(len(t) for t in tables))
-            width = -(-width // 8) * 8
+            width = -(-width // 64) * 64     # in steps of 64 pages, so that a growing context keeps its width (and its graph) for long
             packed = np.full((n_e, width), -1, dtype=np.int32)
             for i, t in enumerate(tables):
                 packed[i, :len(t)] = t
@@ -257,15 +278,48 @@ class Engine:
         step.pick = dev[4][:len(pick)]
         step._tables = dev[5:]
         step.max_rows_per_entry = max(v.n for v in views)
+        step.observer = self.observer
 
-        E = self.spec.hidden_size
+        # A step of single decoded tokens launches a few hundred short kernels; replayed as one HIP graph they follow
+        # each other without the host.  A graph holds addresses and launch sizes, so it is keyed by all that fixes
+        # them (rows, wanted places, widths of the block tables, the attention plans) and dropped when scratch storage
+        # moves.  The row plan is copied to the device before the replay, outside the graph; the graph holds kernels only.
+        key = None
+        if self.graphs and self.observer is None and len(pick) > 0 and all(v.n == 1 for v in views):
+            plans = tuple(step.attention_plan(*req) for req in sorted(self._plan_requests))
+            key = (T, tuple(pick), tuple(a.shape for a in arrays[5:]), tuple(id(p) for p in plans))
+            graph = self._graphs.get(key)
+            if graph is not None and not graph.stale(self):
+                graph.graph.replay()
+                self.graph_replays += 1
+                self._uploader.mark()
+                return graph.logits
+            if graph is not None:
+                self._graphs.clear()
+                self._graph_seen.clear()
+        if key is not None and self._graph_seen.get(key, 0) >= 1:
+            graph = self._capture(step, key, plans)
+            if graph is not None:
+                graph.graph.replay()
+                self.graph_replays += 1
+                self._uploader.mark()
+                return graph.logits
+        logits = self._forward(step)
+        self._plan_requests.update(step.plan_requests())
+        if key is not None:
+            if len(self._graph_seen) > 256:
+                self._graph_seen.clear()
+            self._graph_seen[key] = self._graph_seen.get(key, 0) + 1
+        return logits
+
+    def _forward(self, step: StepState) -> torch.Tensor:
+        T, E = step.rows, self.spec.hidden_size
         x = step.buf("residual", (T, E), torch.float32)
         self.model.embedding.forward(step, x)
-        step.observer = self.observer
         for i, (entry, cache) in enumerate(zip(self.spec.run_order, self._layer_caches)):
             step.run_index = i
             self.model.blocks[entry.layer].forward(step, x, cache)
-        W = len(pick)
+        W = step.pick.shape[0]
         if W == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         rows = step.buf("head.rows", (W, E), self.act_dtype)
@@ -273,6 +327,26 @@ class Engine:
         logits = step.buf("logits", (W, self.spec.vocab_size), torch.float32)
         self.model.head.forward(step, rows, logits)
         return logits
+
+    def _capture(self, step: StepState, key: tuple, plans: tuple) -> Optional["_StepGraph"]:
+        """Records the step's launches (a step of this shape ran before, so every scratch tensor exists) into a graph."""
+        before = (self._workspace.generation, self._uploader.generation)
+        graph = torch.cuda.CUDAGraph()
+        try:
+            with torch.cuda.graph(graph):
+                logits = self._forward(step)
+        except Exception as err:   # a graph is an optimisation: without it the step runs as it always did
+            import warnings
+            warnings.warn(f"llmx_amd: recording a decode step as a HIP graph failed ({err}); steps run without graphs")
+            self.graphs = False
+            return None
+        if (self._workspace.generation, self._uploader.generation) != before:
+            return None            # storage moved while recording: the graph holds stale addresses
+        if len(self._graphs) >= 32:
+            self._graphs.pop(next(iter(self._graphs)))
+        record = _StepGraph(graph, logits, plans, *before)
+        self._graphs[key] = record
+        return record
 
     # -- for measurement ----------------------------------------------------------
     def assume_context(self, request: Hashable, n: int) -> None:

@@ -22,6 +22,7 @@ _NORM_MODES = {"none": ops.QKNORM_NONE, "projection": ops.QKNORM_PROJECTION}
 
 class Attention(Mixer):
     """params: hidden, heads, kv_heads, head_dim, qk_norm ("projection" | "none"), eps, window (None | int), position (PartSpec)."""
+    graph_safe = True
 
     def __init__(self, params, prefix, ctx: BuildContext):
         super().__init__(params, prefix, ctx)

@@ -44,6 +44,10 @@ class Part:
     """Base of every part."""
 
     kind: str = ""
+    #: True when `forward` only launches this package's kernels on the current stream into storage from `step.buf`
+    #: (no allocation, no host synchronisation, no library call that could record a fill into a captured graph);
+    #: the engine replays decode steps as HIP graphs only if every part of the model says so.
+    graph_safe: bool = False
 
     def __init__(self, params: dict, prefix: str, ctx: BuildContext):
         self.params = dict(params)

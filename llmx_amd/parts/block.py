@@ -13,6 +13,8 @@ from .spec import BlockSpec
 
 
 class PreNormBlock:
+    graph_safe = True   # see Part.graph_safe
+
     def __init__(self, spec: BlockSpec, ctx: BuildContext):
         self.mixer_norm = build_part("norm", spec.mixer_norm, ctx)
         self.mixer = build_part("mixer", spec.mixer, ctx)

@@ -15,6 +15,7 @@ from .spec import TensorSpec
 
 class TokenEmbedding(Embedding):
     """params: vocab, hidden; tensor <prefix>weight (vocab, hidden)."""
+    graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
@@ -37,6 +38,7 @@ class TokenEmbedding(Embedding):
 
 class LinearHead(Head):
     """params: vocab, hidden, tied (bool); tensor <prefix>weight (vocab, hidden) unless tied."""
+    graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)

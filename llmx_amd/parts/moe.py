@@ -22,6 +22,7 @@ _SCORES = {"sigmoid": ops.SCORE_SIGMOID, "softmax": ops.SCORE_SOFTMAX}
 
 class RoutedExperts(FeedForward):
     """params: hidden, experts, top_k, intermediate, score ("sigmoid" | "softmax"), correction_bias (bool), normalize (bool), scale."""
+    graph_safe = True
 
     wants_f32_input = True
 
@@ -101,6 +102,7 @@ class RoutedExperts(FeedForward):
 
 class DenseGLU(FeedForward):
     """params: hidden, intermediate.  y = (silu(h.Wg^T) * (h.Wu^T)).Wd^T; tensors gate_proj, up_proj, down_proj (.weight)."""
+    graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)

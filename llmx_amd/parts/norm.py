@@ -17,6 +17,7 @@ from .spec import TensorSpec
 
 class RMSNorm(Norm):
     """params: width, eps; tensor: <prefix>weight (width,)."""
+    graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)

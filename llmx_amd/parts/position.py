@@ -34,6 +34,7 @@ def neox_table(positions: int, rotary_dim: int, theta: float) -> np.ndarray:
 
 class PartialRotary(PositionEncoding):
     """params: rotary_dim (even, at most head_dim; 0 rotates nothing), theta, head_dim."""
+    graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
@@ -51,6 +52,7 @@ class PartialRotary(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """Leaves rows as they are."""
+    graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)

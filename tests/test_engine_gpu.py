@@ -191,6 +191,48 @@ def test_long_decoding(setup):
     check_against_plain(name, dtype, length, 7, got, engine, "l")
 
 
+@pytest.mark.parametrize("name,dtype", [("A", "bfloat16"), ("B", "float32"), ("A16", "bfloat16")])
+def test_decode_steps_replayed_as_graphs_equal_eager_steps(name, dtype):
+    """Steps of single decoded tokens are replayed as HIP graphs once their shape has been seen.  Every replay gives the
+    bits of an engine that never records a graph, with prompts of other requests (eager work), synchronisations, page
+    edges and a change of the batch between the replays."""
+    from llmx_amd.engine import Engine, StepEntry
+    page = TINY[name][2]
+    engines = [Engine.load(model_folder(name), dtype=dtype, kv_tokens=1024, page_tokens=page, max_requests=8, graphs=g) for g in (True, False)]
+    assert engines[0].graphs and not engines[1].graphs
+    prompts = {"a": tokens_for(name, 9, 1), "b": tokens_for(name, 30, 2), "c": tokens_for(name, 3, 3)}
+    extra = tokens_for(name, 70, 4)
+    last = {}
+    for eng in engines:
+        for rid, toks in prompts.items():
+            eng.add_request(rid)
+            last[rid] = eng.step([StepEntry(rid, toks, [len(toks) - 1])]).argmax(dim=1).item()
+    live = ["a", "b", "c"]
+    nxt = dict(last)
+    for i in range(60):
+        outs = []
+        for eng in engines:
+            if i == 12:
+                eng.add_request("x")
+                eng.step([StepEntry("x", extra[:33], [])])        # another request's prompt between the replays
+                torch.cuda.synchronize()
+            if i == 30:
+                eng.step([StepEntry("x", extra[33:], [36])])
+                eng.end_request("x")
+            if i == 40 and "b" in live and eng is engines[0]:
+                pass
+            outs.append(eng.step([StepEntry(rid, [nxt[rid]], [0]) for rid in live]).clone())
+        assert torch.equal(outs[0], outs[1]), f"step {i}: the replayed step differs from the eager one"
+        picks = outs[0].argmax(dim=1).tolist()
+        nxt = {rid: p for rid, p in zip(live, picks)}
+        if i == 40:
+            for eng in engines:
+                eng.end_request("b")
+            live = ["a", "c"]
+            nxt.pop("b")
+    assert engines[0].graph_replays >= 40 and engines[1].graph_replays == 0
+
+
 def test_refusals_leave_nothing_behind(setup):
     from llmx_amd.engine import StepEntry, StepError
     name, dtype, engine = setup
