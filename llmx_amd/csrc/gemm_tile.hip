@@ -13,6 +13,7 @@
 // from zero in step order, the runs' sums added in run order.  So a row's result does not depend on whether its step
 // held few rows or many.
 #include "common.h"
+#include <type_traits>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -40,10 +41,15 @@ struct TileArgs {
     int ks;       // runs K is cut into (the weight-streaming kernel's waves per strip for this shape)
 };
 
-template <int EPI, typename TC, bool GROUPED, bool SPLIT>
+// FAST: K is a multiple of 64 and the runs end on multiples of 64, so nothing in the loop needs a bound: the tiles are
+// loaded without conditions (a row past the tile's rows reads the first row, a feature past N the last; what they
+// produce is never stored, and a column of the product never touches another), LDS holds two tiles and a tile takes one
+// barrier: the tile after the next travels into registers while the next is written to the other half of LDS and this
+// one is multiplied.
+template <int EPI, typename TC, bool GROUPED, bool SPLIT, bool FAST>
 __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
-    __shared__ __attribute__((aligned(16))) bf16_t As[TL_BM * TL_LD];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[TL_BN * TL_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t As[(FAST ? 2 : 1) * TL_BM * TL_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[(FAST ? 2 : 1) * TL_BN * TL_LD];
     __shared__ int rows_a[TL_BM];
     __shared__ int rows_c[TL_BM];
     __shared__ int tile_info[2];
@@ -144,17 +150,22 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         for (int i = 0; i < 4; ++i) {
             const int kc = ((tid + 256 * i) & 7) * 8;
             const bool in = k0 + kc < K;
-            if (i < 2) a_reg[i] = (in && a_ok[i]) ? *reinterpret_cast<const u32x4_t*>(a_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
-            w_reg[i] = (in && w_ok[i]) ? *reinterpret_cast<const u32x4_t*>(w_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
+            if (FAST) {
+                if (i < 2) a_reg[i] = *reinterpret_cast<const u32x4_t*>(a_src[i] + k0);
+                w_reg[i] = *reinterpret_cast<const u32x4_t*>(w_src[i] + k0);
+            } else {
+                if (i < 2) a_reg[i] = (in && a_ok[i]) ? *reinterpret_cast<const u32x4_t*>(a_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
+                w_reg[i] = (in && w_ok[i]) ? *reinterpret_cast<const u32x4_t*>(w_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
+            }
         }
     };
-    auto store_lds = [&]() {
+    auto store_lds = [&](int buf = 0) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int c = tid + 256 * i;
             const int row = c >> 3, kc = (c & 7) * 8;
-            if (i < 2) *reinterpret_cast<u32x4_t*>(&As[row * TL_LD + kc]) = a_reg[i];
-            *reinterpret_cast<u32x4_t*>(&Ws[row * TL_LD + kc]) = w_reg[i];
+            if (i < 2) *reinterpret_cast<u32x4_t*>(&As[buf * TL_BM * TL_LD + row * TL_LD + kc]) = a_reg[i];
+            *reinterpret_cast<u32x4_t*>(&Ws[buf * TL_BN * TL_LD + row * TL_LD + kc]) = w_reg[i];
         }
     };
 
@@ -179,6 +190,58 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     int until_fold = per;                                // steps left in the current run
     bool first_run = true;
 
+    if constexpr (FAST) {
+        const int n_tiles = K / TL_BK, tiles_per_run = per / 2;
+        int until = tiles_per_run;
+        // one tile (both 32-wide steps) out of LDS half `buf`, a constant where it is called
+        auto multiply = [&](auto buf_c) {
+            constexpr int buf = decltype(buf_c)::value;
+#pragma unroll
+            for (int kk = 0; kk < TL_BK; kk += 32) {
+                bf16x8_t wf[4], af[2];
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+                    wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[buf * TL_BN * TL_LD + w_row[f] * TL_LD + kk + lk]));
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    af[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[buf * TL_BM * TL_LD + (32 * wm + 16 * t + lr) * TL_LD + kk + lk]));
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[t], acc[f][t], 0, 0, 0);
+            }
+        };
+        auto tile = [&](int t, auto buf_c) {
+            constexpr int buf = decltype(buf_c)::value;
+            if (t + 1 < n_tiles) store_lds(buf ^ 1);
+            if (t + 2 < n_tiles) load_global((t + 2) * TL_BK);
+            if (SPLIT && until == 0) {
+                // a run of K ends: its sum joins the runs before it, in run order
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        if (first_run) total[f][q] = acc[f][q];
+                        else total[f][q] = f32x4_t{total[f][q][0] + acc[f][q][0], total[f][q][1] + acc[f][q][1],
+                                                   total[f][q][2] + acc[f][q][2], total[f][q][3] + acc[f][q][3]};
+                        acc[f][q] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                    }
+                first_run = false;
+                until = tiles_per_run;
+            }
+            multiply(buf_c);
+            --until;
+            __syncthreads();
+        };
+        load_global(0);
+        store_lds(0);
+        if (n_tiles > 1) load_global(TL_BK);
+        __syncthreads();
+        for (int t = 0; t < n_tiles; t += 2) {
+            tile(t, std::integral_constant<int, 0>{});
+            if (t + 1 < n_tiles) tile(t + 1, std::integral_constant<int, 1>{});
+        }
+    } else {
     load_global(0);
     store_lds();
     __syncthreads();
@@ -221,6 +284,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
             __syncthreads();
         }
     }
+    }
     if (SPLIT && !first_run) {
 #pragma unroll
         for (int f = 0; f < 4; ++f)
@@ -262,14 +326,24 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     }
 }
 
+template <int EPI, typename TC, bool GROUPED, bool SPLIT>
+static void tile_launch_fast(const TileArgs& g, dim3 grid, hipStream_t stream) {
+    // the lean loop needs whole 64-wide tiles and runs that end on them
+    const int steps = (g.K + 31) / 32, per = (steps + g.ks - 1) / g.ks;
+    if (g.K % TL_BK == 0 && (!SPLIT || per % 2 == 0))
+        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true>), grid, dim3(256), 0, stream, g);
+    else
+        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, false>), grid, dim3(256), 0, stream, g);
+}
+
 template <int EPI, typename TC>
 static void tile_launch(const TileArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
     if (grouped) {
-        if (g.ks > 1) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, true, true>), grid, dim3(256), 0, stream, g);
-        else hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, true, false>), grid, dim3(256), 0, stream, g);
+        if (g.ks > 1) tile_launch_fast<EPI, TC, true, true>(g, grid, stream);
+        else tile_launch_fast<EPI, TC, true, false>(g, grid, stream);
     } else {
-        if (g.ks > 1) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, false, true>), grid, dim3(256), 0, stream, g);
-        else hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, false, false>), grid, dim3(256), 0, stream, g);
+        if (g.ks > 1) tile_launch_fast<EPI, TC, false, true>(g, grid, stream);
+        else tile_launch_fast<EPI, TC, false, false>(g, grid, stream);
     }
 }
 

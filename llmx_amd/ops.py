@@ -141,7 +141,7 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[tor
 
 
 SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores
-SKINNY_MAX_GROUPED_ROWS = 128  # routed products of at most this many token rows do
+SKINNY_MAX_GROUPED_ROWS = 16   # routed products of at most this many token rows do (measured: beyond it the tiled kernel streams the experts faster)
 
 
 _KS_OVERRIDE = None   # set by tuning scripts only
