@@ -21,7 +21,6 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 enum : int { TL_STORE = 0, TL_ADD = 1, TL_SWIGLU = 2 };
 
-#define TL_BM 64
 #define TL_BN 128
 #define TL_BK 64
 #define TL_LD 72  // padded row length in bf16 elements (144 bytes)
@@ -39,19 +38,20 @@ struct TileArgs {
     int up_offset;
     int m_tiles;  // dense: number of row tiles
     int ks;       // runs K is cut into (the weight-streaming kernel's waves per strip for this shape)
+    int bm;       // rows a workgroup covers: 64 or 128
 };
 
-// FAST: K is a multiple of 64 and the runs end on multiples of 64, so nothing in the loop needs a bound: the tiles are
+// FAST: K is a multiple of 64 and the runs are an even number of 64-wide tiles, so nothing in the loop needs a bound: the tiles are
 // loaded without conditions (a row past the tile's rows reads the first row, a feature past N the last; what they
 // produce is never stored, and a column of the product never touches another), LDS holds two tiles and a tile takes one
 // barrier: the tile after the next travels into registers while the next is written to the other half of LDS and this
 // one is multiplied.
-template <int EPI, typename TC, bool GROUPED, bool SPLIT, bool FAST>
-__global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
-    __shared__ __attribute__((aligned(16))) bf16_t As[(FAST ? 2 : 1) * TL_BM * TL_LD];
+template <int EPI, typename TC, bool GROUPED, bool SPLIT, bool FAST, int BM>
+__global__ void __launch_bounds__(256, BM == 128 ? 2 : 1) gemm_tile_kernel(TileArgs g) {
+    __shared__ __attribute__((aligned(16))) bf16_t As[(FAST ? 2 : 1) * BM * TL_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Ws[(FAST ? 2 : 1) * TL_BN * TL_LD];
-    __shared__ int rows_a[TL_BM];
-    __shared__ int rows_c[TL_BM];
+    __shared__ int rows_a[BM];
+    __shared__ int rows_c[BM];
     __shared__ int tile_info[2];
     __shared__ int scan_waves[4];
 
@@ -68,7 +68,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         for (int e0 = 0; e0 < g.n_groups; e0 += 256) {
             const int e = e0 + tid;
             const int begin = e < g.n_groups ? g.group_offsets[e] : 0;
-            const int tiles = e < g.n_groups ? (g.group_offsets[e + 1] - begin + TL_BM - 1) / TL_BM : 0;
+            const int tiles = e < g.n_groups ? (g.group_offsets[e + 1] - begin + BM - 1) / BM : 0;
             int incl = tiles;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
@@ -92,14 +92,14 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         __syncthreads();
         const int e = tile_info[0];
         if (e < 0) return;
-        row_begin = g.group_offsets[e] + tile_info[1] * TL_BM;
-        row_end = min(g.group_offsets[e + 1], row_begin + TL_BM);
+        row_begin = g.group_offsets[e] + tile_info[1] * BM;
+        row_end = min(g.group_offsets[e + 1], row_begin + BM);
         W += (size_t)e * g.w_group_stride;
     } else {
-        row_begin = blockIdx.y * TL_BM;
-        row_end = min(g.M, row_begin + TL_BM);
+        row_begin = blockIdx.y * BM;
+        row_end = min(g.M, row_begin + BM);
     }
-    if (tid < TL_BM) {
+    if (tid < BM) {
         const int m = row_begin + tid;
         int ra = -1, rc = -1;
         if (m < row_end) {
@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         const int row = c >> 3, kc = (c & 7) * 8;
         a_ok[i] = false;
         a_src[i] = g.A;
-        if (i < 2) {
+        if (i < BM / 32) {
             const int ra = rows_a[row];
             a_ok[i] = ra >= 0;
             a_src[i] = g.A + (size_t)(ra >= 0 ? ra : 0) * g.lda + kc;
@@ -151,10 +151,10 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
             const int kc = ((tid + 256 * i) & 7) * 8;
             const bool in = k0 + kc < K;
             if (FAST) {
-                if (i < 2) a_reg[i] = *reinterpret_cast<const u32x4_t*>(a_src[i] + k0);
+                if (i < BM / 32) a_reg[i] = *reinterpret_cast<const u32x4_t*>(a_src[i] + k0);
                 w_reg[i] = *reinterpret_cast<const u32x4_t*>(w_src[i] + k0);
             } else {
-                if (i < 2) a_reg[i] = (in && a_ok[i]) ? *reinterpret_cast<const u32x4_t*>(a_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
+                if (i < BM / 32) a_reg[i] = (in && a_ok[i]) ? *reinterpret_cast<const u32x4_t*>(a_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
                 w_reg[i] = (in && w_ok[i]) ? *reinterpret_cast<const u32x4_t*>(w_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
             }
         }
@@ -164,7 +164,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         for (int i = 0; i < 4; ++i) {
             const int c = tid + 256 * i;
             const int row = c >> 3, kc = (c & 7) * 8;
-            if (i < 2) *reinterpret_cast<u32x4_t*>(&As[buf * TL_BM * TL_LD + row * TL_LD + kc]) = a_reg[i];
+            if (i < BM / 32) *reinterpret_cast<u32x4_t*>(&As[buf * BM * TL_LD + row * TL_LD + kc]) = a_reg[i];
             *reinterpret_cast<u32x4_t*>(&Ws[buf * TL_BN * TL_LD + row * TL_LD + kc]) = w_reg[i];
         }
     };
@@ -180,66 +180,71 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         else
             w_row[f] = 64 * wn + 16 * f + lr;
     }
-    f32x4_t acc[4][2], total[SPLIT ? 4 : 1][SPLIT ? 2 : 1];
+    constexpr int TT = BM / 32;   // 16-row tiles a wave holds
+    f32x4_t acc[4][TT], total[SPLIT ? 4 : 1][SPLIT ? TT : 1];
 #pragma unroll
     for (int f = 0; f < 4; ++f)
 #pragma unroll
-        for (int t = 0; t < 2; ++t) acc[f][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int t = 0; t < TT; ++t) acc[f][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
     const int steps_total = (K + 31) >> 5;
     const int per = (steps_total + g.ks - 1) / g.ks;   // 32-wide steps in a run
     int until_fold = per;                                // steps left in the current run
     bool first_run = true;
 
     if constexpr (FAST) {
-        const int n_tiles = K / TL_BK, tiles_per_run = per / 2;
-        int until = tiles_per_run;
-        // one tile (both 32-wide steps) out of LDS half `buf`, a constant where it is called
-        auto multiply = [&](auto buf_c) {
-            constexpr int buf = decltype(buf_c)::value;
-#pragma unroll
-            for (int kk = 0; kk < TL_BK; kk += 32) {
-                bf16x8_t wf[4], af[2];
-#pragma unroll
-                for (int f = 0; f < 4; ++f)
-                    wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[buf * TL_BN * TL_LD + w_row[f] * TL_LD + kk + lk]));
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    af[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[buf * TL_BM * TL_LD + (32 * wm + 16 * t + lr) * TL_LD + kk + lk]));
-#pragma unroll
-                for (int f = 0; f < 4; ++f)
-#pragma unroll
-                    for (int t = 0; t < 2; ++t) acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[t], acc[f][t], 0, 0, 0);
-            }
-        };
+        // runs of whole tiles, an even number of them a run (so a tile's LDS half is known where it is written down):
+        // the loop over a run's tiles carries nothing but the accumulators, the runs are joined between the loops
+        const int n_tiles = K / TL_BK;
+        const int tiles_per_run = SPLIT ? per / 2 : n_tiles;
         auto tile = [&](int t, auto buf_c) {
             constexpr int buf = decltype(buf_c)::value;
             if (t + 1 < n_tiles) store_lds(buf ^ 1);
             if (t + 2 < n_tiles) load_global((t + 2) * TL_BK);
-            if (SPLIT && until == 0) {
-                // a run of K ends: its sum joins the runs before it, in run order
+#pragma unroll
+            for (int kk = 0; kk < TL_BK; kk += 32) {
+                bf16x8_t wf[4], af[TT];
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+                    wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[buf * TL_BN * TL_LD + w_row[f] * TL_LD + kk + lk]));
+#pragma unroll
+                for (int q = 0; q < TT; ++q)
+                    af[q] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[buf * BM * TL_LD + (BM / 2 * wm + 16 * q + lr) * TL_LD + kk + lk]));
 #pragma unroll
                 for (int f = 0; f < 4; ++f)
 #pragma unroll
-                    for (int q = 0; q < 2; ++q) {
-                        if (first_run) total[f][q] = acc[f][q];
-                        else total[f][q] = f32x4_t{total[f][q][0] + acc[f][q][0], total[f][q][1] + acc[f][q][1],
-                                                   total[f][q][2] + acc[f][q][2], total[f][q][3] + acc[f][q][3]};
-                        acc[f][q] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-                    }
-                first_run = false;
-                until = tiles_per_run;
+                    for (int q = 0; q < TT; ++q) acc[f][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[q], acc[f][q], 0, 0, 0);
             }
-            multiply(buf_c);
-            --until;
             __syncthreads();
         };
         load_global(0);
         store_lds(0);
         if (n_tiles > 1) load_global(TL_BK);
         __syncthreads();
-        for (int t = 0; t < n_tiles; t += 2) {
-            tile(t, std::integral_constant<int, 0>{});
-            if (t + 1 < n_tiles) tile(t + 1, std::integral_constant<int, 1>{});
+        int t = 0;
+        for (int run_end = tiles_per_run;; run_end += tiles_per_run) {
+            const int stop = min(run_end, n_tiles);
+            for (; t + 1 < stop; t += 2) {
+                tile(t, std::integral_constant<int, 0>{});
+                tile(t + 1, std::integral_constant<int, 1>{});
+            }
+            if (t < stop) {     // an odd last tile (only when K is one run)
+                tile(t, std::integral_constant<int, 0>{});
+                ++t;
+            }
+            if (t >= n_tiles) break;
+            if (SPLIT) {
+                // a run of K ends: its sum joins the runs before it, in run order
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+#pragma unroll
+                    for (int q = 0; q < TT; ++q) {
+                        if (first_run) total[f][q] = acc[f][q];
+                        else total[f][q] = f32x4_t{total[f][q][0] + acc[f][q][0], total[f][q][1] + acc[f][q][1],
+                                                   total[f][q][2] + acc[f][q][2], total[f][q][3] + acc[f][q][3]};
+                        acc[f][q] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                    }
+                first_run = false;
+            }
         }
     } else {
     load_global(0);
@@ -256,7 +261,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
 #pragma unroll
                     for (int f = 0; f < 4; ++f)
 #pragma unroll
-                        for (int t = 0; t < 2; ++t) {
+                        for (int t = 0; t < TT; ++t) {
                             if (first_run) total[f][t] = acc[f][t];
                             else total[f][t] = f32x4_t{total[f][t][0] + acc[f][t][0], total[f][t][1] + acc[f][t][1],
                                                        total[f][t][2] + acc[f][t][2], total[f][t][3] + acc[f][t][3]};
@@ -265,16 +270,16 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
                     first_run = false;
                     until_fold = per;
                 }
-                bf16x8_t wf[4], af[2];
+                bf16x8_t wf[4], af[TT];
 #pragma unroll
                 for (int f = 0; f < 4; ++f) wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[w_row[f] * TL_LD + kk + lk]));
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    af[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[(32 * wm + 16 * t + lr) * TL_LD + kk + lk]));
+                for (int t = 0; t < TT; ++t)
+                    af[t] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[(BM / 2 * wm + 16 * t + lr) * TL_LD + kk + lk]));
 #pragma unroll
                 for (int f = 0; f < 4; ++f)
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[t], acc[f][t], 0, 0, 0);
+                    for (int t = 0; t < TT; ++t) acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[t], acc[f][t], 0, 0, 0);
                 --until_fold;
             }
         }
@@ -289,7 +294,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
 #pragma unroll
         for (int f = 0; f < 4; ++f)
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < TT; ++t)
                 acc[f][t] = f32x4_t{total[f][t][0] + acc[f][t][0], total[f][t][1] + acc[f][t][1], total[f][t][2] + acc[f][t][2],
                                     total[f][t][3] + acc[f][t][3]};
     }
@@ -297,8 +302,8 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     // acc[f][t][i]: feature (tile f) 4*(lane/16) + i, row 32*wm + 16*t + lane%16
     const int fq = 4 * (lane >> 4);
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const int rc = rows_c[32 * wm + 16 * t + lr];
+    for (int t = 0; t < TT; ++t) {
+        const int rc = rows_c[BM / 2 * wm + 16 * t + lr];
         if (rc < 0) continue;
         TC* crow = (TC*)g.C + (size_t)rc * g.ldc;
         if (EPI == TL_SWIGLU) {
@@ -328,12 +333,14 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
 
 template <int EPI, typename TC, bool GROUPED, bool SPLIT>
 static void tile_launch_fast(const TileArgs& g, dim3 grid, hipStream_t stream) {
-    // the lean loop needs whole 64-wide tiles and runs that end on them
+    // the lean loop needs whole 64-wide tiles and runs of an even number of them
     const int steps = (g.K + 31) / 32, per = (steps + g.ks - 1) / g.ks;
-    if (g.K % TL_BK == 0 && (!SPLIT || per % 2 == 0))
-        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true>), grid, dim3(256), 0, stream, g);
-    else
-        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, false>), grid, dim3(256), 0, stream, g);
+    if (g.K % TL_BK == 0 && (!SPLIT || per % 4 == 0)) {
+        if (g.bm == 128) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true, 128>), grid, dim3(256), 0, stream, g);
+        else hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true, 64>), grid, dim3(256), 0, stream, g);
+    } else {
+        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, false, 64>), grid, dim3(256), 0, stream, g);
+    }
 }
 
 template <int EPI, typename TC>
@@ -356,9 +363,14 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
-    TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
-               w_group_stride, up_offset, (M + TL_BM - 1) / TL_BM, ks};
     if (ks != 1 && ks != 2 && ks != 4 && ks != 8) return -2;
+    // 128-row tiles (each wave 64 x 64: fewer operand reads a product) where rows are many and the lean loop runs
+    const int steps = (K + 31) / 32, per = (steps + ks - 1) / ks;
+    const bool lean = K % TL_BK == 0 && (ks == 1 || per % 4 == 0);
+    const bool many = !grouped && M > 64;   // (measured: the routed products gain nothing from it)
+    const int bm = lean && many ? 128 : 64;
+    TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
+               w_group_stride, up_offset, (M + bm - 1) / bm, ks, bm};
     const int feats = epi == TL_SWIGLU ? 64 : 128;
     dim3 grid((N + feats - 1) / feats, grouped ? max_tiles : g.m_tiles, 1);
     if (grid.y > 65535) return -2;
