@@ -334,6 +334,7 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         engine = Engine.load(folder, dtype="float32", kv_tokens=64, page_tokens=4, max_requests=3)
         needs = engine.model.cache_needs()
         assert [type(n).__name__ for n in needs] == ["KVNeed", "StateNeed", "KVNeed", "StateNeed"]
+        assert not engine.graphs, "a part that does not say graph_safe must keep the engine from recording graphs"
         weights, _ = {}, None
         from safetensors import safe_open
         with safe_open(str(folder / "model.safetensors"), framework="pt") as f:
