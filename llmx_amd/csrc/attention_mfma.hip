@@ -259,23 +259,26 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
     if (key_begin >= key_end) return;
     int pages[8], subs[8], pages_next[8], subs_next[8];
     locate(pages, subs);
-    bf16x8_t kf[2][QS], kf_next[2][QS];
-    load_keys(pages, subs, 0, kf);
+    // Two chunks' loads are always on their way: keys in two register sets that take turns, values in two more.  The
+    // first two value chunks of a segment are asked for before its scores are formed, the first two key chunks of the
+    // next segment while its last values are multiplied.
+    bf16x8_t kf_a[2][QS], kf_b[2][QS];
+    load_keys(pages, subs, 0, kf_a);
+    load_keys(pages, subs, 1, kf_b);
     for (int seg0 = key_begin; seg0 < key_end; seg0 += AM_SEG) {
         locate(pages_next, subs_next);   // the next segment's pages are looked up while this one is worked on
+        bf16x8_t vf_a[DT], vf_b[DT];
+        load_values(pages, subs, 0, vf_a);
+        load_values(pages, subs, 1, vf_b);
         f32x4_t s[8];
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            if (v < 3) load_keys(pages, subs, v + 1, kf_next);
-            else load_keys(pages_next, subs_next, 0, kf_next);
-            chunk_scores<DT>(kf, qf, s[2 * v], s[2 * v + 1]);
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int q = 0; q < QS; ++q) kf[u][q] = kf_next[u][q];
-        }
-        bf16x8_t vf[DT], vf_next[DT];
-        load_values(pages, subs, 0, vf);
+        chunk_scores<DT>(kf_a, qf, s[0], s[1]);
+        load_keys(pages, subs, 2, kf_a);
+        chunk_scores<DT>(kf_b, qf, s[2], s[3]);
+        load_keys(pages, subs, 3, kf_b);
+        chunk_scores<DT>(kf_a, qf, s[4], s[5]);
+        load_keys(pages_next, subs_next, 0, kf_a);
+        chunk_scores<DT>(kf_b, qf, s[6], s[7]);
+        load_keys(pages_next, subs_next, 1, kf_b);
         float m, l;
         bf16x8_t pf[4];
         bool all_in = true;
@@ -293,15 +296,12 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
         f32x4_t o[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            if (v < 3) load_values(pages, subs, v + 1, vf_next);
-            chunk_values<DT>(vf, pf[v], o);
-            if (v < 3) {
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) vf[dt] = vf_next[dt];
-            }
-        }
+        chunk_values<DT>(vf_a, pf[0], o);
+        load_values(pages, subs, 2, vf_a);
+        chunk_values<DT>(vf_b, pf[1], o);
+        load_values(pages, subs, 3, vf_b);
+        chunk_values<DT>(vf_a, pf[2], o);
+        chunk_values<DT>(vf_b, pf[3], o);
         if constexpr (PARTIAL) {
             if (col_ok) {
                 const size_t at = (size_t)(slot + seg0 / AM_SEG - seg_first) * 16 + c;
