@@ -323,7 +323,8 @@ def attention_case(T_lens, Hq, Hkv, D, R, page, dtype, window=0, shuffle_seed=0,
 
 
 @pytest.mark.parametrize("lens,Hq,Hkv,D,R,page", [((1, 2, 5), 4, 2, 16, 8, 4), ((37, 70), 6, 1, 24, 24, 8), ((130,), 8, 2, 64, 32, 16),
-                                                  ((200, 3), 12, 2, 128, 64, 16), ((33,), 2, 2, 48, 0, 16)])
+                                                  ((200, 3), 12, 2, 128, 64, 16), ((33,), 2, 2, 48, 0, 16), ((150, 40), 4, 2, 176, 32, 32),
+                                                  ((140,), 2, 1, 256, 64, 48)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_with_rope_and_pages(lens, Hq, Hkv, D, R, page, dtype):
     got, want = attention_case(lens, Hq, Hkv, D, R, page, dtype)
@@ -346,7 +347,8 @@ def test_attention_split_context(lens, Hq, Hkv, D):
         assert (g - u).abs().max() <= 1.2e-2 * u.abs().max()
 
 
-@pytest.mark.parametrize("L,Hq,Hkv,D,window", [(700, 12, 2, 128, 0), (131, 4, 4, 64, 0), (1000, 6, 1, 48, 0), (900, 8, 2, 64, 300)])
+@pytest.mark.parametrize("L,Hq,Hkv,D,window", [(700, 12, 2, 128, 0), (131, 4, 4, 64, 0), (1000, 6, 1, 48, 0), (900, 8, 2, 64, 300),
+                                               (300, 4, 2, 160, 0), (270, 2, 1, 256, 0), (200, 3, 3, 16, 0)])
 def test_attention_row_is_the_same_bits_alone_or_in_a_tile(L, Hq, Hkv, D, window):
     """The matrix-core kernel gives a row the same bits as a single decoded row (its context shared out over several
     items, or not) and as one of 16 rows of a prompt tile."""

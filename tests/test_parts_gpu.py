@@ -205,6 +205,114 @@ def test_routed_experts_and_dense_glu_parts(dtype, T):
 
 
 # ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_position_encoding_defined_here_serves_the_attention_part(dtype):
+    """Another position encoding (positions squeezed by a factor before the rotation, over the whole head), registered
+    from outside the framework: the attention part takes it by name."""
+    from llmx_amd.parts import LayerCache, PartSpec, build_part
+    from llmx_amd.parts.base import PositionEncoding, register, unregister
+
+    def squeezed_tables(n, R, theta, factor):
+        i = torch.arange(R // 2, dtype=torch.float64)
+        freq = 1.0 / theta ** (2.0 * i / R)
+        angle = (torch.arange(n, dtype=torch.float64) / factor)[:, None] * freq[None, :]
+        return torch.cos(angle), torch.sin(angle)
+
+    class SqueezedRotary(PositionEncoding):
+        def __init__(self, params, prefix, c):
+            super().__init__(params, prefix, c)
+            self.R = int(params["head_dim"])
+            cos, sin = squeezed_tables(c.max_positions, self.R, float(params["theta"]), float(params["factor"]))
+            self.cos_sin = torch.cat([cos, sin], dim=1).float().to(c.device)
+
+        def rotation(self):
+            return self.cos_sin, self.R
+
+    register("position", "toy_squeezed_rotary", SqueezedRotary, replace=True)
+    try:
+        E, heads, kv_heads, D, L, page = 32, 4, 2, 16, 29, 4
+        params = {"hidden": E, "heads": heads, "kv_heads": kv_heads, "head_dim": D, "qk_norm": "none", "eps": 1e-5, "window": None,
+                  "position": PartSpec("toy_squeezed_rotary", {"head_dim": D, "theta": 100.0, "factor": 4.0})}
+        att = build_part("mixer", PartSpec("attention", params, "a."), ctx(dtype))
+        w = {s.name: rnd(*s.shape, scale=0.3, seed=i).to(dtype) for i, s in enumerate(att.tensor_specs(set()))}
+        att.load({k: v.to(DEV) for k, v in w.items()})
+        cache = LayerCache(group=0, k=torch.zeros(8, kv_heads, page, D, dtype=dtype, device=DEV),
+                           v=torch.zeros(8, kv_heads, D, page, dtype=dtype, device=DEV), writes=True)
+        h = rnd(L, E, seed=11).to(dtype)
+        step = make_step(dtype, [(0, L, 0)], [[[7, 6, 5, 4, 3, 2, 1, 0]]], page)
+        out = torch.zeros(L, E, dtype=torch.float32, device=DEV)
+        att.forward(step, h.to(DEV), out, False, cache)
+        rt = None if dtype == torch.float32 else torch.bfloat16
+        hd = h.double()
+        q = (hd @ w["a.q_proj.weight"].double().T).view(L, heads, D)
+        k = (hd @ w["a.k_proj.weight"].double().T).view(L, kv_heads, D)
+        v = (hd @ w["a.v_proj.weight"].double().T).view(L, kv_heads, D)
+        cos, sin = squeezed_tables(L, D, 100.0, 4.0)
+        q, k = pm.apply_partial_rope(q, cos, sin, D), pm.apply_partial_rope(k, cos, sin, D)
+        q, k, v = (pm._rounded(t, rt) for t in (q, k, v))
+        o = pm._rounded(pm.causal_attention(q, k, v, None).reshape(L, heads * D), rt)
+        want = o @ w["a.o_proj.weight"].double().T
+        assert (out.double().cpu() - want).abs().max() <= (3e-5 if dtype == torch.float32 else 2e-2) * want.abs().max()
+    finally:
+        unregister("position", "toy_squeezed_rotary")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_routed_feed_forward_defined_here(dtype):
+    """A feed-forward with routing of its own (the expert is chosen by the row's position, one expert a row, weight 1),
+    made outside the framework from its grouped products: registered, built, loaded by tensor name and run."""
+    from llmx_amd import ops
+    from llmx_amd.parts import PartSpec, TensorSpec, build_part
+    from llmx_amd.parts.base import FeedForward, register, unregister
+
+    class ByPosition(FeedForward):
+        def __init__(self, params, prefix, c):
+            super().__init__(params, prefix, c)
+            self.E, self.X, self.F = int(params["hidden"]), int(params["experts"]), int(params["intermediate"])
+
+        def tensor_specs(self, available):
+            return [TensorSpec(self.name("up"), (self.X, 2 * self.F, self.E)), TensorSpec(self.name("down"), (self.X, self.E, self.F))]
+
+        def load(self, tensors):
+            self.up, self.down = tensors[self.name("up")], tensors[self.name("down")]
+
+        def forward(self, step, h, out, accumulate, h32=None):
+            T, X = step.rows, self.X
+            ids = (step.positions % X).to(torch.int32).view(T, 1).contiguous()
+            weights = torch.ones(T, 1, dtype=torch.float32, device=h.device)
+            i32 = lambda name, n: step.buf("toy." + name, (n,), torch.int32)
+            counts, offsets, pairs, active, n_active = i32("counts", X), i32("offsets", X + 1), i32("pairs", T), i32("active", X), i32("n", 1)
+            ops.moe_align(ids, X, counts, offsets, pairs, active, n_active)
+            act = step.buf("toy.act", (T, self.F), step.act_dtype)
+            ops.grouped_gemm(h, self.up, act, offsets, pairs, 1, ops.EPI_SWIGLU, active, n_active, token_rows=T)
+            y = step.buf("toy.y", (T, self.E), torch.float32)
+            ops.grouped_gemm(act, self.down, y, offsets, pairs, 1, ops.EPI_STORE, active, n_active, token_rows=T)
+            ops.moe_combine(out, y, ids, weights, accumulate)
+
+    register("feed_forward", "toy_by_position", ByPosition, replace=True)
+    try:
+        E, X, Fe = 40, 5, 24
+        for T, past in ((3, 0), (70, 9)):
+            ff = build_part("feed_forward", PartSpec("toy_by_position", {"hidden": E, "experts": X, "intermediate": Fe}, "t."), ctx(dtype))
+            assert not ff.graph_safe
+            w = {s.name: rnd(*s.shape, scale=0.3, seed=i).to(dtype) for i, s in enumerate(ff.tensor_specs(set()))}
+            ff.load({n: t.to(DEV) for n, t in w.items()})
+            h = rnd(T, E, seed=5).to(dtype)
+            step = make_step(dtype, [(0, T, past)])
+            base = rnd(T, E, seed=6)
+            out = base.clone().to(DEV)
+            ff.forward(step, h.to(DEV), out, True)
+            rt = None if dtype == torch.float32 else torch.bfloat16
+            want = base.double().clone()
+            for t in range(T):
+                e = (past + t) % X
+                want[t] += pm.swiglu_expert(h[t].double(), w["t.up"][e].double(), w["t.down"][e].double(), rt)
+            assert (out.double().cpu() - want).abs().max() <= (3e-5 if dtype == torch.float32 else 2e-2) * want.abs().max()
+    finally:
+        unregister("feed_forward", "toy_by_position")
+
+
+# ---------------------------------------------------------------------------
 # A toy architecture made here: layers alternate attention and a mixer that keeps a running state per request.
 ToyState = None
 
