@@ -24,6 +24,17 @@ enum : int { TL_STORE = 0, TL_ADD = 1, TL_SWIGLU = 2 };
 #define TL_BN 128
 #define TL_BK 64
 #define TL_LD 72  // padded row length in bf16 elements (144 bytes)
+#ifndef TL_STAGES
+#define TL_STAGES 2  // tiles in LDS in the lean loop: one being multiplied, the other on its way (48 KB: three workgroups a CU; measured better than deeper stages with fewer workgroups)
+#endif
+
+// Lane l of the wave: 16 bytes from base + offset (bytes, per lane) to LDS at lds + 16 l (lds the same for the whole
+// wave).  Written as an instruction of its own so that waiting for it is the kernel's business: the loop below keeps
+// two tiles' loads in flight and waits by count.
+__device__ __forceinline__ void load_to_lds(const void* base, uint32_t offset, void* lds) {
+    const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(at), "v"(offset), "s"(base) : "memory", "m0");
+}
 
 struct TileArgs {
     const bf16_t* A;
@@ -41,15 +52,15 @@ struct TileArgs {
     int bm;       // rows a workgroup covers: 64 or 128
 };
 
-// FAST: K is a multiple of 64 and the runs are an even number of 64-wide tiles, so nothing in the loop needs a bound: the tiles are
+// FAST: K is a multiple of 64 and the runs end on multiples of 64, so nothing in the loop needs a bound: the tiles are
 // loaded without conditions (a row past the tile's rows reads the first row, a feature past N the last; what they
-// produce is never stored, and a column of the product never touches another), LDS holds two tiles and a tile takes one
-// barrier: the tile after the next travels into registers while the next is written to the other half of LDS and this
-// one is multiplied.
+// produce is never stored, and a column of the product never touches another), straight into LDS, TL_STAGES deep,
+// one barrier a tile.
 template <int EPI, typename TC, bool GROUPED, bool SPLIT, bool FAST, int BM>
-__global__ void __launch_bounds__(256, BM == 128 ? 2 : 1) gemm_tile_kernel(TileArgs g) {
-    __shared__ __attribute__((aligned(16))) bf16_t As[(FAST ? 2 : 1) * BM * TL_LD];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[(FAST ? 2 : 1) * TL_BN * TL_LD];
+__global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
+    // FAST: 3 stages of unpadded 128-byte rows whose 16-byte chunks are swizzled; else one tile of padded rows
+    __shared__ __attribute__((aligned(1024))) bf16_t As[FAST ? TL_STAGES * BM * TL_BK : BM * TL_LD];
+    __shared__ __attribute__((aligned(1024))) bf16_t Ws[FAST ? TL_STAGES * TL_BN * TL_BK : TL_BN * TL_LD];
     __shared__ int rows_a[BM];
     __shared__ int rows_c[BM];
     __shared__ int tile_info[2];
@@ -120,6 +131,7 @@ __global__ void __launch_bounds__(256, BM == 128 ? 2 : 1) gemm_tile_kernel(TileA
     const int K = g.K;
     const bf16_t* a_src[4];
     const bf16_t* w_src[4];
+    uint32_t a_off[4], w_off[4];   // the same places as byte offsets from A and W (the lean loop adds them to a uniform base)
     bool a_ok[4], w_ok[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -127,10 +139,12 @@ __global__ void __launch_bounds__(256, BM == 128 ? 2 : 1) gemm_tile_kernel(TileA
         const int row = c >> 3, kc = (c & 7) * 8;
         a_ok[i] = false;
         a_src[i] = g.A;
+        a_off[i] = 0;
         if (i < BM / 32) {
             const int ra = rows_a[row];
             a_ok[i] = ra >= 0;
             a_src[i] = g.A + (size_t)(ra >= 0 ? ra : 0) * g.lda + kc;
+            a_off[i] = (uint32_t)(((size_t)(ra >= 0 ? ra : 0) * g.lda + kc) * sizeof(bf16_t));
         }
         int wr;
         if (EPI == TL_SWIGLU) {
@@ -143,6 +157,7 @@ __global__ void __launch_bounds__(256, BM == 128 ? 2 : 1) gemm_tile_kernel(TileA
             wr = min(f, g.N - 1);
         }
         w_src[i] = W + (size_t)wr * K + kc;
+        w_off[i] = (uint32_t)(((size_t)wr * K + kc) * sizeof(bf16_t));
     }
     u32x4_t a_reg[4], w_reg[4];
     auto load_global = [&](int k0) {
@@ -151,8 +166,10 @@ __global__ void __launch_bounds__(256, BM == 128 ? 2 : 1) gemm_tile_kernel(TileA
             const int kc = ((tid + 256 * i) & 7) * 8;
             const bool in = k0 + kc < K;
             if (FAST) {
-                if (i < BM / 32) a_reg[i] = *reinterpret_cast<const u32x4_t*>(a_src[i] + k0);
-                w_reg[i] = *reinterpret_cast<const u32x4_t*>(w_src[i] + k0);
+                const char* a_base = reinterpret_cast<const char*>(g.A + k0);
+                const char* w_base = reinterpret_cast<const char*>(W + k0);
+                if (i < BM / 32) a_reg[i] = *reinterpret_cast<const u32x4_t*>(a_base + a_off[i]);
+                w_reg[i] = *reinterpret_cast<const u32x4_t*>(w_base + w_off[i]);
             } else {
                 if (i < BM / 32) a_reg[i] = (in && a_ok[i]) ? *reinterpret_cast<const u32x4_t*>(a_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
                 w_reg[i] = (in && w_ok[i]) ? *reinterpret_cast<const u32x4_t*>(w_src[i] + k0) : u32x4_t{0u, 0u, 0u, 0u};
@@ -192,44 +209,90 @@ __global__ void __launch_bounds__(256, BM == 128 ? 2 : 1) gemm_tile_kernel(TileA
     bool first_run = true;
 
     if constexpr (FAST) {
-        // runs of whole tiles, an even number of them a run (so a tile's LDS half is known where it is written down):
-        // the loop over a run's tiles carries nothing but the accumulators, the runs are joined between the loops
+        // Tiles travel from global memory straight into LDS (no registers in between), TL_STAGES deep: while tile t
+        // is multiplied, the tiles after it are on their way.  A wave's load instruction fills 1 KB of LDS, lane after
+        // lane: 8 rows of 128 bytes.  Rows are not padded; instead chunk c (16 bytes) of row r sits at place
+        // c ^ ((r >> 1) & 7) of the row, so that the operand reads of 16 rows at one k fall into different banks.  The
+        // lane that fills place p of row r therefore fetches chunk p ^ ((r >> 1) & 7) of that row.
+        constexpr int A_LOADS = BM / 32, LOADS = 4 + A_LOADS;   // load instructions a wave issues per tile
         const int n_tiles = K / TL_BK;
         const int tiles_per_run = SPLIT ? per / 2 : n_tiles;
-        auto tile = [&](int t, auto buf_c) {
-            constexpr int buf = decltype(buf_c)::value;
-            if (t + 1 < n_tiles) store_lds(buf ^ 1);
-            if (t + 2 < n_tiles) load_global((t + 2) * TL_BK);
+        uint32_t w_at[4], a_at[A_LOADS];
+        const int place = lane & 7;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = 32 * wave + 8 * j + (lane >> 3);           // row of the W tile
+            const int ch = place ^ ((r >> 1) & 7);
+            int wr;
+            if (EPI == TL_SWIGLU) wr = (r < 64 ? 0 : g.up_offset) + min(n0 + (r & 63), g.N - 1);
+            else wr = min(n0 + r, g.N - 1);
+            w_at[j] = (uint32_t)(((size_t)wr * K + 8 * ch) * sizeof(bf16_t));
+        }
+#pragma unroll
+        for (int j = 0; j < A_LOADS; ++j) {
+            const int r = (BM / 4) * wave + 8 * j + (lane >> 3);     // row of the A tile
+            const int ch = place ^ ((r >> 1) & 7);
+            const int ra = rows_a[r];
+            a_at[j] = (uint32_t)(((size_t)(ra >= 0 ? ra : 0) * g.lda + 8 * ch) * sizeof(bf16_t));
+        }
+        const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+        auto issue = [&](int t, int stage) {
+            const bf16_t* wb = W + (size_t)t * TL_BK;
+            const bf16_t* ab = g.A + (size_t)t * TL_BK;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) load_to_lds(wb, w_at[j], &Ws[(stage * TL_BN + 32 * wave_u + 8 * j) * TL_BK]);
+#pragma unroll
+            for (int j = 0; j < A_LOADS; ++j) load_to_lds(ab, a_at[j], &As[(stage * BM + (BM / 4) * wave_u + 8 * j) * TL_BK]);
+        };
+        // operand reads: row `row` of a stage, chunk kk/8 + lane/16
+        int w_rd[4], a_rd[TT], w_swz[4], a_swz[TT];
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+            w_rd[f] = w_row[f] * TL_BK;
+            w_swz[f] = (w_row[f] >> 1) & 7;
+        }
+#pragma unroll
+        for (int q = 0; q < TT; ++q) {
+            const int r = BM / 2 * wm + 16 * q + lr;
+            a_rd[q] = r * TL_BK;
+            a_swz[q] = (r >> 1) & 7;
+        }
+        const int kg = lane >> 4;
+        auto multiply = [&](int stage) {
+            const bf16_t* ws = &Ws[stage * TL_BN * TL_BK];
+            const bf16_t* as = &As[stage * BM * TL_BK];
 #pragma unroll
             for (int kk = 0; kk < TL_BK; kk += 32) {
                 bf16x8_t wf[4], af[TT];
 #pragma unroll
                 for (int f = 0; f < 4; ++f)
-                    wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ws[buf * TL_BN * TL_LD + w_row[f] * TL_LD + kk + lk]));
+                    wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&ws[w_rd[f] + 8 * ((kk / 8 + kg) ^ w_swz[f])]));
 #pragma unroll
                 for (int q = 0; q < TT; ++q)
-                    af[q] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&As[buf * BM * TL_LD + (BM / 2 * wm + 16 * q + lr) * TL_LD + kk + lk]));
+                    af[q] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&as[a_rd[q] + 8 * ((kk / 8 + kg) ^ a_swz[q])]));
 #pragma unroll
                 for (int f = 0; f < 4; ++f)
 #pragma unroll
                     for (int q = 0; q < TT; ++q) acc[f][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[q], acc[f][q], 0, 0, 0);
             }
-            __syncthreads();
         };
-        load_global(0);
-        store_lds(0);
-        if (n_tiles > 1) load_global(TL_BK);
-        __syncthreads();
-        int t = 0;
+        issue(0, 0);
+#pragma unroll
+        for (int ahead = 1; ahead < TL_STAGES - 1; ++ahead)
+            if (ahead < n_tiles) issue(ahead, ahead);
+        int t = 0, stage = 0;
         for (int run_end = tiles_per_run;; run_end += tiles_per_run) {
             const int stop = min(run_end, n_tiles);
-            for (; t + 1 < stop; t += 2) {
-                tile(t, std::integral_constant<int, 0>{});
-                tile(t + 1, std::integral_constant<int, 1>{});
-            }
-            if (t < stop) {     // an odd last tile (only when K is one run)
-                tile(t, std::integral_constant<int, 0>{});
-                ++t;
+            for (; t < stop; ++t) {
+                // tile t has arrived when at most the loads of tile t+1 are still out; then everybody's have, and
+                // everybody is done with the stage that tile t+2 goes into
+                constexpr int OUT = LOADS * (TL_STAGES - 2);   // loads of the tiles after t that may still be out
+                if (t + TL_STAGES - 2 < n_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (OUT & 15) | ((OUT >> 4) << 14));
+                else __builtin_amdgcn_s_waitcnt(0x0F70);
+                __syncthreads();
+                if (t + TL_STAGES - 1 < n_tiles) issue(t + TL_STAGES - 1, stage == 0 ? TL_STAGES - 1 : stage - 1);
+                multiply(stage);
+                stage = stage == TL_STAGES - 1 ? 0 : stage + 1;
             }
             if (t >= n_tiles) break;
             if (SPLIT) {
@@ -333,9 +396,9 @@ __global__ void __launch_bounds__(256, BM == 128 ? 2 : 1) gemm_tile_kernel(TileA
 
 template <int EPI, typename TC, bool GROUPED, bool SPLIT>
 static void tile_launch_fast(const TileArgs& g, dim3 grid, hipStream_t stream) {
-    // the lean loop needs whole 64-wide tiles and runs of an even number of them
+    // the lean loop needs whole 64-wide tiles and runs that end on them
     const int steps = (g.K + 31) / 32, per = (steps + g.ks - 1) / g.ks;
-    if (g.K % TL_BK == 0 && (!SPLIT || per % 4 == 0)) {
+    if (g.K % TL_BK == 0 && (!SPLIT || per % 2 == 0)) {
         if (g.bm == 128) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true, 128>), grid, dim3(256), 0, stream, g);
         else hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true, 64>), grid, dim3(256), 0, stream, g);
     } else {
@@ -366,8 +429,8 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
     if (ks != 1 && ks != 2 && ks != 4 && ks != 8) return -2;
     // 128-row tiles (each wave 64 x 64: fewer operand reads a product) where rows are many and the lean loop runs
     const int steps = (K + 31) / 32, per = (steps + ks - 1) / ks;
-    const bool lean = K % TL_BK == 0 && (ks == 1 || per % 4 == 0);
-    const bool many = !grouped && M > 64;   // (measured: the routed products gain nothing from it)
+    const bool lean = K % TL_BK == 0 && (ks == 1 || per % 2 == 0);
+    const bool many = false;   // 128-row tiles halve the workgroups a CU holds and measured slower; the kernel keeps the variant
     const int bm = lean && many ? 128 : 64;
     TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
                w_group_stride, up_offset, (M + bm - 1) / bm, ks, bm};
