@@ -522,6 +522,170 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
     if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
 }
 
+// Lane l of the wave: 16 bytes from base + offset (bytes, per lane) to LDS at lds + 16 l (lds the same for the whole
+// wave).  An instruction of its own, so that waiting for it is the kernel's business (it waits by count).
+__device__ __forceinline__ void attention_load_to_lds(const void* base, uint32_t offset, void* lds) {
+    const uint32_t at = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(at), "v"(offset), "s"(base) : "memory", "m0");
+}
+
+// Prompt tiles of head_dim 128, the form for the sizes this engine serves: 8 waves hold 8 items of one request and one
+// KV head.  A segment's keys and values go from the pages straight into LDS (no registers in between), a whole segment
+// ahead: while segment n is worked on, segment n+1 is on its way into the other half of LDS; one barrier a segment.
+// LDS rows are not padded; the 16-byte chunks are placed so that the operand reads miss each other's banks:
+//   keys:   row = key (256 bytes), chunk c (8 dims) at place c ^ (key & 15)
+//   values: per tile of 16 keys a block of 128 dims x 32 bytes, the two chunks of dim d swapped when (d >> 3) & 1
+// and the lane that fills a place fetches the chunk that belongs there.  Per column the arithmetic is that of the
+// kernels above (the same functions on the same values).
+__global__ void __launch_bounds__(512) paged_attention_tiles128_kernel(AttnMfmaArgs a) {
+    constexpr int DT = 8, QS = 4, D = 128;
+    constexpr int K_SEG = AM_SEG * D, V_SEG = AM_SEG * D;   // elements of a segment's keys (values) in LDS
+    __shared__ __attribute__((aligned(1024))) bf16_t Ks[2 * K_SEG];
+    __shared__ __attribute__((aligned(1024))) bf16_t Vs[2 * V_SEG];
+    __shared__ int ranges[8][2];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int* it = a.items + ((size_t)blockIdx.x * 8 + wave) * AM_ITEM_INTS;
+    const int row0 = __builtin_amdgcn_readfirstlane(it[0]), n_rows = __builtin_amdgcn_readfirstlane(it[1]);
+    const int h = __builtin_amdgcn_readfirstlane(it[2]);
+    const int lead_row = a.items[(size_t)blockIdx.x * 8 * AM_ITEM_INTS];   // the first item is never a filler
+    const int lead_head = a.items[(size_t)blockIdx.x * 8 * AM_ITEM_INTS + 2];
+    const int bt = a.page_tokens, Hkv = a.n_kv_heads;
+    const int kvh = lead_head / (a.n_heads / Hkv);
+    const int* table = a.tables + (size_t)a.row_entry[lead_row] * a.max_blocks;
+    const int c = lane & 15, g = lane >> 4;
+    const bool col_ok = c < n_rows;
+    const int t = row0 + (col_ok ? c : 0);
+    int p_col = 0, lo_col = 0, key_begin = 0, key_end = 0, p_first = -1, lo_last = 0;
+    if (n_rows > 0) {
+        p_col = a.pos[t];
+        p_first = __builtin_amdgcn_readfirstlane(a.pos[row0]);
+        const int p_last = __builtin_amdgcn_readfirstlane(a.pos[row0 + n_rows - 1]);
+        lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
+        const int lo_first = (a.window > 0 && p_first - a.window + 1 > 0) ? p_first - a.window + 1 : 0;
+        lo_last = (a.window > 0 && p_last - a.window + 1 > 0) ? p_last - a.window + 1 : 0;
+        key_begin = (lo_first / AM_SEG) * AM_SEG;
+        key_end = p_last + 1;
+    }
+    if (lane == 0) {
+        ranges[wave][0] = n_rows > 0 ? key_begin : 0x7fffffff;
+        ranges[wave][1] = key_end;
+    }
+    __syncthreads();
+    int bb = 0x7fffffff, be = 0;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+        bb = min(bb, ranges[w][0]);
+        be = max(be, ranges[w][1]);
+    }
+    const int block_begin = __builtin_amdgcn_readfirstlane(bb), block_end = __builtin_amdgcn_readfirstlane(be);
+
+    bf16x8_t qf[QS];
+#pragma unroll
+    for (int s = 0; s < QS; ++s) {
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        if (col_ok) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + 32 * s + 8 * g);
+        qf[s] = __builtin_bit_cast(bf16x8_t, v);
+    }
+    f32x4_t o_tot[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o_tot[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_tot = -INFINITY, l_tot = 0.0f;
+
+    // A segment's loads: 32 instructions for its keys (4 keys each: lane l is key l / 16, place l % 16) and 32 for its
+    // values (32 dims of one tile each: lane l is dim l / 2, place l % 2), 8 of them a wave: wave w brings the keys of
+    // tile w (4 instructions) and the values of tile w (4 instructions).  The tile's page comes from the block table.
+    const uint32_t k_lane = (uint32_t)((((lane >> 4) * D) + 8 * ((lane & 15) ^ (lane >> 4))) * sizeof(bf16_t));   // + 4 j keys: see below
+    auto issue = [&](int seg0, int buf) {
+        const int key0 = seg0 + 16 * wave;                   // the wave's tile
+        const int page = key0 < block_end ? __builtin_amdgcn_readfirstlane(table[key0 / bt]) : -1;
+        const int pg = page < 0 ? 0 : page;                  // a tile past the keys reads page 0: its keys are masked
+        const int sub = key0 % bt;
+        const bf16_t* kb = a.k_cache + (((size_t)pg * Hkv + kvh) * bt + sub) * D;
+        const bf16_t* vb = a.v_cache + ((size_t)pg * Hkv + kvh) * D * bt + sub;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // keys 4 j .. 4 j + 3 of the tile: lane is key 4 j + l / 16 (row 16 wave + that), place l % 16 holds chunk
+            // place ^ (key & 15)
+            const int key = 4 * j + (lane >> 4);
+            const uint32_t off = (uint32_t)((key * D + 8 * ((lane & 15) ^ key)) * sizeof(bf16_t));
+            attention_load_to_lds(kb, off, &Ks[buf * K_SEG + (16 * wave + 4 * j) * D]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            // dims 32 j .. 32 j + 31 of the tile: lane is dim 32 j + l / 2, place l % 2 holds chunk place ^ ((dim >> 3) & 1)
+            const int d = 32 * j + (lane >> 1);
+            const int half = (lane & 1) ^ ((d >> 3) & 1);
+            const uint32_t off = (uint32_t)((d * bt + 8 * half) * sizeof(bf16_t));
+            attention_load_to_lds(vb, off, &Vs[buf * V_SEG + wave * 16 * D + 32 * j * 16]);
+        }
+    };
+    (void)k_lane;
+    // operand reads
+    int k_rd[2][QS];   // tile u of a chunk: key 16 u + c, dims 32 s + 8 g: chunk 4 s + g at place (4 s + g) ^ c
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int s = 0; s < QS; ++s) k_rd[u][s] = (16 * u + c) * D + 8 * ((4 * s + g) ^ c);
+    // values: tile tl, dim d = 16 dt + c, keys 4 g .. 4 g + 3: chunk g / 2 at place (g / 2) ^ ((d >> 3) & 1), 8 bytes g % 2 of it
+    int v_rd[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const int d = 16 * dt + c;
+        v_rd[dt] = d * 16 + 8 * ((g >> 1) ^ ((d >> 3) & 1)) + 4 * (g & 1);
+    }
+
+    if (block_begin >= block_end) return;
+    issue(block_begin, 0);
+    int buf = 0;
+    for (int seg0 = block_begin; seg0 < block_end; seg0 += AM_SEG) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);     // this wave's part of the segment has arrived
+        __syncthreads();                         // everybody's has, and nobody reads the other half any more
+        if (seg0 + AM_SEG < block_end) issue(seg0 + AM_SEG, buf ^ 1);
+        if (seg0 >= key_begin && seg0 < key_end) {
+            const bf16_t* ks = &Ks[buf * K_SEG];
+            const bf16_t* vs = &Vs[buf * V_SEG];
+            f32x4_t s[8];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                bf16x8_t kf[2][QS];
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int q = 0; q < QS; ++q)
+                        kf[u][q] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&ks[32 * v * D + k_rd[u][q]]));
+                chunk_scores<DT>(kf, qf, s[2 * v], s[2 * v + 1]);
+            }
+            float m, l;
+            bf16x8_t pf[4];
+            if (seg0 + AM_SEG - 1 <= p_first && seg0 >= lo_last) {
+                segment_softmax<false>(s, 0xffffffffu, a.scale, m, l, pf);   // every key counts for every column
+            } else {
+                segment_softmax<true>(s, segment_mask(seg0, g, col_ok, lo_col, p_col, key_end), a.scale, m, l, pf);
+            }
+            f32x4_t o[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                bf16x8_t vf[DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(&vs[(2 * v) * 16 * D + v_rd[dt]]);
+                    const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(&vs[(2 * v + 1) * 16 * D + v_rd[dt]]);
+                    const u32x4_t x = {v0[0], v0[1], v1[0], v1[1]};
+                    vf[dt] = __builtin_bit_cast(bf16x8_t, x);
+                }
+                chunk_values<DT>(vf, pf[v], o);
+            }
+            fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
+        }
+        buf ^= 1;
+    }
+    if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
+}
+
 // merge: one block per output (row, head).  merge item: {row, head, first_slot, column}.  The row's segments are folded
 // in key order with the formula the attention kernel uses for a tile's segments.  The fold's weights depend on the
 // segments' maxima only, so they are formed for 512 segments at a time by all threads (a prefix maximum, then
@@ -646,7 +810,8 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
     if (WIDE && tid + 128 < D) out[((size_t)t * n_heads + h) * D + tid + 128] = f32_to_bf16(O[WIDE ? 1 : 0] * inv);
 }
 
-// `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 4: one workgroup each 4),
+// `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 8: one workgroup each 8, or
+// each 4 for head sizes other than 128),
 // then the n_direct items that fold their segments themselves (slot < 0), then the n_partial items that write them
 // (slot >= 0).
 extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
@@ -655,7 +820,7 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
                                          void* out, float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
                                          int page_tokens, int max_blocks, int window, hipStream_t stream) {
     if (n_shared + n_direct + n_partial <= 0) return 0;
-    if (n_shared % 4) return -2;
+    if (n_shared % 8) return -2;
     if (head_dim % 16 || head_dim > AM_MAX_D || page_tokens % 16 || n_heads % n_kv_heads) return -2;
     AttnMfmaArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pos, row_entry, tables, items, (bf16_t*)out, part_o,
                    part_ml, scale, n_direct, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
@@ -669,7 +834,9 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
     switch (head_dim / 16) {
 #define AM_CASE(DT)                                                                                                          \
     case DT:                                                                                                                 \
-        if (n_shared > 0) hipLaunchKernelGGL((paged_attention_tiles_kernel<DT>), dim3(n_shared / 4), block, 0, stream, sh);             \
+        if (n_shared > 0 && DT == 8 && page_tokens % 16 == 0)                                                               \
+            hipLaunchKernelGGL(paged_attention_tiles128_kernel, dim3(n_shared / 8), dim3(512), 0, stream, sh);                          \
+        else if (n_shared > 0) hipLaunchKernelGGL((paged_attention_tiles_kernel<DT>), dim3(n_shared / 4), block, 0, stream, sh);        \
         if (n_direct > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, false>), dim3((n_direct + 3) / 4), block, 0, stream, a);  \
         if (n_partial > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, true>), dim3((n_partial + 3) / 4), block, 0, stream, b); \
         break;
