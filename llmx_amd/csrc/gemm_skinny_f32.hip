@@ -94,6 +94,98 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
     }
 }
 
+// Many rows: a workgroup takes 4 strips (64 features) and 64 rows, so that a row's values, once in registers, meet 4
+// strips of W instead of one (the rows' traffic is what bounds this product).  Per output element the instruction, the
+// operands' roles, the steps' order and the waves' order are those of the kernel above: the same bits.
+template <int KS>
+__global__ void __launch_bounds__(64 * KS) gemm_rows_f32_kernel(SkinnyF32Args g) {
+    constexpr int NS = 4, MT = 4;
+    __shared__ float red[KS > 1 ? KS : 1][NS * MT][256];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, kg = lane >> 4;
+    const int n0 = blockIdx.x * 16 * NS;
+    const int K = g.K;
+    const int steps_total = (K + 15) >> 4;
+    const int per_slice = (steps_total + gridDim.z - 1) / gridDim.z;
+    const int slice_begin = blockIdx.z * per_slice, slice_end = min(steps_total, slice_begin + per_slice);
+    const int per = (per_slice + KS - 1) / KS;
+    const int s_begin = min(slice_end, slice_begin + wave * per), s_end = min(slice_end, s_begin + per);
+    float* C = g.C + (size_t)blockIdx.z * g.slice_stride;
+    const float* wp[NS];
+#pragma unroll
+    for (int ns = 0; ns < NS; ++ns) wp[ns] = g.W + (size_t)min(n0 + 16 * ns + r, g.N - 1) * K + kg * 4;
+    const int m0 = blockIdx.y * 16 * MT;
+    const float* ap[MT];
+    bool a_in[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = m0 + t * 16 + r;
+        a_in[t] = m < g.M;
+        ap[t] = g.A + (size_t)(a_in[t] ? m : 0) * g.lda + kg * 4;
+    }
+    f32x4_t acc[NS][MT];
+#pragma unroll
+    for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[ns][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s = s_begin; s < s_end; s += 2) {
+        f32x4_t wf[2][NS], af[2][MT];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int k = (s + u) * 16 + kg * 4;
+            const bool in = (s + u) < s_end && k < K;
+#pragma unroll
+            for (int ns = 0; ns < NS; ++ns)
+                wf[u][ns] = in ? *reinterpret_cast<const f32x4_t*>(wp[ns] + (size_t)(s + u) * 16) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                af[u][t] = (in && a_in[t]) ? *reinterpret_cast<const f32x4_t*>(ap[t] + (size_t)(s + u) * 16) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) acc[ns][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[u][ns][i], af[u][t][i], acc[ns][t], 0, 0, 0);
+    }
+    if (KS > 1) {
+#pragma unroll
+        for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4_t*>(&red[wave][ns * MT + t][lane * 4]) = acc[ns][t];
+        __syncthreads();
+    }
+    // the waves' sums added in wave order; wave q takes the tiles q, q + KS, ... of the workgroup's 16
+    for (int tile = wave; tile < NS * MT; tile += KS) {
+        const int ns = tile / MT, t = tile % MT;
+        f32x4_t v = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (KS > 1) {
+            v = *reinterpret_cast<f32x4_t*>(&red[0][tile][lane * 4]);
+#pragma unroll
+            for (int w = 1; w < KS; ++w) {
+                const f32x4_t o = *reinterpret_cast<f32x4_t*>(&red[w][tile][lane * 4]);
+                v = f32x4_t{v[0] + o[0], v[1] + o[1], v[2] + o[2], v[3] + o[3]};
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < NS; ++a)
+#pragma unroll
+                for (int b = 0; b < MT; ++b)
+                    if (a == ns && b == t) v = acc[a][b];
+        }
+        const int m = m0 + t * 16 + r;
+        if (m >= g.M) continue;
+        float* c = C + (size_t)m * g.ldc + n0 + 16 * ns + 4 * kg;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (n0 + 16 * ns + 4 * kg + i >= g.N) continue;
+            c[i] = g.add ? c[i] + v[i] : v[i];
+        }
+    }
+}
+
 // K a multiple of 4, rows 16-byte aligned.  ks: 1, 2, 4, 8 or 16 waves share a strip's K.  slices > 1: K's steps are
 // cut into `slices` runs first, run z written to C + z * slice_stride (no add then); the caller adds the runs in order.
 extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, int M, int N, int K, int lda, int ldc, int add, int ks,
@@ -104,6 +196,17 @@ extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, in
     int chunks = (M + 63) / 64;
     if (chunks > 1024) chunks = 1024;
     const dim3 grid((N + 15) / 16, M <= 64 ? 1 : chunks, slices);
+    if (M > 64 && N >= 64 && ks <= 8) {
+        const dim3 wide((N + 63) / 64, (M + 63) / 64, slices);
+        if (wide.y > 65535) return -2;
+        switch (ks) {
+            case 1: hipLaunchKernelGGL(gemm_rows_f32_kernel<1>, wide, dim3(64), 0, stream, g); break;
+            case 2: hipLaunchKernelGGL(gemm_rows_f32_kernel<2>, wide, dim3(128), 0, stream, g); break;
+            case 4: hipLaunchKernelGGL(gemm_rows_f32_kernel<4>, wide, dim3(256), 0, stream, g); break;
+            default: hipLaunchKernelGGL(gemm_rows_f32_kernel<8>, wide, dim3(512), 0, stream, g); break;
+        }
+        return LLMX_CHECK_LAUNCH();
+    }
 #define SKF_LAUNCH(KS, MT) hipLaunchKernelGGL((gemm_skinny_f32_kernel<KS, MT>), grid, dim3(64 * KS), 0, stream, g)
 #define SKF_MT(KS) do { if (M <= 16) SKF_LAUNCH(KS, 1); else if (M <= 32) SKF_LAUNCH(KS, 2); else SKF_LAUNCH(KS, 4); } while (0)
     switch (ks) {
