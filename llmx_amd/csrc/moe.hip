@@ -234,12 +234,99 @@ __global__ void __launch_bounds__(1024) moe_align_small_kernel(const int* __rest
     align_in_block(pair_expert, n_pairs, n_experts, cnt, offs, counts, offsets, list, active, n_active);
 }
 
+// Many pairs, with scratch [ceil(n_pairs / 1024)][n_experts] (at most 1024 experts): the pairs are cut into chunks of
+// 1024; (1) each chunk counts its pairs per expert in LDS, (2) one workgroup turns the chunks' counts into the experts'
+// offsets and every chunk's first place within each expert's run, (3) each chunk places its pairs: a pair's place is the
+// chunk's first place plus the number of earlier pairs of its expert in the chunk.  Every expert's pairs stay in
+// increasing order; nothing depends on the order in which atomics land.
+__global__ void __launch_bounds__(1024) moe_chunk_count_kernel(const int* __restrict__ ids, int n_pairs, int n_experts, int* __restrict__ chunk_counts) {
+    __shared__ int cnt[1024];
+    const int tid = threadIdx.x, p = blockIdx.x * 1024 + tid;
+    if (tid < n_experts) cnt[tid] = 0;
+    __syncthreads();
+    const int e = p < n_pairs ? ids[p] : -1;
+    if (e >= 0 && e < n_experts) atomicAdd(&cnt[e], 1);
+    __syncthreads();
+    if (tid < n_experts) chunk_counts[(size_t)blockIdx.x * n_experts + tid] = cnt[tid];
+}
+
+__global__ void __launch_bounds__(1024) moe_chunk_scan_kernel(int n_chunks, int n_experts, int* __restrict__ chunk_counts, int* __restrict__ counts,
+                                                             int* __restrict__ offsets, int* __restrict__ active, int* __restrict__ n_active) {
+    __shared__ int wave_total[16], wave_active[16];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int e = tid;
+    int c = 0;
+    if (e < n_experts)
+        for (int b = 0; b < n_chunks; ++b) c += chunk_counts[(size_t)b * n_experts + e];
+    int incl = c, incl_active = c > 0;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(incl, d, 64), oa = __shfl_up(incl_active, d, 64);
+        if (lane >= d) {
+            incl += o;
+            incl_active += oa;
+        }
+    }
+    if (lane == 63) {
+        wave_total[wave] = incl;
+        wave_active[wave] = incl_active;
+    }
+    __syncthreads();
+    int before = incl - c, active_before = incl_active - (c > 0);
+    for (int w = 0; w < wave; ++w) {
+        before += wave_total[w];
+        active_before += wave_active[w];
+    }
+    if (e >= n_experts) return;
+    counts[e] = c;
+    offsets[e] = before;
+    if (c > 0) active[active_before] = e;
+    if (e == n_experts - 1) {
+        offsets[n_experts] = before + c;
+        n_active[0] = active_before + (c > 0);
+    }
+    // the chunks' first places within the expert's run, in chunk order
+    int at = before;
+    for (int b = 0; b < n_chunks; ++b) {
+        const int n = chunk_counts[(size_t)b * n_experts + e];
+        chunk_counts[(size_t)b * n_experts + e] = at;
+        at += n;
+    }
+}
+
+__global__ void __launch_bounds__(1024) moe_chunk_place_kernel(const int* __restrict__ ids, int n_pairs, int n_experts,
+                                                              const int* __restrict__ chunk_first, int* __restrict__ list) {
+    __shared__ __attribute__((aligned(16))) int pair_expert[1024];
+    const int tid = threadIdx.x, p = blockIdx.x * 1024 + tid;
+    int e = p < n_pairs ? ids[p] : -1;
+    if (e >= n_experts) e = -1;
+    pair_expert[tid] = e;
+    __syncthreads();
+    if (e < 0) return;
+    int rank = 0;
+    const int whole = tid & ~3;
+    for (int q = 0; q < whole; q += 4) {
+        const int4 v = *reinterpret_cast<const int4*>(&pair_expert[q]);
+        rank += (v.x == e) + (v.y == e) + (v.z == e) + (v.w == e);
+    }
+    for (int q = whole; q < tid; ++q) rank += pair_expert[q] == e;
+    list[chunk_first[(size_t)blockIdx.x * n_experts + e] + rank] = p;
+}
+
 // counts [X], offsets [X+1], list [n_pairs], active [X], n_active [1]
+// scratch (optional): [ceil(n_pairs / 1024) * n_experts] ints for steps of many pairs
 extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* counts, int* offsets, int* list, int* active, int* n_active,
-                              hipStream_t stream) {
+                              int* scratch, hipStream_t stream) {
     if (n_pairs <= 0 || n_experts <= 0) return 0;
     if (n_pairs <= ALIGN_SMALL_PAIRS && n_experts <= 1024) {
         hipLaunchKernelGGL(moe_align_small_kernel, dim3(1), dim3(1024), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
+        return LLMX_CHECK_LAUNCH();
+    }
+    if (scratch && n_experts <= 1024) {
+        const int n_chunks = (n_pairs + 1023) / 1024;
+        hipLaunchKernelGGL(moe_chunk_count_kernel, dim3(n_chunks), dim3(1024), 0, stream, ids, n_pairs, n_experts, scratch);
+        hipLaunchKernelGGL(moe_chunk_scan_kernel, dim3(1), dim3(1024), 0, stream, n_chunks, n_experts, scratch, counts, offsets, active, n_active);
+        hipLaunchKernelGGL(moe_chunk_place_kernel, dim3(n_chunks), dim3(1024), 0, stream, ids, n_pairs, n_experts, scratch, list);
         return LLMX_CHECK_LAUNCH();
     }
     hipLaunchKernelGGL(moe_count_kernel, dim3(n_experts), dim3(256), 0, stream, ids, n_pairs, counts);

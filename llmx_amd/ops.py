@@ -61,7 +61,7 @@ def _declare(h) -> None:
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P],
-        "llmx_moe_align": [P, I, I, P, P, P, P, P, P],
+        "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
         "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
@@ -379,20 +379,32 @@ def route_topk(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor,
                                  rows, n_experts, k, score, 1 if normalize else 0, float(scale), _stream()), "route_topk")
 
 
+def moe_align_scratch(n_pairs: int, n_experts: int) -> int:
+    """Ints of scratch that moe_align wants for this many pairs (0: none)."""
+    return 0 if n_pairs <= 1024 or n_experts > 1024 else -(-n_pairs // 1024) * n_experts
+
+
 def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
-              active: torch.Tensor, n_active: torch.Tensor) -> None:
+              active: torch.Tensor, n_active: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> None:
     """Groups the pairs p = t*k + j by expert (stable): counts [X], offsets [X+1], pairs [T*k], and the experts that
-    have rows in increasing order: active [X] (first n_active[0] entries)."""
+    have rows in increasing order: active [X] (first n_active[0] entries).  `scratch`: moe_align_scratch(...) int32 for
+    steps of many pairs (made here when it is not given)."""
     n_pairs = ids.numel()
+    need = moe_align_scratch(n_pairs, n_experts)
+    if need and scratch is None:
+        scratch = torch.empty(need, dtype=torch.int32, device=ids.device)
+    if scratch is not None and scratch.numel() < need:
+        raise KernelError(f"moe_align: scratch of {scratch.numel()} ints, {need} needed")
     _check(lib().llmx_moe_align(_dev(ids, "ids", torch.int32), n_pairs, n_experts, _dev(counts, "counts", torch.int32, (n_experts,)),
                                 _dev(offsets, "offsets", torch.int32, (n_experts + 1,)), _dev(pairs, "pairs", torch.int32, (n_pairs,)),
                                 _dev(active, "active", torch.int32, (n_experts,)), _dev(n_active, "n_active", torch.int32, (1,)),
-                                _stream()), "moe_align")
+                                _dev(scratch if need else None, "scratch", torch.int32), _stream()), "moe_align")
 
 
 def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
                      normalize: bool, scale: float, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
-                     active: torch.Tensor, n_active: torch.Tensor, parts: Optional[torch.Tensor] = None) -> None:
+                     active: torch.Tensor, n_active: torch.Tensor, parts: Optional[torch.Tensor] = None,
+                     scratch: Optional[torch.Tensor] = None) -> None:
     """route_topk followed by moe_align; a step of at most 16 rows (sigmoid scores, at most 256 experts and 64 picks) does
     both in one launch, with the same bits."""
     rows, n_experts = z.shape
@@ -406,7 +418,7 @@ def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.T
             _dev(n_active, "n_active", torch.int32, (1,)), _stream()), "route_topk_align")
         return
     route_topk(z, bias, ids, weights, k, score, normalize, scale, parts)
-    moe_align(ids, n_experts, counts, offsets, pairs, active, n_active)
+    moe_align(ids, n_experts, counts, offsets, pairs, active, n_active, scratch)
 
 
 def moe_combine(x: torch.Tensor, y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, accumulate: bool = True) -> None:

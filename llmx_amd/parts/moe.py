@@ -90,8 +90,10 @@ class RoutedExperts(FeedForward):
         pairs = step.buf("experts.pairs", (T * k,), torch.int32)
         active = step.buf("experts.active", (X,), torch.int32)
         n_active = step.buf("experts.n_active", (1,), torch.int32)
+        need = ops.moe_align_scratch(T * k, X)
+        scratch = step.buf("experts.align_scratch", (need,), torch.int32) if need else None
         ops.route_topk_align(z, self.bias, ids, weights, k, self.score, self.normalize, self.scale, counts, offsets, pairs, active, n_active,
-                             parts=parts)
+                             parts=parts, scratch=scratch)
         step.observe("routing", logits=z, ids=ids, weights=weights)
         act = step.buf("experts.act", (T * k, self.intermediate), step.act_dtype)
         ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T)

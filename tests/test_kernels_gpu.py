@@ -182,7 +182,7 @@ def routed_setup(T, X, k, seed):
 
 
 @pytest.mark.parametrize("T,X,k,E,F", [(1, 8, 2, 64, 32), (5, 16, 4, 96, 48), (17, 24, 3, 72, 40), (40, 256, 8, 256, 128), (150, 6, 2, 64, 32),
-                                       (700, 5, 2, 136, 72)])
+                                       (700, 5, 2, 136, 72), (2100, 300, 3, 64, 32)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_routed_products(T, X, k, E, F, dtype):
     """moe_align, the two grouped products and the combine against a loop over pairs; experts without rows included."""
