@@ -6,7 +6,8 @@ A step is one decode step of the whole batch: B requests, each at a context that
 step, one new token each, logits -> greedy token on the device -> ids read back (the reference's batched `tg`,
 /root/reference/src/cli/main.cpp:1246-1254, reads each pass's results before the next).  Prints one JSON line:
 `value` = decoded tokens a second at the default batch; `points` = the same at batch 1 and 64; `prefill` = one
-2,048-token prompt from an empty cache; `roofline` = bytes the decode step has to read / its time against HBM's 8 TB/s.
+2,048-token prompt from an empty cache; `roofline` = bytes the decode step has to read / its time against HBM's 8 TB/s;
+`calibration` = what a device copy, a read-only pass and a square bf16 library product reach on this card.
 Token ids are a fixed LCG sequence; weights are N(0, 0.02) generated on the device.
 """
 
@@ -37,6 +38,8 @@ def parse():
     ap.add_argument("--context", type=int, default=0, help="tokens each sequence holds at the last timed step (0: the configuration's)")
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-calibration", action="store_true", help="skip the copy, read and library-product rates of the card")
+    ap.add_argument("--logits-to-host", action="store_true", help="also measure the default batch with every step's logits copied to the host")
     ap.add_argument("--only-prefill", action="store_true", help="for profiling: measure the prefill alone and print its record")
     ap.add_argument("--context-fill", choices=["synthetic", "prefill"], default="synthetic",
                     help="how the context before the timed steps gets into the cache: random keys and values written "
@@ -104,7 +107,35 @@ class DistinctExperts:
             self.counts.append(int(torch.unique(tensors["ids"]).numel()))
 
 
-def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch):
+def calibrate(torch, device):
+    """What this card gives a plain program: a device-to-device copy (bytes read plus written), a read-only pass
+    (a sum over 4 GiB) and a square bf16 library product, beside the published 8 TB/s and 2.5 PFLOP/s."""
+    def best(fn, reps=5):
+        fn()
+        torch.cuda.synchronize()
+        t = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            t.append(time.perf_counter() - t0)
+        return min(t)
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.float32, device=device).normal_()
+    dst = torch.empty_like(src)
+    copy_gbs = 2 * 4 * n / best(lambda: dst.copy_(src)) / 1e9
+    read_gbs = 4 * n / best(lambda: src.sum()) / 1e9
+    del dst, src
+    m = 8192
+    a = torch.empty(m, m, dtype=torch.bfloat16, device=device).normal_()
+    b = torch.empty(m, m, dtype=torch.bfloat16, device=device).normal_()
+    tflops = 2 * m ** 3 / best(lambda: torch.matmul(a, b)) / 1e12
+    del a, b
+    torch.cuda.empty_cache()
+    return {"copy_gbs": round(copy_gbs, 1), "read_gbs": round(read_gbs, 1), "bf16_gemm_tflops": round(tflops, 1)}
+
+
+def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch, read_logits=False):
     from llmx_amd import ops
     from llmx_amd.engine import StepEntry
     c = engine.config
@@ -126,11 +157,14 @@ def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch):
     run_decode.fill_s = time.perf_counter() - t_fill
     last = [lcg_ids(1, c.vocab_size, 7 + i)[0] for i in range(batch)]
     out = sampler_out[:batch]
+    host_logits = torch.empty(batch, c.vocab_size, dtype=torch.float32, pin_memory=True) if read_logits else None
 
     def one():
         nonlocal last
         logits = engine.step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, last)])
         ops.argmax_rows(logits, out)
+        if read_logits:
+            host_logits.copy_(logits)     # the reference's bench reads every step's logits on the host
         last = out.tolist()   # the ids come back to the host, as a serving loop reads them
 
     # the first warm-up step also counts the experts the batch touches per layer
@@ -237,6 +271,9 @@ def main():
     }
 
     pts = {}
+    if a.logits_to_host:
+        dtb, _ = run_decode(engine, sampler_out, a.batch, context, a.steps, a.warmup, a.context_fill, torch, read_logits=True)
+        pts[f"decode_b{a.batch}_logits_to_host"] = round(a.batch * a.steps / dtb, 2)
     for b in points:
         steps = a.steps
         dtb, _ = run_decode(engine, sampler_out, b, context, steps, a.warmup, a.context_fill, torch)
@@ -246,6 +283,8 @@ def main():
 
     if not a.no_prefill:
         result["prefill"] = run_prefill(engine, cfg, sampler_out, torch)
+    if not a.no_calibration:
+        result["calibration"] = calibrate(torch, sampler_out.device)
     print(json.dumps(result))
 
 

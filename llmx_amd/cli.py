@@ -2,8 +2,10 @@
 
 Flags keep the reference's names and meanings where it has them (main.cpp:2018-2038 sampling, :541-574 execution):
 --max-tokens/-n, --temp, --topk, --topp, --min-p, --penalty, --presence-penalty, --frequency-penalty, --seed,
---ignore-eos, --dtype, --ubatch, --kv-tokens, --verbose.  There is no tokenizer here: a prompt is a list of token ids
-(comma or space separated), given on the line, with --file, or made up with --prompt-len.  A usage error exits with
+--ignore-eos, --stop, --dtype, --ubatch, --kv-tokens, --verbose; logits: --then-ids, --last, --per-token, --top;
+perplexity: --ctx-size/-c, --chunks, --per-token.  There is no tokenizer here: a prompt is a list of token ids
+(comma or space separated), given on the line, with --file, or made up with --prompt-len; a stop text is a sequence
+of token ids.  A usage error exits with
 status 2 (main.cpp:100-103); a flag given twice is refused (:129-159).
 """
 
@@ -42,6 +44,7 @@ def _add_sampling(p):
     p.add_argument("--frequency-penalty", type=float, default=d.frequency_penalty, action=_Once)
     p.add_argument("--seed", type=int, default=d.seed, action=_Once, help="0 keeps the fixed default generator state")
     p.add_argument("--ignore-eos", nargs=0, default=False, action=_Once, help="the end token is never drawn")
+    p.add_argument("--stop", default="", action=_Once, help="token ids; generation ends when the generated ids end with them")
 
 
 def _add_exec(p):
@@ -70,7 +73,7 @@ def _params(a):
     from .sampling.params import SamplingParams
     return SamplingParams(max_tokens=a.max_tokens, temp=a.temp, top_k=a.topk, top_p=a.topp, min_p=a.min_p, penalty=a.penalty,
                           presence_penalty=a.presence_penalty, frequency_penalty=a.frequency_penalty, seed=a.seed,
-                          ignore_eos=bool(a.ignore_eos)).validate()
+                          ignore_eos=bool(a.ignore_eos), stop=tuple(_ids(a.stop)) if a.stop else ()).validate()
 
 
 def _lcg_ids(n: int, vocab: int, seed: int = 1):
@@ -127,7 +130,11 @@ def cmd_generate(a) -> int:
 def cmd_logits(a) -> int:
     """Top-N logits of the last positions, whole or token by token (the reference's `llmx logits`, main.cpp:934-980)."""
     from .engine import Engine, StepEntry
-    ids = _ids(a.prompt) if a.prompt is not None else _ids(Path(a.file).read_text())
+    ids = _prompt_ids(a, "logits")
+    if a.then_ids:
+        ids = ids + _ids(Path(a.then_ids).read_text())
+    if not ids:
+        raise SystemExit2("logits: empty prompt")
     engine = Engine.load(a.model, dtype=a.dtype, kv_tokens=a.kv_tokens or len(ids) + a.page_tokens, page_tokens=a.page_tokens, max_requests=1)
     engine.add_request(0)
     last = min(a.last or 1, len(ids))
@@ -146,8 +153,53 @@ def cmd_logits(a) -> int:
     print(f"tokens: {len(ids)}")
     for off, row in enumerate(rows):
         vals, idx = row.topk(min(a.top, row.numel()))
-        print(f"{len(ids) - len(rows) + off} " + " ".join(f"{int(i)} {float(v):.6f}" for v, i in zip(vals, idx)))
+        if a.last:          # one line a position: the position, then id and logit of each of the top
+            print(f"{len(ids) - len(rows) + off} " + " ".join(f"{int(i)} {float(v):.6f}" for v, i in zip(vals, idx)))
+        else:               # the last position alone: one line for each of the top
+            for v, i in zip(vals, idx):
+                print(f"{int(i)} {float(v):.6f}")
     return 0
+
+
+def _prompt_ids(a, command: str):
+    if a.prompt is not None and a.file:
+        raise SystemExit2(f"{command}: token ids on the line or --file, not both")
+    if a.prompt is not None:
+        return _ids(a.prompt)
+    if a.file:
+        return _ids(Path(a.file).read_text())
+    if getattr(a, "then_ids", None):
+        return []
+    raise SystemExit2(f"{command} needs token ids: on the line or with --file")
+
+
+def cmd_perplexity(a) -> int:
+    """Mean negative log-likelihood over windows of token ids (the reference's `llmx perplexity`, main.cpp:982-1008)."""
+    from .engine import Engine
+    from .engine.perplexity import MIN_WINDOW, perplexity
+    ids = _prompt_ids(a, "perplexity")
+    if len(ids) < MIN_WINDOW:
+        raise SystemExit2(f"perplexity: need at least {MIN_WINDOW} tokens")
+    window = min(a.ctx_size or len(ids), len(ids))
+    engine = Engine.load(a.model, dtype=a.dtype, kv_tokens=a.kv_tokens or window + a.page_tokens, page_tokens=a.page_tokens, max_requests=1)
+    window = min(window, engine.max_positions)
+    r = perplexity(engine, ids, window, a.chunks, a.per_token, a.ubatch)
+    if a.verbose:
+        for w, (scored, nll) in enumerate(r.windows):
+            print(f"chunk {w + 1}: scored {scored}, mean NLL {nll / scored:.9f}")
+    print(f"tokens: {len(ids)}")
+    print(f"used tokens: {r.used_tokens}")
+    print(f"scored tokens: {r.scored_tokens}")
+    print(f"chunks: {len(r.windows)}")
+    print(f"context size: {r.context}")
+    print(f"mean NLL: {r.mean_nll:.9f}")
+    print(f"perplexity: {r.perplexity:.6g}")
+    return 0
+
+
+def cmd_replay(a) -> int:
+    from .tools.trace_run import main as replay
+    return replay(a.rest)
 
 
 def cmd_random(a) -> int:
@@ -162,7 +214,7 @@ def cmd_random(a) -> int:
 
 
 def build_parser():
-    ap = argparse.ArgumentParser(prog="llmx", description="MiniMax-M3 on one MI355X: generate, logits, random, bench")
+    ap = argparse.ArgumentParser(prog="llmx", description="MiniMax-M3 on one MI355X: generate, logits, perplexity, replay, random, bench")
     sub = ap.add_subparsers(dest="command", required=True)
     g = sub.add_parser("generate", help="generate tokens after a prompt of token ids")
     g.add_argument("model", help="model folder (config.json + model.safetensors)")
@@ -176,11 +228,24 @@ def build_parser():
     l.add_argument("model")
     l.add_argument("prompt", nargs="?", default=None)
     l.add_argument("--file", "-f", default=None)
+    l.add_argument("--then-ids", default=None, help="a file of token ids appended to the prompt")
     l.add_argument("--last", type=int, default=0, help="report this many final positions")
     l.add_argument("--per-token", action="store_true", help="feed the tokens one step each")
     l.add_argument("--top", type=int, default=10)
     _add_exec(l)
     l.set_defaults(run=cmd_logits)
+    x = sub.add_parser("perplexity", help="mean negative log-likelihood of token ids, in windows from an empty history")
+    x.add_argument("model")
+    x.add_argument("prompt", nargs="?", default=None)
+    x.add_argument("--file", "-f", default=None, help="a file of token ids")
+    x.add_argument("--ctx-size", "-c", type=int, default=0, action=_Once, help="window tokens (default: all the ids, at most the model's context)")
+    x.add_argument("--chunks", type=int, default=0, action=_Once, help="windows at most (default: all)")
+    x.add_argument("--per-token", action="store_true", help="one token a step: the decode path")
+    _add_exec(x)
+    x.set_defaults(run=cmd_perplexity)
+    t = sub.add_parser("replay", help="feed a trace of steps through the model and write logits (bin/trace_run)", add_help=False)
+    t.add_argument("rest", nargs=argparse.REMAINDER)
+    t.set_defaults(run=cmd_replay)
     r = sub.add_parser("random", help="write a model folder with seeded random weights")
     r.add_argument("--config", required=True, help="a config.json")
     r.add_argument("--out", required=True)
@@ -198,7 +263,10 @@ def build_parser():
 
 def main(argv=None) -> int:
     ap = build_parser()
+    argv = sys.argv[1:] if argv is None else list(argv)
     try:
+        if argv and argv[0] == "replay":      # its own parser reads every flag, --help included
+            return cmd_replay(argparse.Namespace(rest=argv[1:]))
         a = ap.parse_args(argv)
         return a.run(a)
     except SystemExit2 as e:

@@ -248,6 +248,48 @@ class Engine:
             self.cache.commit(r)
         return logits
 
+    # -- wrappers over step, for one request (the reference's Model::prefill / step / score, runtime.hpp:1278-1385) --
+    def prefill(self, request: Hashable, tokens: Sequence[int], portion: int = 512) -> torch.Tensor:
+        """Feeds `tokens` in portions of at most `portion`; returns the float32 logits [vocab] after the last token."""
+        tokens = list(tokens)
+        if not tokens:
+            raise StepError("prefill: no tokens")
+        if portion < 1:
+            raise StepError("prefill: a portion holds at least one token")
+        row = None
+        for s in range(0, len(tokens), portion):
+            part = tokens[s:s + portion]
+            last = s + len(part) == len(tokens)
+            out = self.step([StepEntry(request, part, [len(part) - 1] if last else [])])
+            if last:
+                row = out[0]
+        return row
+
+    def decode_one(self, request: Hashable, token: int) -> torch.Tensor:
+        """Feeds one token; returns the float32 logits [vocab] after it."""
+        return self.step([StepEntry(request, [int(token)], [0])])[0]
+
+    def score(self, request: Hashable, tokens: Sequence[int], portion: int = 512, each=None) -> Optional[torch.Tensor]:
+        """The logits at every position of `tokens`, fed in portions.
+
+        With `each`, it is called as each(first_position, logits [n, vocab]) per portion (the storage is reused by
+        the next one) and nothing is returned; without, the rows come back as one float32 tensor [len(tokens), vocab].
+        """
+        tokens = list(tokens)
+        if not tokens:
+            raise StepError("score: no tokens")
+        if portion < 1:
+            raise StepError("score: a portion holds at least one token")
+        rows = None if each else torch.empty(len(tokens), self.spec.vocab_size, dtype=torch.float32, device=self.device)
+        for s in range(0, len(tokens), portion):
+            part = tokens[s:s + portion]
+            out = self.step([StepEntry(request, part, list(range(len(part))))])
+            if each:
+                each(s, out)
+            else:
+                rows[s:s + len(part)] = out
+        return rows
+
     def _run(self, entries: List[StepEntry], views: List[EntryView], T: int) -> torch.Tensor:
         n_e = len(entries)
         token_ids = np.empty(T, dtype=np.int32)

@@ -7,7 +7,8 @@ Policy (decisions only; it owns no model and is tested with a simulated executor
     head of the queue does not fit, admission stops (no overtaking) until running requests finish and free pages.
   * A step takes the decoding requests first, one token each, in order of admission, then portions of prompts in order
     of admission while the step's token budget lasts; a portion wants logits only when it reaches the prompt's end.
-  * A request finishes on its end token (not kept, unless ignore_eos) or at max_tokens; its pages and slot go back at once.
+  * A request finishes on its end token (not kept, unless ignore_eos), when its generated ids end with one of its
+    stop sequences, or at max_tokens; its pages and slot go back at once.
 The shape follows the reference's scheduler (/root/reference/src/server/scheduler.hpp:1187-1376 form, :752-766 admission,
 :2514-2571 retire; reservation: /root/reference/src/server/policy.hpp:153-158).
 """
@@ -36,7 +37,7 @@ class Request:
     generated: List[int] = field(default_factory=list)
     fed: int = 0                       # tokens of prompt + generated already in the cache
     state: str = "waiting"             # waiting | running | finished
-    finish_reason: Optional[str] = None  # "eos" | "length"
+    finish_reason: Optional[str] = None  # "eos" | "stop" | "length"
     reserved: List[int] = field(default_factory=list)
     rng: XorShift64 = None
     order: int = -1                    # order of admission
@@ -151,7 +152,9 @@ class Scheduler:
                 r.finish_reason = "eos"
             else:
                 r.generated.append(tok)
-                if len(r.generated) >= r.params.max_tokens:
+                if any(len(r.generated) >= len(s) and tuple(r.generated[-len(s):]) == s for s in r.params.stop):
+                    r.finish_reason = "stop"       # the token that completes a stop sequence is kept and not fed
+                elif len(r.generated) >= r.params.max_tokens:
                     r.finish_reason = "length"
             if r.finish_reason:
                 done.append(r)

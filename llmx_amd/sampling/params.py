@@ -24,6 +24,7 @@ class SamplingParams:
     frequency_penalty: float = 0.0
     seed: int = 0                    # 0 keeps the generator's fixed default state
     ignore_eos: bool = False         # the end token is never drawn
+    stop: tuple = ()                 # sequences of token ids; generation ends when the generated ids end with one
 
     def validate(self) -> "SamplingParams":
         def bad(name, why):
@@ -46,6 +47,7 @@ class SamplingParams:
             raise bad("frequency_penalty", "must lie in [-2, 2]")
         if self.seed < 0 or self.seed > _M64:
             raise bad("seed", "must fit 64 unsigned bits")
+        self.stop = normalize_stop(self.stop)
         if self.temp > 0.0 and self.top_p < 1.0 and not 0 < self.top_k <= MAX_DEVICE_TOP_K:
             raise bad("top_p", f"below 1 needs a top_k between 1 and {MAX_DEVICE_TOP_K} on this engine")
         if self.temp > 0.0 and self.top_k > MAX_DEVICE_TOP_K:
@@ -59,6 +61,29 @@ class SamplingParams:
     @property
     def penalized(self) -> bool:
         return (self.penalty > 0.0 and self.penalty != 1.0) or self.presence_penalty != 0.0 or self.frequency_penalty != 0.0
+
+
+MAX_STOPS, MAX_STOP_TOKENS = 16, 256
+
+
+def normalize_stop(stop) -> tuple:
+    """A tuple of tuples of token ids from one sequence of ids or several.
+
+    The reference stops on a text (/root/reference/src/inference/generate.hpp:33, at most 16 of 256 bytes each on its
+    server); without a tokenizer a sequence of token ids stands for the text.
+    """
+    if not stop:
+        return ()
+    seqs = [stop] if all(isinstance(t, int) for t in stop) else list(stop)
+    out = []
+    for s in seqs:
+        s = tuple(int(t) for t in s)
+        if not s or len(s) > MAX_STOP_TOKENS or any(t < 0 for t in s):
+            raise ValueError(f"sampling: a stop sequence holds 1 to {MAX_STOP_TOKENS} token ids")
+        out.append(s)
+    if len(out) > MAX_STOPS:
+        raise ValueError(f"sampling: stop holds at most {MAX_STOPS} sequences")
+    return tuple(out)
 
 
 class XorShift64:

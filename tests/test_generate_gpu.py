@@ -77,6 +77,61 @@ def test_eos_ends_a_request():
     assert len(ignoring) == 6 and ignoring[:3] == free[:3] and free[3] not in ignoring[3:4]
 
 
+def test_a_stop_sequence_ends_a_request():
+    from llmx_amd import Engine, SamplingParams, generate
+    name = "B"
+    cfg, w = plain(name)
+    prompt = tokens_for(name, 9, 31)
+    free = plain_model.greedy(cfg, w, prompt, 8)
+    engine = engine_for(name)
+    got = generate(engine, [prompt, prompt], [SamplingParams(max_tokens=8, temp=0.0, stop=tuple(free[3:5])),
+                                              SamplingParams(max_tokens=8, temp=0.0, stop=((free[1], free[0]),))])
+    at = next(i for i in range(1, 8) if free[i - 1:i + 1] == free[3:5])      # the pair's first appearance
+    assert got[0] == free[:at + 1]                                            # the completing token is kept
+    pairs = [free[i - 1:i + 1] for i in range(1, 8)]
+    if [free[1], free[0]] not in pairs:
+        assert got[1] == free                                                 # a sequence that never appears stops nothing
+
+
+def test_wrappers_over_step_and_perplexity():
+    """prefill, decode_one and score are the step function for one request; perplexity in windows, through the prompt
+    path and token by token, equals the plain implementation's log-softmax in double."""
+    from llmx_amd.engine.perplexity import perplexity
+    name = "A"
+    cfg, w = plain(name)
+    ids = tokens_for(name, 45, 13)
+    logits = plain_model.forward(cfg, w, ids).double()
+    engine = engine_for(name)
+    engine.add_request("r")
+    row = engine.prefill("r", ids[:30], portion=7)
+    assert (row.cpu() - logits[29].float()).abs().max() < 2e-5
+    row = engine.decode_one("r", ids[30])
+    assert (row.cpu() - logits[30].float()).abs().max() < 2e-5 and engine.length("r") == 31
+    engine.end_request("r")
+    engine.add_request("s")
+    rows = engine.score("s", ids, portion=11)
+    engine.end_request("s")
+    assert rows.shape == (45, cfg["vocab_size"]) and (rows.cpu() - logits.float()).abs().max() < 2e-5
+
+    def plain_nll(window):
+        z = plain_model.forward(cfg, w, window).double()
+        lp = torch.log_softmax(z, dim=1)
+        return -sum(float(lp[i, window[i + 1]]) for i in range(len(window) - 1))
+    want = [plain_nll(ids[0:20]), plain_nll(ids[20:40]), plain_nll(ids[40:45])]
+    for per_token in (False, True):
+        r = perplexity(engine, ids, context=20, per_token=per_token, portion=6)
+        assert [s for s, _ in r.windows] == [19, 19, 4] and r.used_tokens == 45 and r.scored_tokens == 42
+        for (scored, got), w_ in zip(r.windows, want):
+            assert abs(got - w_) < 4e-5 * scored          # a logit and the log of the sum within 2e-5 each
+        assert abs(r.mean_nll - sum(want) / 42) < 2e-5
+    two = perplexity(engine, ids, context=20, max_chunks=2)
+    assert len(two.windows) == 2 and two.scored_tokens == 38
+    assert perplexity(engine, ids[:41], context=20).used_tokens == 40       # a rest of one token scores nothing
+    with pytest.raises(ValueError, match="at least 2"):
+        perplexity(engine, ids[:1])
+    assert all(engine.cache.pages_in_use(g) == 0 for g in range(len(engine.cache.groups)))
+
+
 def test_command_line(tmp_path):
     name = "A"
     cfg, w = plain(name)
@@ -100,3 +155,23 @@ def test_command_line(tmp_path):
     logits = plain_model.forward(cfg, w, prompt)
     last = lines[-1].split()
     assert int(last[0]) == 10 and int(last[1]) == int(logits[-1].argmax()) and abs(float(last[2]) - float(logits[-1].max())) < 1e-4
+    # --then-ids appends ids from a file; without --last the top list of the last position comes one id a line
+    more = tmp_path / "more.txt"
+    more.write_text(" ".join(map(str, prompt[6:])))
+    lg = subprocess.run([os.path.join(ROOT, "bin", "llmx"), "logits", model_folder(name), ",".join(map(str, prompt[:6])), "--then-ids", str(more),
+                         "--top", "3", "--dtype", "f32", "--page-tokens", "4", "--per-token"], capture_output=True, text=True, timeout=300)
+    assert lg.returncode == 0, lg.stderr[-2000:]
+    lines = lg.stdout.strip().split("\n")
+    assert lines[0] == "tokens: 11" and len(lines) == 4 and int(lines[1].split()[0]) == int(logits[-1].argmax())
+    ids_file = tmp_path / "ids.txt"
+    ids_file.write_text(",".join(map(str, prompt * 3)))
+    pp = subprocess.run([os.path.join(ROOT, "bin", "llmx"), "perplexity", model_folder(name), "--file", str(ids_file), "-c", "16", "--chunks", "2",
+                         "--dtype", "f32", "--page-tokens", "4", "--verbose"], capture_output=True, text=True, timeout=300)
+    assert pp.returncode == 0, pp.stderr[-2000:]
+    out = dict(line.split(": ", 1) for line in pp.stdout.strip().split("\n") if not line.startswith("chunk "))
+    assert out["tokens"] == "33" and out["used tokens"] == "32" and out["scored tokens"] == "30" and out["chunks"] == "2" and out["context size"] == "16"
+    z = [torch.log_softmax(plain_model.forward(cfg, w, (prompt * 3)[s:s + 16]).double(), dim=1) for s in (0, 16)]
+    nll = -sum(float(z[k][i, (prompt * 3)[16 * k + i + 1]]) for k in range(2) for i in range(15)) / 30
+    assert abs(float(out["mean NLL"]) - nll) < 2e-5
+    bad = subprocess.run([os.path.join(ROOT, "bin", "llmx"), "perplexity", model_folder(name), "7"], capture_output=True, text=True, timeout=120)
+    assert bad.returncode == 2 and "at least 2" in bad.stderr

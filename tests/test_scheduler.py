@@ -74,6 +74,27 @@ def test_eos_and_ignore_eos():
     assert s.finished["b"].generated == [5, 5, EOS, 5] and s.finished["b"].finish_reason == "length"
 
 
+def test_stop_sequences():
+    """Generation ends when the generated ids end with a stop sequence; the completing token is kept (the reference
+    keeps the token that completes its stop text and does not feed it: /root/reference/src/inference/generate.hpp:29-36)."""
+    s = Scheduler([GroupSpec("kv", 4, 100)], 3, 16, eos_token_id=EOS)
+    seq = [5, 6, 7, 6, 7, 8, 9]
+    s.submit(Request("one", [1, 2], SamplingParams(max_tokens=7, temp=0.0, stop=(7, 8))))
+    s.submit(Request("two", [1, 2], SamplingParams(max_tokens=7, temp=0.0, stop=((9, 9), (6, 7, 6)))))
+    s.submit(Request("none", [1, 2], SamplingParams(max_tokens=7, temp=0.0, stop=((8, 7),))))
+    plans = run(s, token_for=lambda r, i: seq[i])
+    assert s.finished["one"].generated == [5, 6, 7, 6, 7, 8] and s.finished["one"].finish_reason == "stop"
+    assert s.finished["two"].generated == [5, 6, 7, 6] and s.finished["two"].finish_reason == "stop"
+    assert s.finished["none"].generated == seq and s.finished["none"].finish_reason == "length"
+    # the completing token is never fed: after the step that drew it the request is gone
+    assert all(e.request != "two" for p in plans[4:] for e in p)
+    assert s.reserved == [0]
+    assert SamplingParams(stop=()).validate().stop == ()
+    for bad in (((),), tuple(range(300)), ((1,),) * 17, (-1,)):
+        with pytest.raises(ValueError, match="stop"):
+            SamplingParams(stop=bad).validate()
+
+
 def test_fifo_admission_and_reservation():
     """Pages run out: a request waits in the queue until running ones finish; nobody overtakes the head of the queue;
     a running request never fails to get a page (the cache manager is driven alongside and never raises)."""
