@@ -109,7 +109,7 @@ class DistinctExperts:
 
 def calibrate(torch, device):
     """What this card gives a plain program: a device-to-device copy (bytes read plus written), a read-only pass
-    (a sum over 4 GiB) and a square bf16 library product, beside the published 8 TB/s and 2.5 PFLOP/s."""
+    (a kernel that streams 4 GiB and keeps nothing) and a square bf16 library product, beside the published 8 TB/s and 2.5 PFLOP/s."""
     def best(fn, reps=5):
         fn()
         torch.cuda.synchronize()
@@ -124,7 +124,9 @@ def calibrate(torch, device):
     src = torch.empty(n, dtype=torch.float32, device=device).normal_()
     dst = torch.empty_like(src)
     copy_gbs = 2 * 4 * n / best(lambda: dst.copy_(src)) / 1e9
-    read_gbs = 4 * n / best(lambda: src.sum()) / 1e9
+    from llmx_amd import ops
+    flag = torch.zeros(1, dtype=torch.int32, device=device)
+    read_gbs = 4 * n / best(lambda: ops.read_probe(src, flag)) / 1e9
     del dst, src
     m = 8192
     a = torch.empty(m, m, dtype=torch.bfloat16, device=device).normal_()

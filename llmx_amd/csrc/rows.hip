@@ -158,3 +158,29 @@ extern "C" int llmx_fill_random(void* out, int dtype, long n, unsigned long long
         hipLaunchKernelGGL(fill_random_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)out, (size_t)n, (uint64_t)key, kind, a, b);
     return LLMX_CHECK_LAUNCH();
 }
+
+// Reads `bytes` (a multiple of 16) once and keeps nothing: what the card gives a kernel that only streams from memory.
+// Each workgroup takes a contiguous share, each thread holds 8 loads of 16 bytes in flight; the fold of the values is
+// stored only if it hits one fixed value, so the loads cannot be dropped.
+__global__ void __launch_bounds__(256) read_probe_kernel(const uint4* __restrict__ p, size_t n_vec, size_t share, unsigned* __restrict__ out) {
+    const size_t base = (size_t)blockIdx.x * share;
+    const size_t end = base + share < n_vec ? base + share : n_vec;
+    unsigned acc = 0;
+    for (size_t i = base + threadIdx.x; i < end; i += 256 * 8) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = i + 256 * u < end ? p[i + 256 * u] : uint4{0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (acc == 0x12345678u) out[0] = acc;
+}
+
+extern "C" int llmx_read_probe(const void* p, long bytes, int* out, hipStream_t stream) {
+    if (bytes <= 0 || bytes % 16 || ((uintptr_t)p & 15)) return -2;
+    const size_t n_vec = (size_t)bytes / 16;
+    const unsigned blocks = 4096;
+    const size_t share = (n_vec + blocks - 1) / blocks;
+    hipLaunchKernelGGL(read_probe_kernel, dim3(blocks), dim3(256), 0, stream, (const uint4*)p, n_vec, share, (unsigned*)out);
+    return LLMX_CHECK_LAUNCH();
+}

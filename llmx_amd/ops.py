@@ -56,6 +56,7 @@ def _declare(h) -> None:
         "llmx_moe_combine": [P, P, P, P, I, I, I, I, P],
         "llmx_fill_i32": [P, I, L, P],
         "llmx_fill_random": [P, I, L, ctypes.c_ulonglong, I, F, F, P],
+        "llmx_read_probe": [P, L, P, P],
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
@@ -437,6 +438,11 @@ def fill_random(t: torch.Tensor, key: int, kind: int, a: float, b: float) -> Non
     """Seeded fill: kind 0 = a + b * normal, kind 1 = uniform in [a, b); element i depends on (key, i) only."""
     _check(lib().llmx_fill_random(_dev(t, "t"), _code(t.dtype), t.numel(), key & ((1 << 64) - 1), int(kind), float(a), float(b),
                                   _stream()), "fill_random")
+
+
+def read_probe(t: torch.Tensor, out: torch.Tensor) -> None:
+    """Streams the tensor's bytes (a multiple of 16) through a kernel that keeps nothing: a measure of the card's read rate."""
+    _check(lib().llmx_read_probe(_dev(t, "t"), t.numel() * t.element_size(), _dev(out, "out", torch.int32), _stream()), "read_probe")
 
 
 _SCRATCH: dict = {}
