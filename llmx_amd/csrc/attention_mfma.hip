@@ -141,10 +141,11 @@ __device__ __forceinline__ void store_output(bf16_t* dst, int g, const f32x4_t (
     }
 }
 
-// item: {row0, n_rows, head0, n_heads, split, n_splits, slot, unused}
+// item: {row0, n_rows, head0, n_heads, split, n_splits, slot, slots}
 //   columns c = 0 .. n_rows*n_heads-1: row = row0 + c / n_heads, head = head0 + c % n_heads
 //   slot < 0: the item folds its segments itself and writes the final output; otherwise segment s of the row (counted
-//   from the row's first segment) goes to part_*[(slot + s) * 16 + c]
+//   from the row's first segment) goes to part_*[slot * 16 + c * slots + s], `slots` being the segments the row's
+//   group was given: a column's segments lie one after the other, so the merge streams them
 struct AttnMfmaArgs {
     const bf16_t* q;        // [T, n_heads, D]
     const bf16_t* k_cache;  // [pages, kv_heads, page_tokens, D]
@@ -154,7 +155,7 @@ struct AttnMfmaArgs {
     const int* tables;
     const int* items;
     bf16_t* out;            // [T, n_heads * D]
-    float* part_o;          // [slots * 16, D]
+    float* part_o;          // [slots * 16 + MERGE_PAD, D]
     float* part_ml;         // [slots * 16, 2]: segment max, segment sum
     float scale;
     int n_items, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window;
@@ -174,7 +175,7 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
     const int row0 = __builtin_amdgcn_readfirstlane(it[0]), n_rows = __builtin_amdgcn_readfirstlane(it[1]);
     const int head0 = __builtin_amdgcn_readfirstlane(it[2]), n_heads_item = __builtin_amdgcn_readfirstlane(it[3]);
     const int split = __builtin_amdgcn_readfirstlane(it[4]), n_splits = __builtin_amdgcn_readfirstlane(it[5]);
-    const int slot = __builtin_amdgcn_readfirstlane(it[6]);
+    const int slot = __builtin_amdgcn_readfirstlane(it[6]), slots = __builtin_amdgcn_readfirstlane(it[7]);
     const int D = 16 * DT, bt = a.page_tokens, Hkv = a.n_kv_heads;
     const int c = lane & 15, g = lane >> 4;
     const int n_cols = n_rows * n_heads_item;
@@ -304,7 +305,7 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
         chunk_values<DT>(vf_b, pf[3], o);
         if constexpr (PARTIAL) {
             if (col_ok) {
-                const size_t at = (size_t)(slot + seg0 / AM_SEG - seg_first) * 16 + c;
+                const size_t at = (size_t)slot * 16 + (size_t)c * slots + (seg0 / AM_SEG - seg_first);
                 float* dst = a.part_o + at * D;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(dst + 16 * dt + 4 * g) = o[dt];
@@ -686,43 +687,54 @@ __global__ void __launch_bounds__(512) paged_attention_tiles128_kernel(AttnMfmaA
     if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
 }
 
-// merge: one block per output (row, head).  merge item: {row, head, first_slot, column}.  The row's segments are folded
-// in key order with the formula the attention kernel uses for a tile's segments.  The fold's weights depend on the
-// segments' maxima only, so they are formed for 512 segments at a time by all threads (a prefix maximum, then
+// merge: one block per output (row, head).  merge item: {row, head, first_slot, column, slots}.  The row's segments are
+// folded in key order with the formula the attention kernel uses for a tile's segments.  The fold's weights depend on
+// the segments' maxima only, so they are formed for 512 segments at a time by all threads (a prefix maximum, then
 // fold_weights per segment); what is left of the chain is O = O * a + o * b per segment, with thread d owning dim d and
-// 32 segments' loads in flight.  Same operations on the same values as a sequential fold: the same bits.
+// 64 segments' loads in flight (two rounds of 32 whose registers are asked for again as soon as they are folded).  A
+// round in which every segment folds (none empty, none the first) runs the bare chain; the others choose per segment.
+// Same operations on the same values as a sequential fold: the same bits.  Loads run up to MERGE_PAD segments past a
+// row's last one and are never used: part_o has that many rows more than its slots.
 #define MERGE_CHUNK 512
 #define MERGE_DEPTH 32
+#define MERGE_RING 2
+#define MERGE_PAD (MERGE_DEPTH * MERGE_RING)
 template <bool WIDE>   // WIDE: head_dim above 128, two dims a thread
 __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restrict__ merges, const int* __restrict__ pos,
                                                             const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                             bf16_t* __restrict__ out, int n_heads, int D, int window) {
+    static_assert(MERGE_CHUNK % (MERGE_DEPTH * MERGE_RING) == 0, "a chunk is a whole number of turns of the ring");
     __shared__ __attribute__((aligned(16))) float seg_a[MERGE_CHUNK], seg_b[MERGE_CHUNK], seg_l[MERGE_CHUNK];
     __shared__ __attribute__((aligned(16))) int seg_code[MERGE_CHUNK];   // 0: empty segment, 1: the first one that is not (the state becomes it), 2: fold
+    // a round is plain when its first segment folds or is the row's first, every other one folds, and nothing but the
+    // row's end follows them: 1 (the first folds) or 2 (the first starts the state); 0 otherwise
+    __shared__ int round_plain[MERGE_CHUNK / MERGE_DEPTH];
     __shared__ float wave_top[2];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int* mi = merges + (size_t)blockIdx.x * AM_ITEM_INTS;
-    const int t = mi[0], h = mi[1], first = mi[2], c = mi[3];
+    const int t = mi[0], h = mi[1], first = mi[2], c = mi[3], slots = mi[4];
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int n_seg = p / AM_SEG - lo / AM_SEG + 1;
-    const float* base_o = part_o + ((size_t)first * 16 + c) * D;
-    const float* base_ml = part_ml + ((size_t)first * 16 + c) * 2;
-    const size_t stride_o = (size_t)16 * D, stride_ml = 32;
+    const float* base_o = part_o + ((size_t)first * 16 + (size_t)c * slots) * D;
+    const float* base_ml = part_ml + ((size_t)first * 16 + (size_t)c * slots) * 2;
     float M = -INFINITY, L = 0.0f;   // the same in every thread
     float O[WIDE ? 2 : 1] = {};       // dims tid and tid + 128
-    // a round's values: segments first .. first + MERGE_DEPTH - 1 (one past the end is read from the last and never used)
     const int d0 = tid < D ? tid : 0, d1 = tid + 128 < D ? tid + 128 : 0;
-    float ahead[WIDE ? 2 : 1][MERGE_DEPTH];
-    auto fetch = [&](int first_seg) {
+    float ring[MERGE_RING][WIDE ? 2 : 1][MERGE_DEPTH];
+    // a column's segments lie within a few hundred KB of its base: 32-bit byte offsets from it
+    const uint32_t seg_bytes = (uint32_t)D * 4u;
+    auto fetch = [&](float (&to)[WIDE ? 2 : 1][MERGE_DEPTH], int first_seg) {
+        const uint32_t at0 = (uint32_t)first_seg * seg_bytes + (uint32_t)d0 * 4u, at1 = (uint32_t)first_seg * seg_bytes + (uint32_t)d1 * 4u;
 #pragma unroll
         for (int u = 0; u < MERGE_DEPTH; ++u) {
-            const float* src = base_o + (size_t)min(first_seg + u, n_seg - 1) * stride_o;
-            ahead[0][u] = src[d0];
-            if constexpr (WIDE) ahead[1][u] = src[d1];
+            to[0][u] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(base_o) + (at0 + (uint32_t)u * seg_bytes));
+            if constexpr (WIDE) to[1][u] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(base_o) + (at1 + (uint32_t)u * seg_bytes));
         }
     };
-    fetch(0);
+#pragma unroll
+    for (int r = 0; r < MERGE_RING; ++r)
+        if (MERGE_DEPTH * r < n_seg) fetch(ring[r], MERGE_DEPTH * r);
     for (int c0 = 0; c0 < n_seg; c0 += MERGE_CHUNK) {
         // the thread's 4 segments of the chunk: maxima and sums
         float mv[4], lv[4], before[4];
@@ -730,8 +742,8 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
         for (int u = 0; u < 4; ++u) {
             const int sg = c0 + 4 * tid + u;
             const bool in = sg < n_seg;
-            mv[u] = in ? base_ml[(size_t)sg * stride_ml] : -INFINITY;
-            lv[u] = in ? base_ml[(size_t)sg * stride_ml + 1] : 0.0f;
+            mv[u] = in ? base_ml[(size_t)sg * 2] : -INFINITY;
+            lv[u] = in ? base_ml[(size_t)sg * 2 + 1] : 0.0f;
         }
         // the maximum of everything before each segment: earlier chunks, earlier threads, the thread's earlier segments
         float mine = fmaxf(fmaxf(mv[0], mv[1]), fmaxf(mv[2], mv[3]));
@@ -752,9 +764,11 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
             before[u] = run;
             run = fmaxf(run, mv[u]);
         }
+        bool folds = true;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int at = 4 * tid + u;
+            const bool round_first = (at % MERGE_DEPTH) == 0;
             int code = 0;
             float fa = 1.0f, fb = 0.0f;
             if (mv[u] != -INFINITY) {
@@ -764,42 +778,81 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
                     fold_weights(before[u], mv[u], fa, fb, mn);
                 }
             }
+            folds = folds && (code == 2 || (code == 1 && round_first) || c0 + at >= n_seg);
             seg_code[at] = code;
             seg_a[at] = fa;
             seg_b[at] = fb;
             seg_l[at] = lv[u];
         }
+        // 8 threads hold a round's 32 segments
+        const unsigned long long every = __ballot(folds);
+        if ((lane & 7) == 0) round_plain[tid >> 3] = ((every >> lane) & 0xffull) == 0xffull ? (mv[0] != -INFINITY && before[0] == -INFINITY ? 2 : 1) : 0;
         M = fmaxf(M, fmaxf(wave_top[0], wave_top[1]));
         __syncthreads();
         const int n = min(MERGE_CHUNK, n_seg - c0);
-        for (int s0 = 0; s0 < n; s0 += MERGE_DEPTH) {
-            // the next round's values are asked for before this round's are folded
-            float ov[WIDE ? 2 : 1][MERGE_DEPTH];
+        for (int s0 = 0; s0 < n; s0 += MERGE_DEPTH * MERGE_RING) {
 #pragma unroll
-            for (int u = 0; u < MERGE_DEPTH; ++u) {
-                ov[0][u] = ahead[0][u];
-                if constexpr (WIDE) ov[1][u] = ahead[1][u];
-            }
-            fetch(c0 + s0 + MERGE_DEPTH);
-            f32x4_t fa[MERGE_DEPTH / 4], fb[MERGE_DEPTH / 4], fl[MERGE_DEPTH / 4];
-            u32x4_t fc[MERGE_DEPTH / 4];
+            for (int r = 0; r < MERGE_RING; ++r) {
+                const int at = s0 + MERGE_DEPTH * r;      // the round's first segment within the chunk
+                if (at < n) {                             // the same for every thread
+                    f32x4_t fa[MERGE_DEPTH / 4], fb[MERGE_DEPTH / 4], fl[MERGE_DEPTH / 4];
 #pragma unroll
-            for (int u = 0; u < MERGE_DEPTH / 4; ++u) {
-                fa[u] = *reinterpret_cast<const f32x4_t*>(&seg_a[s0 + 4 * u]);
-                fb[u] = *reinterpret_cast<const f32x4_t*>(&seg_b[s0 + 4 * u]);
-                fl[u] = *reinterpret_cast<const f32x4_t*>(&seg_l[s0 + 4 * u]);
-                fc[u] = *reinterpret_cast<const u32x4_t*>(&seg_code[s0 + 4 * u]);
-            }
+                    for (int u = 0; u < MERGE_DEPTH / 4; ++u) {
+                        fa[u] = *reinterpret_cast<const f32x4_t*>(&seg_a[at + 4 * u]);
+                        fb[u] = *reinterpret_cast<const f32x4_t*>(&seg_b[at + 4 * u]);
+                        fl[u] = *reinterpret_cast<const f32x4_t*>(&seg_l[at + 4 * u]);
+                    }
+                    const int plain = round_plain[at / MERGE_DEPTH];
+                    const int count = min(MERGE_DEPTH, n - at);     // the round's segments that exist
+                    if (plain) {
+                        if (plain == 2) {
+                            L = fl[0][0];
+                            O[0] = ring[r][0][0];
+                            if constexpr (WIDE) O[1] = ring[r][1][0];
+                        } else {
+                            L = L * fa[0][0] + fl[0][0] * fb[0][0];
+                            O[0] = O[0] * fa[0][0] + ring[r][0][0] * fb[0][0];
+                            if constexpr (WIDE) O[1] = O[1] * fa[0][0] + ring[r][1][0] * fb[0][0];
+                        }
+                        if (count == MERGE_DEPTH) {
 #pragma unroll
-            for (int u = 0; u < MERGE_DEPTH; ++u) {
-                const uint32_t code = (s0 + u < n) ? fc[u / 4][u % 4] : 0u;
-                const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
-                const float l_fold = L * a + l * b, o0_fold = O[0] * a + ov[0][u] * b;
-                L = code == 2u ? l_fold : (code == 1u ? l : L);
-                O[0] = code == 2u ? o0_fold : (code == 1u ? ov[0][u] : O[0]);
-                if constexpr (WIDE) {
-                    const float o1_fold = O[1] * a + ov[1][u] * b;
-                    O[1] = code == 2u ? o1_fold : (code == 1u ? ov[1][u] : O[1]);
+                            for (int u = 1; u < MERGE_DEPTH; ++u) {
+                                const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
+                                L = L * a + l * b;
+                                O[0] = O[0] * a + ring[r][0][u] * b;
+                                if constexpr (WIDE) O[1] = O[1] * a + ring[r][1][u] * b;
+                            }
+                        } else {
+#pragma unroll
+                            for (int u = 1; u < MERGE_DEPTH; ++u) {
+                                if (u < count) {    // the same for every thread
+                                    const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
+                                    L = L * a + l * b;
+                                    O[0] = O[0] * a + ring[r][0][u] * b;
+                                    if constexpr (WIDE) O[1] = O[1] * a + ring[r][1][u] * b;
+                                }
+                            }
+                        }
+                    } else {
+                        u32x4_t fc[MERGE_DEPTH / 4];
+#pragma unroll
+                        for (int u = 0; u < MERGE_DEPTH / 4; ++u) fc[u] = *reinterpret_cast<const u32x4_t*>(&seg_code[at + 4 * u]);
+#pragma unroll
+                        for (int u = 0; u < MERGE_DEPTH; ++u) {
+                            const uint32_t code = (at + u < n) ? fc[u / 4][u % 4] : 0u;
+                            const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
+                            const float l_fold = L * a + l * b, o0_fold = O[0] * a + ring[r][0][u] * b;
+                            L = code == 2u ? l_fold : (code == 1u ? l : L);
+                            O[0] = code == 2u ? o0_fold : (code == 1u ? ring[r][0][u] : O[0]);
+                            if constexpr (WIDE) {
+                                const float o1_fold = O[1] * a + ring[r][1][u] * b;
+                                O[1] = code == 2u ? o1_fold : (code == 1u ? ring[r][1][u] : O[1]);
+                            }
+                        }
+                    }
+                    // the round's registers are free: ask for the round one turn of the ring ahead
+                    const int next = c0 + at + MERGE_DEPTH * MERGE_RING;
+                    if (next < n_seg) fetch(ring[r], next);
                 }
             }
         }
@@ -809,6 +862,9 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
     if (tid < D) out[((size_t)t * n_heads + h) * D + tid] = f32_to_bf16(O[0] * inv);
     if (WIDE && tid + 128 < D) out[((size_t)t * n_heads + h) * D + tid + 128] = f32_to_bf16(O[WIDE ? 1 : 0] * inv);
 }
+
+// Rows part_o must have beyond its slots' (see the merge).
+extern "C" int llmx_attention_partial_pad() { return MERGE_PAD; }
 
 // `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 8: one workgroup each 8, or
 // each 4 for head sizes other than 128),
@@ -845,12 +901,13 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
 #undef AM_CASE
         default: return -2;
     }
-    if (n_merges > 0)
+    if (n_merges > 0) {
         if (head_dim > 128)
             hipLaunchKernelGGL(attention_merge_kernel<true>, dim3(n_merges), dim3(128), 0, stream, merges, pos, part_o, part_ml, (bf16_t*)out, n_heads,
                                head_dim, window);
         else
             hipLaunchKernelGGL(attention_merge_kernel<false>, dim3(n_merges), dim3(128), 0, stream, merges, pos, part_o, part_ml, (bf16_t*)out, n_heads,
                                head_dim, window);
+    }
     return LLMX_CHECK_LAUNCH();
 }

@@ -57,6 +57,7 @@ def _declare(h) -> None:
         "llmx_fill_i32": [P, I, L, P],
         "llmx_fill_random": [P, I, L, ctypes.c_ulonglong, I, F, F, P],
         "llmx_read_probe": [P, L, P, P],
+        "llmx_attention_partial_pad": [],
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
@@ -314,9 +315,9 @@ def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, 
                 items.append([row0s[i], 1, head0, nh, 0, 1, -1, 0])
                 continue
             for c in range(nh):
-                merges.append([row0s[i], head0 + c, slot, c, 0, 0, 0, 0])
+                merges.append([row0s[i], head0 + c, slot, c, seg_cap, 0, 0, 0])
             for sp in range(n_splits):
-                items.append([row0s[i], 1, head0, nh, sp, n_splits, slot, 0])
+                items.append([row0s[i], 1, head0, nh, sp, n_splits, slot, seg_cap])
             slot += seg_cap
     plan = AttentionPlan(shared, items, merges, slot, device)
     if len(_PLAN_CACHE) > 256:
@@ -348,7 +349,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         if plan.n_slots:
             if scratch is None:
                 scratch = lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=q.device)
-            part_o = scratch("attention.part_o", (plan.n_slots * 16, head_dim), torch.float32)
+            # the merge's loads run a fixed number of segments past a row's last one (never used)
+            part_o = scratch("attention.part_o", (plan.n_slots * 16 + lib().llmx_attention_partial_pad(), head_dim), torch.float32)
             part_ml = scratch("attention.part_ml", (plan.n_slots * 16, 2), torch.float32)
         _check(lib().llmx_paged_attention_mfma(*common, _dev(plan.items, "items", torch.int32), plan.n_shared, plan.n_direct,
                                                plan.n_items - plan.n_shared - plan.n_direct,
