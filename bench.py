@@ -39,7 +39,8 @@ def parse():
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-calibration", action="store_true", help="skip the copy, read and library-product rates of the card")
-    ap.add_argument("--logits-to-host", action="store_true", help="also measure the default batch with every step's logits copied to the host")
+    ap.add_argument("--no-logits-to-host", action="store_true",
+                    help="skip the extra point: the default batch with every step's logits copied to the host")
     ap.add_argument("--only-prefill", action="store_true", help="for profiling: measure the prefill alone and print its record")
     ap.add_argument("--context-fill", choices=["synthetic", "prefill"], default="synthetic",
                     help="how the context before the timed steps gets into the cache: random keys and values written "
@@ -273,7 +274,7 @@ def main():
     }
 
     pts = {}
-    if a.logits_to_host:
+    if points and not a.no_logits_to_host:
         dtb, _ = run_decode(engine, sampler_out, a.batch, context, a.steps, a.warmup, a.context_fill, torch, read_logits=True)
         pts[f"decode_b{a.batch}_logits_to_host"] = round(a.batch * a.steps / dtb, 2)
     for b in points:
