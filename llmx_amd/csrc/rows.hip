@@ -40,13 +40,50 @@ __global__ void __launch_bounds__(RMS_THREADS) rmsnorm_kernel(const float* __res
     }
 }
 
+// The same for rows of at most RMS_THREADS * RMS_KEPT values: a thread keeps its values and the weights in registers,
+// all asked for before the sum is formed, so the kernel waits for memory once.  The same operations in the same order.
+#define RMS_KEPT 8
+template <typename TO>
+__global__ void __launch_bounds__(RMS_THREADS) rmsnorm_kept_kernel(const float* __restrict__ x, const int* __restrict__ pick,
+                                                                 const float* __restrict__ w, float eps, TO* __restrict__ out,
+                                                                 float* __restrict__ out32, int n) {
+    __shared__ float scratch[RMS_THREADS / 64];
+    const int r = blockIdx.x;
+    const float* row = x + (size_t)(pick ? pick[r] : r) * n;
+    float v[RMS_KEPT], nw[RMS_KEPT];
+#pragma unroll
+    for (int e = 0; e < RMS_KEPT; ++e) {
+        const int i = threadIdx.x + e * RMS_THREADS;
+        v[e] = i < n ? row[i] : 0.0f;
+        nw[e] = i < n ? w[i] : 0.0f;
+    }
+    float sq = 0.0f;     // strided_squares' order (an element past the end adds fmaf(0, 0, s) = s)
+#pragma unroll
+    for (int e = 0; e < RMS_KEPT; ++e) sq = fmaf(v[e], v[e], sq);
+    const float s = block_sum<RMS_THREADS / 64>(sq, scratch);
+    const float scale = 1.0f / sqrtf(s / (float)n + eps);
+#pragma unroll
+    for (int e = 0; e < RMS_KEPT; ++e) {
+        const int i = threadIdx.x + e * RMS_THREADS;
+        if (i < n) {
+            const float y = v[e] * (scale * nw[e]);
+            if (out) st(out + (size_t)r * n + i, y);
+            if (out32) out32[(size_t)r * n + i] = y;
+        }
+    }
+}
+
 extern "C" int llmx_rmsnorm(const float* x, const int* pick, const float* w, float eps, void* out, int out_dtype, float* out32,
                             int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (out_dtype == LLMX_F32)
-        hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (float*)out, out32, n);
-    else
-        hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (bf16_t*)out, out32, n);
+    const bool kept = n <= RMS_THREADS * RMS_KEPT;
+    if (out_dtype == LLMX_F32) {
+        if (kept) hipLaunchKernelGGL(rmsnorm_kept_kernel<float>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (float*)out, out32, n);
+        else hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (float*)out, out32, n);
+    } else {
+        if (kept) hipLaunchKernelGGL(rmsnorm_kept_kernel<bf16_t>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (bf16_t*)out, out32, n);
+        else hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (bf16_t*)out, out32, n);
+    }
     return LLMX_CHECK_LAUNCH();
 }
 
@@ -58,11 +95,19 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(float* __restrict__ x,
     const int t = blockIdx.y;
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= width) return;
-    float s = 0.0f;
-    for (int j = 0; j < k; ++j)
-        if (ids[t * k + j] >= 0) s += w[t * k + j] * y[((size_t)t * k + j) * width + i];
     float* o = x + (size_t)t * width + i;
-    *o = accumulate ? *o + s : s;
+    const float old = accumulate ? *o : 0.0f;
+    float s = 0.0f;
+    for (int j0 = 0; j0 < k; j0 += 8) {
+        // the slots' rows are asked for whether or not a slot has an expert (its row exists either way), so nothing waits for the ids
+        float yv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) yv[u] = j0 + u < k ? y[((size_t)t * k + j0 + u) * width + i] : 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (j0 + u < k && ids[t * k + j0 + u] >= 0) s += w[t * k + j0 + u] * yv[u];
+    }
+    *o = accumulate ? old + s : s;
 }
 
 // The same sums, four neighbouring elements a thread (width a multiple of 4): 16-byte loads for steps of many rows.

@@ -143,6 +143,7 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[tor
 
 
 SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores
+TILE_FILL = 1024              # feature tiles of 128 from which the tiled kernel fills the chip with one tile of rows
 SKINNY_MAX_GROUPED_ROWS = 16   # routed products of at most this many token rows do (measured: beyond it the tiled kernel streams the experts faster)
 
 
@@ -172,7 +173,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
     N = w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]   # swiglu: w holds gate rows, then up rows
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
-    if not force_generic and M <= SKINNY_MAX_ROWS and _skinny_ok(a, w, c, epilogue):
+    # beyond 16 rows a product wide enough to fill the chip with tiles streams its weights faster through the tiled kernel
+    # (the LM head); both kernels give a row the same bits
+    skinny = M <= 16 or (M <= SKINNY_MAX_ROWS and -(-N // 128) < TILE_FILL)
+    if not force_generic and skinny and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()),
                "gemm_skinny")
