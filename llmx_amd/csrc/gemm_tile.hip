@@ -58,7 +58,7 @@ struct TileArgs {
 // one barrier a tile.
 template <int EPI, typename TC, bool GROUPED, bool SPLIT, bool FAST, int BM>
 __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
-    // FAST: 3 stages of unpadded 128-byte rows whose 16-byte chunks are swizzled; else one tile of padded rows
+    // FAST: TL_STAGES tiles of unpadded 128-byte rows whose 16-byte chunks are swizzled; else one tile of padded rows
     __shared__ __attribute__((aligned(1024))) bf16_t As[FAST ? TL_STAGES * BM * TL_BK : BM * TL_LD];
     __shared__ __attribute__((aligned(1024))) bf16_t Ws[FAST ? TL_STAGES * TL_BN * TL_BK : TL_BN * TL_LD];
     __shared__ int rows_a[BM];
