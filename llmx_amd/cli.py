@@ -202,6 +202,21 @@ def cmd_replay(a) -> int:
     return replay(a.rest)
 
 
+def cmd_bench(rest) -> int:
+    """bench.py at the repository's root, with its own flags."""
+    import runpy
+    script = Path(__file__).resolve().parent.parent / "bench.py"
+    old = sys.argv
+    sys.argv = [str(script)] + list(rest)
+    try:
+        runpy.run_path(str(script), run_name="__main__")
+    except SystemExit as e:
+        return int(e.code or 0)
+    finally:
+        sys.argv = old
+    return 0
+
+
 def cmd_random(a) -> int:
     """Writes a model folder (config.json, model.safetensors) with seeded random weights."""
     from .models import read_config
@@ -257,7 +272,7 @@ def build_parser():
     r.set_defaults(run=cmd_random)
     b = sub.add_parser("bench", help="decode and prefill throughput of a random-weight model (see bench.py)")
     b.add_argument("rest", nargs=argparse.REMAINDER)
-    b.set_defaults(run=lambda a: __import__("runpy").run_path(str(Path(__file__).resolve().parent.parent / "bench.py"), run_name="__main__") and 0)
+    b.set_defaults(run=lambda a: cmd_bench(a.rest))
     return ap
 
 
@@ -267,6 +282,8 @@ def main(argv=None) -> int:
     try:
         if argv and argv[0] == "replay":      # its own parser reads every flag, --help included
             return cmd_replay(argparse.Namespace(rest=argv[1:]))
+        if argv and argv[0] == "bench":
+            return cmd_bench(argv[1:])
         a = ap.parse_args(argv)
         return a.run(a)
     except SystemExit2 as e:
