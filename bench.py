@@ -7,7 +7,10 @@ step, one new token each, logits -> greedy token on the device -> ids read back 
 /root/reference/src/cli/main.cpp:1246-1254, reads each pass's results before the next).  Prints one JSON line:
 `value` = decoded tokens a second at the default batch; `points` = the same at batch 1 and 64; `prefill` = one
 2,048-token prompt from an empty cache; `roofline` = bytes the decode step has to read / its time against HBM's 8 TB/s;
-`calibration` = what a device copy, a read-only pass and a square bf16 library product reach on this card.
+`calibration` = what a device copy, a read-only pass and a square bf16 library product reach on this card.  The prefill
+record's `frac` is its flops over the bf16 peak; beside it `hbm_frac` is the weights it has to read (the experts its
+tokens picked, counted in the warm-up run) over its time against 8 TB/s: few rows an expert make the step a
+weight-streaming one.
 Token ids are a fixed LCG sequence; weights are N(0, 0.02) generated on the device.
 """
 
@@ -195,10 +198,12 @@ def run_prefill(engine, cfg, sampler_out, torch):
     from llmx_amd.engine import StepEntry
     T = PREFILL_TOKENS
     times = []
-    for rep in range(3):   # the first is the warm-up
+    watcher = DistinctExperts()
+    for rep in range(3):   # the first is the warm-up; it also counts the experts the prompt touches per layer
         rid = f"p{rep}"
         engine.add_request(rid)
         ids = lcg_ids(T, cfg.vocab_size, 500 + rep)
+        engine.observer = watcher if rep == 0 else None
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         logits = engine.step([StepEntry(rid, ids, [T - 1])])
@@ -207,10 +212,15 @@ def run_prefill(engine, cfg, sampler_out, torch):
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         engine.end_request(rid)
+    engine.observer = None
     t = min(times[1:])
     flops = prefill_flops(cfg, T)
+    # what the step has to read: every weight it uses once (the experts the prompt's tokens picked), as for decode
+    distinct = sum(watcher.counts) / max(1, len(watcher.counts))
+    need = decode_bytes(cfg, 0, 0, distinct)
     return {"value": round(T / t, 1), "tokens": T, "ms": round(t * 1e3, 3), "frac": round(flops / t / PEAK_FLOPS["bf16"], 5),
-            "tflop": round(flops / 1e12, 2)}
+            "tflop": round(flops / 1e12, 2), "distinct_experts_per_layer": round(distinct, 1), "weights_read_gb": round(need / 1e9, 1),
+            "hbm_frac": round(need / t / 1e9 / HBM_PEAK_GBS, 4)}
 
 
 def main():

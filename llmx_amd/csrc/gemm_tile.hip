@@ -8,6 +8,10 @@
 // through the expert-sorted pair list and C's rows scattered to the pairs.  SwiGLU form: the tile's 128 weight rows
 // are 64 gate rows and the 64 up rows of the same features, and silu(gate) * up is stored.
 //
+// Three forms of the lean loop share this arithmetic: 4 waves on 64 x 128 (three workgroups a CU), 4 waves on 128 x 128
+// (each wave 64 x 64: fewer operand reads a product) and the wide form of 8 waves on 128 x 256 further down; the
+// launcher says which runs when.
+//
 // The arithmetic of an output element is the weight-streaming kernel's, bit for bit: the same 16x16x32 instruction with
 // the weights as its A operand and the same k-slots, K cut into the same `ks` runs of 32-wide steps, each run summed
 // from zero in step order, the runs' sums added in run order.  So a row's result does not depend on whether its step
@@ -50,7 +54,17 @@ struct TileArgs {
     int m_tiles;  // dense: number of row tiles
     int ks;       // runs K is cut into (the weight-streaming kernel's waves per strip for this shape)
     int bm;       // rows a workgroup covers: 64 or 128
+    const int* tile_stats;  // grouped, optional: [0] = sum over groups of ceil(rows / 128)
+    int run_if_big;         // with tile_stats: 1: this launch works only if the groups fill 128-row tiles, 0: only if not
 };
+
+// Whether the groups' rows fill tiles of 128 rows: at most a quarter of the tiles' rows would be padding.  The launcher
+// cannot know (the counts are on the device), so it launches the form for either case and one of them leaves at once.
+__device__ __forceinline__ bool tile_launch_runs(const TileArgs& g) {
+    if (!g.tile_stats) return true;
+    const bool big = (long)g.tile_stats[0] * 128 * 4 <= (long)g.M * 5;
+    return big == (g.run_if_big != 0);
+}
 
 // FAST: K is a multiple of 64 and the runs end on multiples of 64, so nothing in the loop needs a bound: the tiles are
 // loaded without conditions (a row past the tile's rows reads the first row, a feature past N the last; what they
@@ -59,14 +73,16 @@ struct TileArgs {
 template <int EPI, typename TC, bool GROUPED, bool SPLIT, bool FAST, int BM>
 __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     // FAST: TL_STAGES tiles of unpadded 128-byte rows whose 16-byte chunks are swizzled; else one tile of padded rows
-    __shared__ __attribute__((aligned(1024))) bf16_t As[FAST ? TL_STAGES * BM * TL_BK : BM * TL_LD];
-    __shared__ __attribute__((aligned(1024))) bf16_t Ws[FAST ? TL_STAGES * TL_BN * TL_BK : TL_BN * TL_LD];
+    constexpr int STAGES = TL_STAGES;
+    __shared__ __attribute__((aligned(1024))) bf16_t As[FAST ? STAGES * BM * TL_BK : BM * TL_LD];
+    __shared__ __attribute__((aligned(1024))) bf16_t Ws[FAST ? STAGES * TL_BN * TL_BK : TL_BN * TL_LD];
     __shared__ int rows_a[BM];
     __shared__ int rows_c[BM];
     __shared__ int tile_info[2];
     __shared__ int scan_waves[4];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    if (GROUPED && !tile_launch_runs(g)) return;
     constexpr int FEATS = (EPI == TL_SWIGLU) ? 64 : 128;  // output features a workgroup covers
     const int n0 = blockIdx.x * FEATS;
     const bf16_t* W = g.W;
@@ -278,7 +294,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         };
         issue(0, 0);
 #pragma unroll
-        for (int ahead = 1; ahead < TL_STAGES - 1; ++ahead)
+        for (int ahead = 1; ahead < STAGES - 1; ++ahead)
             if (ahead < n_tiles) issue(ahead, ahead);
         int t = 0, stage = 0;
         for (int run_end = tiles_per_run;; run_end += tiles_per_run) {
@@ -286,13 +302,13 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
             for (; t < stop; ++t) {
                 // tile t has arrived when at most the loads of tile t+1 are still out; then everybody's have, and
                 // everybody is done with the stage that tile t+2 goes into
-                constexpr int OUT = LOADS * (TL_STAGES - 2);   // loads of the tiles after t that may still be out
-                if (t + TL_STAGES - 2 < n_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (OUT & 15) | ((OUT >> 4) << 14));
+                constexpr int OUT = LOADS * (STAGES - 2);   // loads of the tiles after t that may still be out
+                if (t + STAGES - 2 < n_tiles) __builtin_amdgcn_s_waitcnt(0x0F70 | (OUT & 15) | ((OUT >> 4) << 14));
                 else __builtin_amdgcn_s_waitcnt(0x0F70);
                 __syncthreads();
-                if (t + TL_STAGES - 1 < n_tiles) issue(t + TL_STAGES - 1, stage == 0 ? TL_STAGES - 1 : stage - 1);
+                if (t + STAGES - 1 < n_tiles) issue(t + STAGES - 1, stage == 0 ? STAGES - 1 : stage - 1);
                 multiply(stage);
-                stage = stage == TL_STAGES - 1 ? 0 : stage + 1;
+                stage = stage == STAGES - 1 ? 0 : stage + 1;
             }
             if (t >= n_tiles) break;
             if (SPLIT) {
@@ -394,60 +410,352 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     }
 }
 
+// The wide form of the lean loop, for products with many rows a group: a workgroup of 8 waves computes 128 rows x 256
+// weight rows (each wave 64 x 64 as 4 x 4 products), three tiles deep in LDS (144 KB: one workgroup a CU, two waves a
+// SIMD).  What bounds the 4-wave form is the tiles' way into LDS: a 64 x 128 tile needs 24 KB per 1 MFLOP and a tile is
+// asked for only one multiplication ahead, far less than the memory's latency; here 48 KB serve 4 MFLOP and two tiles
+// (96 KB) are on their way while one is multiplied.  Per output element nothing differs from the other forms: the same
+// instruction, the same k-slots, the same runs.
+#define WD_BM 128
+#define WD_BN 256
+#define WD_STAGES 3
 template <int EPI, typename TC, bool GROUPED, bool SPLIT>
-static void tile_launch_fast(const TileArgs& g, dim3 grid, hipStream_t stream) {
-    // the lean loop needs whole 64-wide tiles and runs that end on them
-    const int steps = (g.K + 31) / 32, per = (steps + g.ks - 1) / g.ks;
-    if (g.K % TL_BK == 0 && (!SPLIT || per % 2 == 0)) {
-        if (g.bm == 128) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true, 128>), grid, dim3(256), 0, stream, g);
-        else hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true, 64>), grid, dim3(256), 0, stream, g);
+__global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
+    __shared__ __attribute__((aligned(1024))) bf16_t As[WD_STAGES * WD_BM * TL_BK];
+    __shared__ __attribute__((aligned(1024))) bf16_t Ws[WD_STAGES * WD_BN * TL_BK];
+    __shared__ int rows_a[WD_BM];
+    __shared__ int rows_c[WD_BM];
+    __shared__ int tile_info[2];
+    __shared__ int scan_waves[8];
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    if (GROUPED && !tile_launch_runs(g)) return;
+    constexpr int HALF = WD_BN / 2;                               // SwiGLU: gate rows, then the up rows of the same features
+    constexpr int FEATS = (EPI == TL_SWIGLU) ? HALF : WD_BN;      // output features a workgroup covers
+    const int n0 = blockIdx.x * FEATS;
+    const bf16_t* W = g.W;
+    int row_begin, row_end;
+    if (GROUPED) {
+        // which (expert, row tile) this workgroup has: experts in order, each with ceil(rows / 128) tiles
+        if (tid == 0) tile_info[0] = -1;
+        int base = 0;
+        for (int e0 = 0; e0 < g.n_groups; e0 += 512) {
+            const int e = e0 + tid;
+            const int begin = e < g.n_groups ? g.group_offsets[e] : 0;
+            const int tiles = e < g.n_groups ? (g.group_offsets[e + 1] - begin + WD_BM - 1) / WD_BM : 0;
+            int incl = tiles;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int o = __shfl_up(incl, d, 64);
+                if (lane >= d) incl += o;
+            }
+            if (lane == 63) scan_waves[wave] = incl;
+            __syncthreads();
+            int before = base, round_total = 0;
+            for (int w = 0; w < 8; ++w) {
+                if (w < wave) before += scan_waves[w];
+                round_total += scan_waves[w];
+            }
+            const int first = before + incl - tiles;
+            if ((int)blockIdx.y >= first && (int)blockIdx.y < first + tiles) {
+                tile_info[0] = e;
+                tile_info[1] = (int)blockIdx.y - first;
+            }
+            base += round_total;
+            __syncthreads();
+            if ((int)blockIdx.y < base) break;
+        }
+        __syncthreads();
+        const int e = tile_info[0];
+        if (e < 0) return;
+        row_begin = g.group_offsets[e] + tile_info[1] * WD_BM;
+        row_end = min(g.group_offsets[e + 1], row_begin + WD_BM);
+        W += (size_t)e * g.w_group_stride;
     } else {
-        hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, false, 64>), grid, dim3(256), 0, stream, g);
+        row_begin = blockIdx.y * WD_BM;
+        row_end = min(g.M, row_begin + WD_BM);
     }
+    if (tid < WD_BM) {
+        const int m = row_begin + tid;
+        int ra = -1, rc = -1;
+        if (m < row_end) {
+            if (GROUPED) {
+                const int p = g.list[m];
+                ra = p / g.a_div;
+                rc = p;
+            } else {
+                ra = rc = m;
+            }
+        }
+        rows_a[tid] = ra;
+        rows_c[tid] = rc;
+    }
+    __syncthreads();
+
+    const int K = g.K;
+    // wave (wm, wn): rows 64 * wm .. (4 tiles of 16), 4 tiles of 16 weight rows
+    const int wm = wave >> 2, wn = wave & 3;
+    const int lr = lane & 15;
+    int w_row[4];  // LDS rows of the wave's 4 feature tiles
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+        if (EPI == TL_SWIGLU)
+            w_row[f] = (f < 2 ? 0 : HALF) + 32 * wn + 16 * (f & 1) + lr;   // tiles 0,1: gate rows; tiles 2,3: the up rows of the same features
+        else
+            w_row[f] = 64 * wn + 16 * f + lr;
+    }
+    constexpr int TT = 4;
+    f32x4_t acc[4][TT], total[SPLIT ? 4 : 1][SPLIT ? TT : 1];
+#pragma unroll
+    for (int f = 0; f < 4; ++f)
+#pragma unroll
+        for (int t = 0; t < TT; ++t) acc[f][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    const int steps_total = (K + 31) >> 5;
+    const int per = (steps_total + g.ks - 1) / g.ks;   // 32-wide steps in a run
+    bool first_run = true;
+
+    // the same unpadded, swizzled rows as the 4-wave form: chunk c (16 bytes) of row r sits at place c ^ ((r >> 1) & 7)
+    constexpr int W_LOADS = 4, A_LOADS = 2, LOADS = W_LOADS + A_LOADS;   // load instructions a wave issues per tile
+    const int n_tiles = K / TL_BK;
+    const int tiles_per_run = SPLIT ? per / 2 : n_tiles;
+    uint32_t w_at[W_LOADS], a_at[A_LOADS];
+    const int place = lane & 7;
+#pragma unroll
+    for (int j = 0; j < W_LOADS; ++j) {
+        const int r = 32 * wave + 8 * j + (lane >> 3);           // row of the W tile
+        const int ch = place ^ ((r >> 1) & 7);
+        int wr;
+        if (EPI == TL_SWIGLU) wr = (r < HALF ? 0 : g.up_offset) + min(n0 + (r & (HALF - 1)), g.N - 1);
+        else wr = min(n0 + r, g.N - 1);
+        w_at[j] = (uint32_t)(((size_t)wr * K + 8 * ch) * sizeof(bf16_t));
+    }
+#pragma unroll
+    for (int j = 0; j < A_LOADS; ++j) {
+        const int r = 16 * wave + 8 * j + (lane >> 3);           // row of the A tile
+        const int ch = place ^ ((r >> 1) & 7);
+        const int ra = rows_a[r];
+        a_at[j] = (uint32_t)(((size_t)(ra >= 0 ? ra : 0) * g.lda + 8 * ch) * sizeof(bf16_t));
+    }
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto issue = [&](int t, int stage) {
+        const bf16_t* wb = W + (size_t)t * TL_BK;
+        const bf16_t* ab = g.A + (size_t)t * TL_BK;
+#pragma unroll
+        for (int j = 0; j < W_LOADS; ++j) load_to_lds(wb, w_at[j], &Ws[(stage * WD_BN + 32 * wave_u + 8 * j) * TL_BK]);
+#pragma unroll
+        for (int j = 0; j < A_LOADS; ++j) load_to_lds(ab, a_at[j], &As[(stage * WD_BM + 16 * wave_u + 8 * j) * TL_BK]);
+    };
+    int w_rd[4], a_rd[TT], w_swz[4], a_swz[TT];
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+        w_rd[f] = w_row[f] * TL_BK;
+        w_swz[f] = (w_row[f] >> 1) & 7;
+    }
+#pragma unroll
+    for (int q = 0; q < TT; ++q) {
+        const int r = 64 * wm + 16 * q + lr;
+        a_rd[q] = r * TL_BK;
+        a_swz[q] = (r >> 1) & 7;
+    }
+    const int kg = lane >> 4;
+    // the operands of one half (32 of k) of a stage's tile
+    auto read_half = [&](int stage, int kk, bf16x8_t (&wf)[4], bf16x8_t (&af)[TT]) {
+        const bf16_t* ws = &Ws[stage * WD_BN * TL_BK];
+        const bf16_t* as = &As[stage * WD_BM * TL_BK];
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+            wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&ws[w_rd[f] + 8 * ((kk / 8 + kg) ^ w_swz[f])]));
+#pragma unroll
+        for (int q = 0; q < TT; ++q)
+            af[q] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&as[a_rd[q] + 8 * ((kk / 8 + kg) ^ a_swz[q])]));
+    };
+    auto multiply_half = [&](const bf16x8_t (&wf)[4], const bf16x8_t (&af)[TT]) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+#pragma unroll
+            for (int q = 0; q < TT; ++q) acc[f][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[q], acc[f][q], 0, 0, 0);
+    };
+    // Three tiles in LDS; while a tile's first half is multiplied its second half's operands are read, and while the
+    // second half is multiplied the next tile's first: the matrix cores and LDS work at the same time, also within a
+    // wave.  One barrier a tile, in its middle: by then a wave has all operands of tile t in registers, so after the
+    // barrier tile t's stage takes tile t+3, and tile t+1 (awaited before the barrier) can be read by everybody.
+    issue(0, 0);
+    if (1 < n_tiles) issue(1, 1);
+    if (2 < n_tiles) issue(2, 2);
+    {
+        const int out = (n_tiles > 2 ? 2 : n_tiles - 1) * LOADS;   // loads of the tiles after the first that may still be out
+        if (out == 2 * LOADS) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * LOADS));
+        else if (out == LOADS) __builtin_amdgcn_s_waitcnt(0x0F70 | LOADS);
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __syncthreads();
+    bf16x8_t wf_a[4], af_a[TT], wf_b[4], af_b[TT];
+    read_half(0, 0, wf_a, af_a);
+    int t = 0, stage = 0;
+    const int last = n_tiles - 1;   // the last tile has no tile after it: it runs after the loop, so the loop's body has no branch around its reads
+    for (int run_end = tiles_per_run;; run_end += tiles_per_run) {
+        const int stop = min(run_end, last);
+        for (; t < stop; ++t) {
+            read_half(stage, 32, wf_b, af_b);
+            multiply_half(wf_a, af_a);
+            const int next = stage == 2 ? 0 : stage + 1;
+            // this wave's operand reads of tile t are done, and its part of tile t+1 has arrived (tile t+2's may be out)
+            if (t + 2 < n_tiles) __builtin_amdgcn_s_waitcnt(0x0070 | LOADS);
+            else __builtin_amdgcn_s_waitcnt(0x0070);
+            __syncthreads();
+            if (t + 3 < n_tiles) issue(t + 3, stage);
+            read_half(next, 0, wf_a, af_a);
+            multiply_half(wf_b, af_b);
+            stage = next;
+        }
+        if (SPLIT && t == run_end && t < n_tiles) {
+            // a run of K ends: its sum joins the runs before it, in run order
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+#pragma unroll
+                for (int q = 0; q < TT; ++q) {
+                    if (first_run) total[f][q] = acc[f][q];
+                    else total[f][q] = f32x4_t{total[f][q][0] + acc[f][q][0], total[f][q][1] + acc[f][q][1],
+                                               total[f][q][2] + acc[f][q][2], total[f][q][3] + acc[f][q][3]};
+                    acc[f][q] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                }
+            first_run = false;
+        }
+        if (t >= last) break;
+    }
+    read_half(stage, 32, wf_b, af_b);
+    multiply_half(wf_a, af_a);
+    multiply_half(wf_b, af_b);
+    if (SPLIT && !first_run) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f)
+#pragma unroll
+            for (int q = 0; q < TT; ++q)
+                acc[f][q] = f32x4_t{total[f][q][0] + acc[f][q][0], total[f][q][1] + acc[f][q][1], total[f][q][2] + acc[f][q][2],
+                                    total[f][q][3] + acc[f][q][3]};
+    }
+
+    // acc[f][q][i]: feature (tile f) 4*(lane/16) + i, row 64*wm + 16*q + lane%16
+    const int fq = 4 * (lane >> 4);
+#pragma unroll
+    for (int q = 0; q < TT; ++q) {
+        const int rc = rows_c[64 * wm + 16 * q + lr];
+        if (rc < 0) continue;
+        TC* crow = (TC*)g.C + (size_t)rc * g.ldc;
+        if (EPI == TL_SWIGLU) {
+#pragma unroll
+            for (int f = 0; f < 2; ++f)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + 32 * wn + 16 * f + fq + i;
+                    if (n >= g.N) continue;
+                    const float gt = acc[f][q][i], u = acc[f + 2][q][i];
+                    st(crow + n, (gt / (1.0f + expf(-gt))) * u);
+                }
+        } else {
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + 64 * wn + 16 * f + fq + i;
+                    if (n >= g.N) continue;
+                    float x = acc[f][q][i];
+                    if (EPI == TL_ADD) x = ld(crow + n) + x;
+                    st(crow + n, x);
+                }
+        }
+    }
+}
+
+// form: which kernel takes the product.  The lean forms need whole 64-wide tiles of K and runs that end on them.
+enum : int { FORM_64 = 0, FORM_128 = 1, FORM_WIDE = 2, FORM_BOUNDED = 3 };
+
+template <int EPI, typename TC, bool GROUPED, bool SPLIT>
+static void tile_launch_form(const TileArgs& g, int form, dim3 grid, hipStream_t stream) {
+    if (form == FORM_WIDE) hipLaunchKernelGGL((gemm_wide_kernel<EPI, TC, GROUPED, SPLIT>), grid, dim3(512), 0, stream, g);
+    else if (form == FORM_128) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true, 128>), grid, dim3(256), 0, stream, g);
+    else if (form == FORM_64) hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, true, 64>), grid, dim3(256), 0, stream, g);
+    else hipLaunchKernelGGL((gemm_tile_kernel<EPI, TC, GROUPED, SPLIT, false, 64>), grid, dim3(256), 0, stream, g);
 }
 
 template <int EPI, typename TC>
-static void tile_launch(const TileArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
+static void tile_launch(const TileArgs& g, int form, dim3 grid, bool grouped, hipStream_t stream) {
     if (grouped) {
-        if (g.ks > 1) tile_launch_fast<EPI, TC, true, true>(g, grid, stream);
-        else tile_launch_fast<EPI, TC, true, false>(g, grid, stream);
+        if (g.ks > 1) tile_launch_form<EPI, TC, true, true>(g, form, grid, stream);
+        else tile_launch_form<EPI, TC, true, false>(g, form, grid, stream);
     } else {
-        if (g.ks > 1) tile_launch_fast<EPI, TC, false, true>(g, grid, stream);
-        else tile_launch_fast<EPI, TC, false, false>(g, grid, stream);
+        if (g.ks > 1) tile_launch_form<EPI, TC, false, true>(g, form, grid, stream);
+        else tile_launch_form<EPI, TC, false, false>(g, form, grid, stream);
     }
 }
 
+static int tile_launch_typed(const TileArgs& g, int form, dim3 grid, bool grouped, int epi, int c_dtype, hipStream_t stream) {
+    if (epi == TL_SWIGLU) {
+        if (c_dtype == LLMX_BF16) tile_launch<TL_SWIGLU, bf16_t>(g, form, grid, grouped, stream);
+        else tile_launch<TL_SWIGLU, float>(g, form, grid, grouped, stream);
+    } else if (epi == TL_ADD) {
+        if (c_dtype != LLMX_F32) return -2;
+        tile_launch<TL_ADD, float>(g, form, grid, grouped, stream);
+    } else if (epi == TL_STORE) {
+        if (c_dtype == LLMX_BF16) tile_launch<TL_STORE, bf16_t>(g, form, grid, grouped, stream);
+        else tile_launch<TL_STORE, float>(g, form, grid, grouped, stream);
+    } else {
+        return -2;
+    }
+    return 0;
+}
+
+static int form_rows(int form) { return form == FORM_64 || form == FORM_BOUNDED ? 64 : 128; }
+static int form_feats(int form, int epi) { return (epi == TL_SWIGLU ? 64 : 128) * (form == FORM_WIDE ? 2 : 1); }
+
 // A and W bfloat16, K a multiple of 8.  n_groups == 0: dense over M rows.  n_groups > 0: grouped over the n_pairs = M
-// rows of `list`; `max_tiles` bounds the (expert, row tile) pairs (at most min(groups, pairs) + pairs / 64).
+// rows of `list`; `max_tiles` bounds the (expert, row tile) pairs of 64-row tiles (at most min(groups, pairs) + pairs / 64).
 // ks: the runs K is cut into; the caller passes what the weight-streaming kernel uses for this N and K.
+// tile_stats (grouped, optional): device int [1], the sum over groups of ceil(rows / 128), from the grouping.
+//
+// Which form runs (every form gives an output element the same bits):
+//   dense: the wide form (8 waves, 128 x 256, three tiles deep) where its tiles fill the chip one and a half times,
+//     else 64-row tiles (three workgroups a CU; more, smaller tiles fill the chip better when there are few).
+//   grouped with tile_stats: both a 128-row form (wide for long K, 4 waves for short K) and the 64-row form are
+//     launched; on the device the one that fits the groups' rows works and the other leaves at once.
 extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                               int n_groups, int max_tiles, const int* group_offsets, const int* list, int a_div, long w_group_stride,
-                              int up_offset, hipStream_t stream) {
+                              int up_offset, const int* tile_stats, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
     if (ks != 1 && ks != 2 && ks != 4 && ks != 8) return -2;
-    // 128-row tiles (each wave 64 x 64: fewer operand reads a product) where rows are many and the lean loop runs
     const int steps = (K + 31) / 32, per = (steps + ks - 1) / ks;
     const bool lean = K % TL_BK == 0 && (ks == 1 || per % 2 == 0);
-    const bool many = false;   // 128-row tiles halve the workgroups a CU holds and measured slower; the kernel keeps the variant
-    const int bm = lean && many ? 128 : 64;
     TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
-               w_group_stride, up_offset, (M + bm - 1) / bm, ks, bm};
-    const int feats = epi == TL_SWIGLU ? 64 : 128;
-    dim3 grid((N + feats - 1) / feats, grouped ? max_tiles : g.m_tiles, 1);
-    if (grid.y > 65535) return -2;
-    if (epi == TL_SWIGLU) {
-        if (c_dtype == LLMX_BF16) tile_launch<TL_SWIGLU, bf16_t>(g, grid, grouped, stream);
-        else tile_launch<TL_SWIGLU, float>(g, grid, grouped, stream);
-    } else if (epi == TL_ADD) {
-        if (c_dtype != LLMX_F32) return -2;
-        tile_launch<TL_ADD, float>(g, grid, grouped, stream);
-    } else if (epi == TL_STORE) {
-        if (c_dtype == LLMX_BF16) tile_launch<TL_STORE, bf16_t>(g, grid, grouped, stream);
-        else tile_launch<TL_STORE, float>(g, grid, grouped, stream);
+               w_group_stride, up_offset, 0, ks, 64, nullptr, 0};
+    auto launch = [&](int form, int tiles_y) -> int {
+        g.bm = form_rows(form);
+        g.m_tiles = (M + g.bm - 1) / g.bm;
+        const int feats = form_feats(form, epi);
+        dim3 grid((N + feats - 1) / feats, grouped ? tiles_y : g.m_tiles, 1);
+        if (grid.y > 65535) return -2;
+        return tile_launch_typed(g, form, grid, grouped, epi, c_dtype, stream);
+    };
+    int rc;
+    if (!lean) {
+        rc = launch(FORM_BOUNDED, max_tiles);
+    } else if (!grouped) {
+        const long wide_tiles = (long)((M + WD_BM - 1) / WD_BM) * ((N + form_feats(FORM_WIDE, epi) - 1) / form_feats(FORM_WIDE, epi));
+        rc = launch(wide_tiles >= 384 ? FORM_WIDE : FORM_64, 0);
+    } else if (tile_stats) {
+        // 128-row tiles: each group adds at most one partial tile
+        const int big_tiles = (n_groups < M ? n_groups : M) + M / 128;
+        g.tile_stats = tile_stats;
+        g.run_if_big = 1;
+        rc = launch(K >= 2048 ? FORM_WIDE : FORM_128, big_tiles < max_tiles ? big_tiles : max_tiles);
+        if (rc == 0) {
+            g.run_if_big = 0;
+            rc = launch(FORM_64, max_tiles);
+        }
     } else {
-        return -2;
+        rc = launch(FORM_64, max_tiles);
     }
+    if (rc) return rc;
     return LLMX_CHECK_LAUNCH();
 }

@@ -251,8 +251,9 @@ __global__ void __launch_bounds__(1024) moe_chunk_count_kernel(const int* __rest
 }
 
 __global__ void __launch_bounds__(1024) moe_chunk_scan_kernel(int n_chunks, int n_experts, int* __restrict__ chunk_counts, int* __restrict__ counts,
-                                                             int* __restrict__ offsets, int* __restrict__ active, int* __restrict__ n_active) {
-    __shared__ int wave_total[16], wave_active[16];
+                                                             int* __restrict__ offsets, int* __restrict__ active, int* __restrict__ n_active,
+                                                             int* __restrict__ tiles128) {
+    __shared__ int wave_total[16], wave_active[16], wave_tiles[16];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int e = tid;
     int c = 0;
@@ -267,11 +268,21 @@ __global__ void __launch_bounds__(1024) moe_chunk_scan_kernel(int n_chunks, int 
             incl_active += oa;
         }
     }
+    // how many tiles of 128 rows the experts' runs make: the products choose their tile size by it
+    int t128 = (c + 127) / 128;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) t128 += __shfl_xor(t128, d, 64);
     if (lane == 63) {
         wave_total[wave] = incl;
         wave_active[wave] = incl_active;
+        wave_tiles[wave] = t128;
     }
     __syncthreads();
+    if (tid == 0 && tiles128) {
+        int sum = 0;
+        for (int w = 0; w < 16; ++w) sum += wave_tiles[w];
+        tiles128[0] = sum;
+    }
     int before = incl - c, active_before = incl_active - (c > 0);
     for (int w = 0; w < wave; ++w) {
         before += wave_total[w];
@@ -315,8 +326,9 @@ __global__ void __launch_bounds__(1024) moe_chunk_place_kernel(const int* __rest
 
 // counts [X], offsets [X+1], list [n_pairs], active [X], n_active [1]
 // scratch (optional): [ceil(n_pairs / 1024) * n_experts] ints for steps of many pairs
+// tiles128 (optional) [1]: with scratch and many pairs, the sum over experts of ceil(rows / 128)
 extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* counts, int* offsets, int* list, int* active, int* n_active,
-                              int* scratch, hipStream_t stream) {
+                              int* scratch, int* tiles128, hipStream_t stream) {
     if (n_pairs <= 0 || n_experts <= 0) return 0;
     if (n_pairs <= ALIGN_SMALL_PAIRS && n_experts <= 1024) {
         hipLaunchKernelGGL(moe_align_small_kernel, dim3(1), dim3(1024), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
@@ -325,7 +337,7 @@ extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* c
     if (scratch && n_experts <= 1024) {
         const int n_chunks = (n_pairs + 1023) / 1024;
         hipLaunchKernelGGL(moe_chunk_count_kernel, dim3(n_chunks), dim3(1024), 0, stream, ids, n_pairs, n_experts, scratch);
-        hipLaunchKernelGGL(moe_chunk_scan_kernel, dim3(1), dim3(1024), 0, stream, n_chunks, n_experts, scratch, counts, offsets, active, n_active);
+        hipLaunchKernelGGL(moe_chunk_scan_kernel, dim3(1), dim3(1024), 0, stream, n_chunks, n_experts, scratch, counts, offsets, active, n_active, tiles128);
         hipLaunchKernelGGL(moe_chunk_place_kernel, dim3(n_chunks), dim3(1024), 0, stream, ids, n_pairs, n_experts, scratch, list);
         return LLMX_CHECK_LAUNCH();
     }

@@ -63,12 +63,12 @@ def _declare(h) -> None:
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P],
-        "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P],
+        "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
         "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
         "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P],
-        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
+        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
@@ -183,7 +183,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                    _split_k(-(-N // 16), K), 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm_tile")
+                                    _split_k(-(-N // 16), K), 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, 0, _stream()), "gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm")
@@ -191,7 +191,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_
 
 def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor, a_div: int,
                  epilogue: int = EPI_STORE, active: Optional[torch.Tensor] = None, n_active: Optional[torch.Tensor] = None,
-                 token_rows: Optional[int] = None, force_generic: bool = False) -> None:
+                 token_rows: Optional[int] = None, force_generic: bool = False, tile_stats: Optional[torch.Tensor] = None) -> None:
     """For each group g: rows p in pairs[offsets[g]:offsets[g+1]] get c[p] = a[p // a_div] @ w[g]^T.
 
     With EPI_SWIGLU w[g] holds gate rows then up rows and c[p] = silu(gate) * up.  `active` / `n_active` (from
@@ -218,7 +218,8 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
     if not force_generic and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                     _split_k(-(-N // 16), K), G, min(G, n_pairs) + n_pairs // 64, _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                    _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
+                                    _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0,
+                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), _stream()),
                "grouped_gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
@@ -391,11 +392,16 @@ def moe_align_scratch(n_pairs: int, n_experts: int) -> int:
     return 0 if n_pairs <= 1024 or n_experts > 1024 else -(-n_pairs // 1024) * n_experts
 
 
+TILE_STATS_MIN_PAIRS = 4096    # from this many pairs on the grouping also counts the experts' tiles of 128 rows
+
+
 def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
-              active: torch.Tensor, n_active: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> None:
+              active: torch.Tensor, n_active: torch.Tensor, scratch: Optional[torch.Tensor] = None,
+              tile_stats: Optional[torch.Tensor] = None) -> None:
     """Groups the pairs p = t*k + j by expert (stable): counts [X], offsets [X+1], pairs [T*k], and the experts that
     have rows in increasing order: active [X] (first n_active[0] entries).  `scratch`: moe_align_scratch(...) int32 for
-    steps of many pairs (made here when it is not given)."""
+    steps of many pairs (made here when it is not given).  `tile_stats` int32 [1]: for TILE_STATS_MIN_PAIRS pairs or
+    more it receives the sum over experts of ceil(rows / 128), by which grouped_gemm chooses its tile size."""
     n_pairs = ids.numel()
     need = moe_align_scratch(n_pairs, n_experts)
     if need and scratch is None:
@@ -405,13 +411,15 @@ def moe_align(ids: torch.Tensor, n_experts: int, counts: torch.Tensor, offsets: 
     _check(lib().llmx_moe_align(_dev(ids, "ids", torch.int32), n_pairs, n_experts, _dev(counts, "counts", torch.int32, (n_experts,)),
                                 _dev(offsets, "offsets", torch.int32, (n_experts + 1,)), _dev(pairs, "pairs", torch.int32, (n_pairs,)),
                                 _dev(active, "active", torch.int32, (n_experts,)), _dev(n_active, "n_active", torch.int32, (1,)),
-                                _dev(scratch if need else None, "scratch", torch.int32), _stream()), "moe_align")
+                                _dev(scratch if need else None, "scratch", torch.int32),
+                                _dev(tile_stats if need and n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)),
+                                _stream()), "moe_align")
 
 
 def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor, weights: torch.Tensor, k: int, score: int,
                      normalize: bool, scale: float, counts: torch.Tensor, offsets: torch.Tensor, pairs: torch.Tensor,
                      active: torch.Tensor, n_active: torch.Tensor, parts: Optional[torch.Tensor] = None,
-                     scratch: Optional[torch.Tensor] = None) -> None:
+                     scratch: Optional[torch.Tensor] = None, tile_stats: Optional[torch.Tensor] = None) -> None:
     """route_topk followed by moe_align; a step of at most 16 rows (sigmoid scores, at most 256 experts and 64 picks) does
     both in one launch, with the same bits."""
     rows, n_experts = z.shape
@@ -425,7 +433,7 @@ def route_topk_align(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.T
             _dev(n_active, "n_active", torch.int32, (1,)), _stream()), "route_topk_align")
         return
     route_topk(z, bias, ids, weights, k, score, normalize, scale, parts)
-    moe_align(ids, n_experts, counts, offsets, pairs, active, n_active, scratch)
+    moe_align(ids, n_experts, counts, offsets, pairs, active, n_active, scratch, tile_stats)
 
 
 def moe_combine(x: torch.Tensor, y: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, accumulate: bool = True) -> None:

@@ -92,13 +92,15 @@ class RoutedExperts(FeedForward):
         n_active = step.buf("experts.n_active", (1,), torch.int32)
         need = ops.moe_align_scratch(T * k, X)
         scratch = step.buf("experts.align_scratch", (need,), torch.int32) if need else None
+        # for steps of many pairs the grouping also counts the experts' tiles of 128 rows, by which the products choose their tiles
+        tile_stats = step.buf("experts.tile_stats", (1,), torch.int32) if T * k >= ops.TILE_STATS_MIN_PAIRS else None
         ops.route_topk_align(z, self.bias, ids, weights, k, self.score, self.normalize, self.scale, counts, offsets, pairs, active, n_active,
-                             parts=parts, scratch=scratch)
+                             parts=parts, scratch=scratch, tile_stats=tile_stats)
         step.observe("routing", logits=z, ids=ids, weights=weights)
         act = step.buf("experts.act", (T * k, self.intermediate), step.act_dtype)
-        ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T)
+        ops.grouped_gemm(h, self.w_gate_up, act, offsets, pairs, k, ops.EPI_SWIGLU, active, n_active, token_rows=T, tile_stats=tile_stats)
         y = step.buf("experts.y", (T * k, self.hidden), torch.float32)
-        ops.grouped_gemm(act, self.w_down, y, offsets, pairs, 1, ops.EPI_STORE, active, n_active, token_rows=T)
+        ops.grouped_gemm(act, self.w_down, y, offsets, pairs, 1, ops.EPI_STORE, active, n_active, token_rows=T, tile_stats=tile_stats)
         ops.moe_combine(out, y, ids, weights, accumulate)
 
 

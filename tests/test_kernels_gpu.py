@@ -126,6 +126,80 @@ def test_gemm_matrix_cores_bf16(M, N, K):
             assert torch.equal(few, c[rows]), "a row's bits depend on how many rows the product has"
 
 
+@pytest.mark.parametrize("M,N,K", [(1500, 8200, 128), (1536, 8192, 768), (1408, 8320, 3072)])
+def test_gemm_wide_tiles_give_the_bits_of_small_tiles(M, N, K):
+    """Products of many rows and features run on 128 x 256 tiles (8 waves); a row's bits are those of the 64-row tiles
+    that fewer rows take, for one run of K and for several, with ragged edges, for every epilogue."""
+    o = ops()
+    a = rnd(M, K, dtype=torch.bfloat16)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=1, scale=0.2)
+    c = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    o.gemm(a, w, c)
+    small = torch.empty_like(c)
+    for r0 in range(0, M, 200):
+        o.gemm(a[r0:r0 + 200], w, small[r0:r0 + 200])
+    assert torch.equal(c, small)
+    want = a.double() @ w.double().T                      # the library's float64 product as a calculator
+    assert (c.double() - want).abs().max() <= 1e-5 * math.sqrt(K) * want.abs().max()
+    cb = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    o.gemm(a, w, cb)
+    assert torch.equal(cb, c.to(torch.bfloat16))
+    base = rnd(M, N, seed=9)
+    acc = base.clone()
+    o.gemm(a, w, acc, o.EPI_ADD)
+    assert torch.equal(acc, base + c)
+    F = (N // 2) // 8 * 8
+    wgu = torch.cat([w[:F], w[N - F:]]).contiguous()
+    act, act_small = torch.empty(M, F, dtype=torch.bfloat16, device=DEV), torch.empty(M, F, dtype=torch.bfloat16, device=DEV)
+    o.gemm(a, wgu, act, o.EPI_SWIGLU)
+    for r0 in range(0, M, 200):
+        o.gemm(a[r0:r0 + 200], wgu, act_small[r0:r0 + 200], o.EPI_SWIGLU)
+    assert torch.equal(act, act_small)
+
+
+@pytest.mark.parametrize("T,X,k,E,F,full", [(1024, 8, 4, 128, 64, 8), (1100, 7, 4, 2048, 72, 5), (1024, 64, 4, 128, 64, 64)])
+def test_routed_products_choose_their_tiles_on_the_device(T, X, k, E, F, full):
+    """With the grouping's count of 128-row tiles the routed products run on 128-row tiles where the experts' rows fill
+    them (the wide form for long K) and on 64-row tiles where they do not; the bits are the same either way."""
+    o = ops()
+    g = torch.Generator().manual_seed(T + X)
+    ids = torch.stack([torch.randperm(full, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    ids[3, 1] = -1
+    ids_d = ids.to(DEV)
+    h = rnd(T, E, dtype=torch.bfloat16)
+    wgu = rnd(X, 2 * F, E, dtype=torch.bfloat16, seed=1, scale=0.3)
+    wd = rnd(X, E, F, dtype=torch.bfloat16, seed=2, scale=0.3)
+    counts, offsets = torch.empty(X, dtype=torch.int32, device=DEV), torch.empty(X + 1, dtype=torch.int32, device=DEV)
+    pairs, active = torch.full((T * k,), -7, dtype=torch.int32, device=DEV), torch.full((X,), -1, dtype=torch.int32, device=DEV)
+    n_active, stats = torch.empty(1, dtype=torch.int32, device=DEV), torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    o.moe_align(ids_d, X, counts, offsets, pairs, active, n_active, tile_stats=stats)
+    assert int(stats) == int(((counts.cpu() + 127) // 128).sum())
+    big = int(stats) * 128 * 4 <= T * k * 5
+    assert big == (full <= 8), "the case does not exercise the form it was made for"
+    outs = []
+    for ts in (None, stats):
+        act = torch.zeros(T * k, F, dtype=torch.bfloat16, device=DEV)
+        o.grouped_gemm(h, wgu, act, offsets, pairs, k, o.EPI_SWIGLU, active, n_active, token_rows=T, tile_stats=ts)
+        y = torch.zeros(T * k, E, dtype=torch.float32, device=DEV)
+        o.grouped_gemm(act, wd, y, offsets, pairs, 1, o.EPI_STORE, active, n_active, token_rows=T, tile_stats=ts)
+        outs.append((act, y))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    # against the formula, on the rows of a few tokens
+    for t in (0, 3, T - 1):
+        for j in range(k):
+            e = int(ids[t, j])
+            if e < 0:
+                assert not outs[1][1][t * k + j].any()
+                continue
+            gt = wgu[e, :F].double() @ h[t].double()
+            u = wgu[e, F:].double() @ h[t].double()
+            want = (gt / (1 + torch.exp(-gt))) * u
+            got = outs[1][0][t * k + j].double()
+            assert (got - want).abs().max() <= 1e-2 * want.abs().max()
+            want_y = wd[e].double() @ got
+            assert (outs[1][1][t * k + j].double() - want_y).abs().max() <= 1e-4 * want_y.abs().max()
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 8, 64), (3, 16, 96), (8, 256, 3072), (17, 24, 100), (70, 40, 72), (2048, 256, 3072), (5, 13, 30)])
 def test_gemm_f32_matrix_cores(M, N, K):
     """The router's product: true float32 on the float32 matrix instruction; a row's bits do not depend on the batch."""
