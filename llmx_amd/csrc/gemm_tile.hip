@@ -40,6 +40,35 @@ __device__ __forceinline__ void load_to_lds(const void* base, uint32_t offset, v
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(at), "v"(offset), "s"(base) : "memory", "m0");
 }
 
+// Four neighbouring features of one output row (n a multiple of 4): one 16-byte (float) or 8-byte (bfloat16) access
+// when the row allows it, element by element at a ragged edge.  ADD: the values join what the row holds.
+template <bool ADD, typename TC>
+__device__ __forceinline__ void store_quad(TC* crow, int n, int N, bool rows_aligned, const float (&v)[4]) {
+    if (rows_aligned && n + 3 < N) {
+        if constexpr (std::is_same<TC, float>::value) {
+            f32x4_t x = {v[0], v[1], v[2], v[3]};
+            if (ADD) {
+                const f32x4_t old = *reinterpret_cast<const f32x4_t*>(crow + n);
+                x = f32x4_t{old[0] + x[0], old[1] + x[1], old[2] + x[2], old[3] + x[3]};
+            }
+            *reinterpret_cast<f32x4_t*>(crow + n) = x;
+        } else {
+            typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+            const u32x2_t x = {(uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16),
+                               (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16)};
+            *reinterpret_cast<u32x2_t*>(crow + n) = x;
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (n + i >= N) continue;
+        float x = v[i];
+        if (ADD) x = ld(crow + n + i) + x;
+        st(crow + n + i, x);
+    }
+}
+
 struct TileArgs {
     const bf16_t* A;
     const bf16_t* W;
@@ -380,6 +409,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
 
     // acc[f][t][i]: feature (tile f) 4*(lane/16) + i, row 32*wm + 16*t + lane%16
     const int fq = 4 * (lane >> 4);
+    const bool rows_aligned = g.ldc % 4 == 0 && ((uintptr_t)g.C & 15) == 0;   // a lane's four features make one access
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
         const int rc = rows_c[BM / 2 * wm + 16 * t + lr];
@@ -387,25 +417,21 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         TC* crow = (TC*)g.C + (size_t)rc * g.ldc;
         if (EPI == TL_SWIGLU) {
 #pragma unroll
-            for (int f = 0; f < 2; ++f)
+            for (int f = 0; f < 2; ++f) {
+                float v[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const int n = n0 + 32 * wn + 16 * f + fq + i;
-                    if (n >= g.N) continue;
                     const float gt = acc[f][t][i], u = acc[f + 2][t][i];
-                    st(crow + n, (gt / (1.0f + expf(-gt))) * u);
+                    v[i] = (gt / (1.0f + expf(-gt))) * u;
                 }
+                store_quad<false>(crow, n0 + 32 * wn + 16 * f + fq, g.N, rows_aligned, v);
+            }
         } else {
 #pragma unroll
-            for (int f = 0; f < 4; ++f)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int n = n0 + 64 * wn + 16 * f + fq + i;
-                    if (n >= g.N) continue;
-                    float x = acc[f][t][i];
-                    if (EPI == TL_ADD) x = ld(crow + n) + x;
-                    st(crow + n, x);
-                }
+            for (int f = 0; f < 4; ++f) {
+                const float v[4] = {acc[f][t][0], acc[f][t][1], acc[f][t][2], acc[f][t][3]};
+                store_quad<EPI == TL_ADD>(crow, n0 + 64 * wn + 16 * f + fq, g.N, rows_aligned, v);
+            }
         }
     }
 }
@@ -637,6 +663,7 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
 
     // acc[f][q][i]: feature (tile f) 4*(lane/16) + i, row 64*wm + 16*q + lane%16
     const int fq = 4 * (lane >> 4);
+    const bool rows_aligned = g.ldc % 4 == 0 && ((uintptr_t)g.C & 15) == 0;   // a lane's four features make one access
 #pragma unroll
     for (int q = 0; q < TT; ++q) {
         const int rc = rows_c[64 * wm + 16 * q + lr];
@@ -644,25 +671,21 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
         TC* crow = (TC*)g.C + (size_t)rc * g.ldc;
         if (EPI == TL_SWIGLU) {
 #pragma unroll
-            for (int f = 0; f < 2; ++f)
+            for (int f = 0; f < 2; ++f) {
+                float v[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const int n = n0 + 32 * wn + 16 * f + fq + i;
-                    if (n >= g.N) continue;
                     const float gt = acc[f][q][i], u = acc[f + 2][q][i];
-                    st(crow + n, (gt / (1.0f + expf(-gt))) * u);
+                    v[i] = (gt / (1.0f + expf(-gt))) * u;
                 }
+                store_quad<false>(crow, n0 + 32 * wn + 16 * f + fq, g.N, rows_aligned, v);
+            }
         } else {
 #pragma unroll
-            for (int f = 0; f < 4; ++f)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int n = n0 + 64 * wn + 16 * f + fq + i;
-                    if (n >= g.N) continue;
-                    float x = acc[f][q][i];
-                    if (EPI == TL_ADD) x = ld(crow + n) + x;
-                    st(crow + n, x);
-                }
+            for (int f = 0; f < 4; ++f) {
+                const float v[4] = {acc[f][q][0], acc[f][q][1], acc[f][q][2], acc[f][q][3]};
+                store_quad<EPI == TL_ADD>(crow, n0 + 64 * wn + 16 * f + fq, g.N, rows_aligned, v);
+            }
         }
     }
 }
