@@ -737,8 +737,9 @@ static int form_feats(int form, int epi) { return (epi == TL_SWIGLU ? 64 : 128) 
 // tile_stats (grouped, optional): device int [1], the sum over groups of ceil(rows / 128), from the grouping.
 //
 // Which form runs (every form gives an output element the same bits):
-//   dense: the wide form (8 waves, 128 x 256, three tiles deep) where its tiles fill the chip one and a half times,
-//     else 64-row tiles (three workgroups a CU; more, smaller tiles fill the chip better when there are few).
+//   dense: the wide form (8 waves, 128 x 256, three tiles deep) where it has at least 192 tiles for the 256 CUs
+//     (measured on 2,048 rows: 8,192 features 113 against 165 us, 3,072 features 100 against 108 us), else 64-row
+//     tiles (three workgroups a CU; more, smaller tiles fill the chip better when there are few).
 //   grouped with tile_stats: both a 128-row form (wide for long K, 4 waves for short K) and the 64-row form are
 //     launched; on the device the one that fits the groups' rows works and the other leaves at once.
 extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
@@ -765,7 +766,7 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
         rc = launch(FORM_BOUNDED, max_tiles);
     } else if (!grouped) {
         const long wide_tiles = (long)((M + WD_BM - 1) / WD_BM) * ((N + form_feats(FORM_WIDE, epi) - 1) / form_feats(FORM_WIDE, epi));
-        rc = launch(wide_tiles >= 384 ? FORM_WIDE : FORM_64, 0);
+        rc = launch(wide_tiles >= 192 ? FORM_WIDE : FORM_64, 0);
     } else if (tile_stats) {
         // 128-row tiles: each group adds at most one partial tile
         const int big_tiles = (n_groups < M ? n_groups : M) + M / 128;
