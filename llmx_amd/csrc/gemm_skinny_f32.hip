@@ -99,8 +99,8 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
 // operands' roles, the steps' order and the waves' order are those of the kernel above: the same bits.
 template <int KS>
 __global__ void __launch_bounds__(64 * KS) gemm_rows_f32_kernel(SkinnyF32Args g) {
-    constexpr int NS = 4, MT = 4;
-    __shared__ float red[KS > 1 ? KS : 1][NS * MT][256];
+    constexpr int NS = 4, MT = 4, HALF = NS * MT / 2;
+    __shared__ float red[KS > 1 ? KS : 1][HALF][256];   // half of the tiles at a time: 64 KB at 8 waves, so two workgroups share a CU
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 15, kg = lane >> 4;
     const int n0 = blockIdx.x * 16 * NS;
@@ -150,39 +150,50 @@ __global__ void __launch_bounds__(64 * KS) gemm_rows_f32_kernel(SkinnyF32Args g)
 #pragma unroll
                     for (int t = 0; t < MT; ++t) acc[ns][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[u][ns][i], af[u][t][i], acc[ns][t], 0, 0, 0);
     }
-    if (KS > 1) {
+    // the waves' sums added in wave order, the first 8 tiles of the workgroup's 16 and then the other 8; wave q takes the
+    // tiles q, q + KS, ... of a half
 #pragma unroll
-        for (int ns = 0; ns < NS; ++ns)
-#pragma unroll
-            for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4_t*>(&red[wave][ns * MT + t][lane * 4]) = acc[ns][t];
-        __syncthreads();
-    }
-    // the waves' sums added in wave order; wave q takes the tiles q, q + KS, ... of the workgroup's 16
-    for (int tile = wave; tile < NS * MT; tile += KS) {
-        const int ns = tile / MT, t = tile % MT;
-        f32x4_t v = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int half = 0; half < 2; ++half) {
         if (KS > 1) {
-            v = *reinterpret_cast<f32x4_t*>(&red[0][tile][lane * 4]);
 #pragma unroll
-            for (int w = 1; w < KS; ++w) {
-                const f32x4_t o = *reinterpret_cast<f32x4_t*>(&red[w][tile][lane * 4]);
-                v = f32x4_t{v[0] + o[0], v[1] + o[1], v[2] + o[2], v[3] + o[3]};
+            for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    if ((ns * MT + t) / HALF == half) *reinterpret_cast<f32x4_t*>(&red[wave][(ns * MT + t) % HALF][lane * 4]) = acc[ns][t];
+            __syncthreads();
+        }
+        for (int slot = wave; slot < HALF; slot += KS) {
+            const int tile = half * HALF + slot;
+            const int ns = tile / MT, t = tile % MT;
+            f32x4_t v = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            if (KS > 1) {
+                v = *reinterpret_cast<f32x4_t*>(&red[0][slot][lane * 4]);
+#pragma unroll
+                for (int w = 1; w < KS; ++w) {
+                    const f32x4_t o = *reinterpret_cast<f32x4_t*>(&red[w][slot][lane * 4]);
+                    v = f32x4_t{v[0] + o[0], v[1] + o[1], v[2] + o[2], v[3] + o[3]};
+                }
+            } else {
+#pragma unroll
+                for (int a = 0; a < NS; ++a)
+#pragma unroll
+                    for (int b = 0; b < MT; ++b)
+                        if (a == ns && b == t) v = acc[a][b];
             }
-        } else {
+            const int m = m0 + t * 16 + r;
+            if (m >= g.M) continue;
+            float* c = C + (size_t)m * g.ldc + n0 + 16 * ns + 4 * kg;
+            if (!g.add && g.ldc % 4 == 0 && n0 + 16 * ns + 4 * kg + 3 < g.N && ((uintptr_t)C & 15) == 0) {
+                *reinterpret_cast<f32x4_t*>(c) = v;     // a lane's four neighbouring features in one access
+                continue;
+            }
 #pragma unroll
-            for (int a = 0; a < NS; ++a)
-#pragma unroll
-                for (int b = 0; b < MT; ++b)
-                    if (a == ns && b == t) v = acc[a][b];
+            for (int i = 0; i < 4; ++i) {
+                if (n0 + 16 * ns + 4 * kg + i >= g.N) continue;
+                c[i] = g.add ? c[i] + v[i] : v[i];
+            }
         }
-        const int m = m0 + t * 16 + r;
-        if (m >= g.M) continue;
-        float* c = C + (size_t)m * g.ldc + n0 + 16 * ns + 4 * kg;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if (n0 + 16 * ns + 4 * kg + i >= g.N) continue;
-            c[i] = g.add ? c[i] + v[i] : v[i];
-        }
+        if (KS > 1) __syncthreads();
     }
 }
 
