@@ -445,6 +445,14 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
 #define WD_BM 128
 #define WD_BN 256
 #define WD_STAGES 3
+// The order within half a tile: an operand read after every two multiplications, so the reads are early and spread out.
+#define WD_INTERLEAVE()                                      \
+    do {                                                     \
+        _Pragma("unroll") for (int sg = 0; sg < 8; ++sg) {   \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0); \
+        }                                                    \
+    } while (0)
 template <int EPI, typename TC, bool GROUPED, bool SPLIT>
 __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
     __shared__ __attribute__((aligned(1024))) bf16_t As[WD_STAGES * WD_BM * TL_BK];
@@ -624,6 +632,7 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
         for (; t < stop; ++t) {
             read_half(stage, 32, wf_b, af_b);
             multiply_half(wf_a, af_a);
+            WD_INTERLEAVE();
             const int next = stage == 2 ? 0 : stage + 1;
             // this wave's operand reads of tile t are done, and its part of tile t+1 has arrived (tile t+2's may be out)
             if (t + 2 < n_tiles) __builtin_amdgcn_s_waitcnt(0x0070 | LOADS);
@@ -632,6 +641,7 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
             if (t + 3 < n_tiles) issue(t + 3, stage);
             read_half(next, 0, wf_a, af_a);
             multiply_half(wf_b, af_b);
+            WD_INTERLEAVE();
             stage = next;
         }
         if (SPLIT && t == run_end && t < n_tiles) {
