@@ -306,20 +306,32 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         auto multiply = [&](int stage) {
             const bf16_t* ws = &Ws[stage * TL_BN * TL_BK];
             const bf16_t* as = &As[stage * BM * TL_BK];
+            // the operands of both halves of the tile are asked for at once; the second half's arrive while the first is multiplied
+            bf16x8_t wf[2][4], af[2][TT];
 #pragma unroll
-            for (int kk = 0; kk < TL_BK; kk += 32) {
-                bf16x8_t wf[4], af[TT];
+            for (int hk = 0; hk < 2; ++hk) {
+                const int kk = 32 * hk;
 #pragma unroll
                 for (int f = 0; f < 4; ++f)
-                    wf[f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&ws[w_rd[f] + 8 * ((kk / 8 + kg) ^ w_swz[f])]));
+                    wf[hk][f] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&ws[w_rd[f] + 8 * ((kk / 8 + kg) ^ w_swz[f])]));
 #pragma unroll
                 for (int q = 0; q < TT; ++q)
-                    af[q] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&as[a_rd[q] + 8 * ((kk / 8 + kg) ^ a_swz[q])]));
+                    af[hk][q] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&as[a_rd[q] + 8 * ((kk / 8 + kg) ^ a_swz[q])]));
+            }
+#pragma unroll
+            for (int hk = 0; hk < 2; ++hk)
 #pragma unroll
                 for (int f = 0; f < 4; ++f)
 #pragma unroll
-                    for (int q = 0; q < TT; ++q) acc[f][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[f], af[q], acc[f][q], 0, 0, 0);
+                    for (int q = 0; q < TT; ++q) acc[f][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[hk][f], af[hk][q], acc[f][q], 0, 0, 0);
+            // order: the first half's reads, then a read of the second half after every multiplication while they last
+            __builtin_amdgcn_sched_group_barrier(0x100, 4 + TT, 0);
+#pragma unroll
+            for (int sg = 0; sg < 4 + TT; ++sg) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             }
+            __builtin_amdgcn_sched_group_barrier(0x008, 8 * TT - (4 + TT), 0);
         };
         issue(0, 0);
 #pragma unroll
