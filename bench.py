@@ -51,12 +51,7 @@ def parse():
     return ap.parse_args()
 
 
-def baseline():
-    with open(os.path.join(ROOT, "BASELINE.json")) as f:
-        return json.load(f)
-
-
-# BASELINE.json configs[2]: the real layer sizes.
+# The real layer sizes: 24 layers of the 62-layer model's widths (the third configuration of the benchmark's list).
 def real_config(layers: int, context: int):
     from llmx_amd import MiniMaxM3Config
     return MiniMaxM3Config(vocab_size=200064, hidden_size=3072, num_hidden_layers=layers, num_attention_heads=48,
@@ -233,7 +228,6 @@ def main():
     from llmx_amd import Engine, RandomInit, ops
     from llmx_amd.engine import StepEntry
 
-    base = baseline()
     full_layers, context = 24, 4096
     context = a.context or context
     layers = a.layers or full_layers
@@ -268,7 +262,7 @@ def main():
         "data": "synthetic: LCG token ids, N(0,0.02) weights generated on the device; context before the timed steps: "
                 + ("random keys and values written to the cache" if a.context_fill == "synthetic" else "prompts run through the model"),
         "config": {
-            "model": "MiniMax-M3 slice (BASELINE configs[2])", "layers": layers, "layers_of_config": full_layers, "layers_full_model": 62,
+            "model": "MiniMax-M3 slice (real layer sizes, configs[2])", "layers": layers, "layers_of_config": full_layers, "layers_full_model": 62,
             "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "rotary_dim": cfg.rotary_dim, "experts": cfg.num_local_experts, "top_k": cfg.num_experts_per_tok,
             "expert_intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "global_batch": a.batch, "seq_len": context,

@@ -1,7 +1,7 @@
 """Logit equality across cuttings on a random-weight slice with the real layer sizes (too large for the test suite).
 
-    python -m llmx_amd.tools.slice_check --dtype float32 --layers 8      # BASELINE configs[3]: about 116 GB of weights
-    python -m llmx_amd.tools.slice_check --dtype bfloat16 --layers 24    # configs[2]
+    python -m llmx_amd.tools.slice_check --dtype float32 --layers 8      # the 8-layer float32 slice: about 116 GB of weights
+    python -m llmx_amd.tools.slice_check --dtype bfloat16 --layers 24    # the 24-layer bfloat16 slice the benchmark runs
 
 Four sequences of 300 to 1,000 seeded random tokens are run (1) each alone and whole, (2) most in one step and the last
 32 tokens one by one, (3) in 64-token portions, (4) mixed, up to four live requests with portions of some beside decoded
