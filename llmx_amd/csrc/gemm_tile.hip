@@ -88,7 +88,7 @@ struct TileArgs {
 };
 
 // Whether the groups' rows fill tiles of 128 rows well enough: the tiles hold at most 1.6 times the rows (measured on
-// the prompt's routing: a 2,048-token step takes 32.3 ms with the bound at 1.25, 30.2 ms at 1.6, 31.2 ms at 2).  The launcher
+// the prompt's routing on one machine: a 2,048-token step takes 30.9 ms with the bound at 1.25, 30.3 ms at 1.6, 30.2 ms at 2).  The launcher
 // cannot know (the counts are on the device), so it launches the form for either case and one of them leaves at once.
 __device__ __forceinline__ bool tile_launch_runs(const TileArgs& g) {
     if (!g.tile_stats) return true;
