@@ -198,6 +198,21 @@ def test_routed_products_choose_their_tiles_on_the_device(T, X, k, E, F, full):
             assert (got - want).abs().max() <= 1e-2 * want.abs().max()
             want_y = wd[e].double() @ got
             assert (outs[1][1][t * k + j].double() - want_y).abs().max() <= 1e-4 * want_y.abs().max()
+    # rows at the tiles' edges have the bits the weight-streaming kernel gives them alone
+    off, lst = offsets.cpu().tolist(), pairs.cpu().tolist()
+    act, y = outs[1]
+    for e in range(X):
+        n = off[e + 1] - off[e]
+        for at in sorted({0, 63, 64, 127, 128, n - 65, n - 1}):
+            if not 0 <= at < n:
+                continue
+            p = lst[off[e] + at]
+            a1 = torch.empty(1, F, dtype=torch.bfloat16, device=DEV)
+            o.gemm(h[p // k:p // k + 1], wgu[e], a1, o.EPI_SWIGLU)
+            assert torch.equal(a1[0], act[p]), f"expert {e}, row {at} of {n}"
+            y1 = torch.empty(1, E, dtype=torch.float32, device=DEV)
+            o.gemm(act[p:p + 1], wd[e], y1)
+            assert torch.equal(y1[0], y[p]), f"expert {e}, row {at} of {n}"
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 8, 64), (3, 16, 96), (8, 256, 3072), (17, 24, 100), (70, 40, 72), (2048, 256, 3072), (5, 13, 30)])
