@@ -298,3 +298,26 @@ def test_real_layer_widths(wide_folder, dtype):
     rows = torch.cat([engine.step([StepEntry("p", tokens[a:b], list(range(b - a)))]).clone() for a, b in cuts]).cpu()
     engine.end_request("p")
     assert torch.equal(rows, whole), f"portions differ from the whole prompt in {dtype}"
+
+
+def test_a_long_portion_takes_the_wide_tiles_and_gives_the_bits_of_short_ones(wide_folder):
+    """800 rows at the real layer widths run the dense products on the wide tiles and the routed ones (6,400 pairs) on
+    tiles chosen on the device; the same prompt in portions that stay below those sizes gives the same logits bit for bit."""
+    from llmx_amd.engine import Engine, StepEntry
+    import random
+    rng = random.Random(11)
+    tokens = [rng.randrange(1000) for _ in range(800)]
+    want_rows = list(range(0, 800, 37)) + [799]
+    engine = Engine.load(wide_folder, dtype="bfloat16", kv_tokens=2048, page_tokens=16, max_requests=2)
+    engine.add_request("w")
+    whole = engine.step([StepEntry("w", tokens, want_rows)]).clone()
+    engine.end_request("w")
+    assert bool(torch.isfinite(whole).all())
+    engine.add_request("p")
+    rows = []
+    for a, b in [(0, 300), (300, 330), (330, 650), (650, 799), (799, 800)]:
+        want = [r - a for r in want_rows if a <= r < b]
+        out = engine.step([StepEntry("p", tokens[a:b], want)])
+        rows.append(out.clone())
+    engine.end_request("p")
+    assert torch.equal(torch.cat(rows), whole)
