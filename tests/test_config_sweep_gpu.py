@@ -4,7 +4,7 @@ The two tiny configurations fix two points of the space of sizes; this file walk
 steps of 16 up to 256, head counts and groups that are no power of two (one KV head, one query head a group, five
 groups), rotation of none, part or all of a head, one expert, an odd number of experts, every pick count, widths
 that are only multiples of two, odd vocabularies, all page sizes.  Each configuration runs whole, with the last 32
-tokens one by one, and in portions of changing size, in both dtypes; the cuttings must agree bit for bit and the
+tokens one by one, in portions of changing size, and as six requests mixed through a pool for four, in both dtypes; the cuttings must agree bit for bit and the
 whole run must agree with the plain implementation within the bounds of test_engine_gpu (the plain implementation
 is given the engine's expert picks, each checked to be one of the best within rounding).  A size that a kernel does
 not take must be refused with an error, never computed wrongly: a refusal would fail here by name.
@@ -85,3 +85,8 @@ def test_a_drawn_configuration(seed, wide, length, dtype):
     cut = engine_tests.run_cut(engine, "p", tokens, helpers.portions(length))
     assert torch.equal(cut, whole), f"{helpers.TINY[name][0]}: portions differ from the whole prompt"
     assert engine.cache.pages_in_use() == 0
+    # six requests through a pool for four, mixed in steps: each must have the bits of its run alone
+    _, prompts, mixed = engine_tests.run_mixed(name, dtype)
+    for i, prompt in enumerate(prompts):
+        assert torch.equal(mixed[i], engine_tests.run_whole(engine, "w", prompt)), \
+            f"{helpers.TINY[name][0]}: request {i} in the mix differs from its run alone"

@@ -122,14 +122,16 @@ def test_first_tokens(setup):
         assert float((got.double() - want).abs().max()) <= tol * float(want.abs().max())
 
 
-def test_mixed_requests_with_page_reuse(setup):
-    """Up to four live requests; portions of some beside decoded tokens of others; the pool is so small that pages
-    freed by finished requests are handed out again."""
+MIXED_LENGTHS = [40, 23, 67, 9, 31, 52]
+MIXED_SEEDS = [1, 2, 3, 4, 5, 6]
+
+
+def run_mixed(name, dtype):
+    """Six requests through a pool for four: up to four live, portions of some beside decoded tokens of others, some left
+    out of a step.  Returns the engine, the prompts and each request's logits [length, vocab] as the steps gave them."""
     from llmx_amd.engine import StepEntry
-    name, dtype, _ = setup
     page = TINY[name][2]
-    lengths = [40, 23, 67, 9, 31, 52]
-    seeds = [1, 2, 3, 4, 5, 6]
+    lengths, seeds = MIXED_LENGTHS, MIXED_SEEDS
     # four live requests of at most 67 tokens: pages for 4 * 72 tokens, far fewer than all six hold together
     engine = watch(make_engine(name, dtype, kv_tokens=4 * (-(-67 // page) * page), max_requests=4), name, dtype)
     toks = [tokens_for(name, n, s) for n, s in zip(lengths, seeds)]
@@ -174,11 +176,18 @@ def test_mixed_requests_with_page_reuse(setup):
     assert engine.cache.pages_in_use() == 0
     total_pages = sum(-(-n // page) for n in lengths)
     assert len(used_pages) < total_pages, "the pool was large enough that no page was used again"
+    return engine, toks, [torch.cat(got[i]) for i in range(len(lengths))]
+
+
+def test_mixed_requests_with_page_reuse(setup):
+    """Up to four live requests; portions of some beside decoded tokens of others; the pool is so small that pages
+    freed by finished requests are handed out again."""
+    name, dtype, _ = setup
+    engine, toks, mixed = run_mixed(name, dtype)
     alone = make_engine(name, dtype)
-    for i, (n, s) in enumerate(zip(lengths, seeds)):
-        mixed = torch.cat(got[i])
-        check_against_plain(name, dtype, n, s, mixed, engine, i)
-        assert torch.equal(mixed, run_whole(alone, "w", toks[i])), f"request {i} in the mix differs from its run alone"
+    for i, (n, s) in enumerate(zip(MIXED_LENGTHS, MIXED_SEEDS)):
+        check_against_plain(name, dtype, n, s, mixed[i], engine, i)
+        assert torch.equal(mixed[i], run_whole(alone, "w", toks[i])), f"request {i} in the mix differs from its run alone"
 
 
 def test_long_decoding(setup):
