@@ -175,3 +175,29 @@ def test_command_line(tmp_path):
     assert abs(float(out["mean NLL"]) - nll) < 2e-5
     bad = subprocess.run([os.path.join(ROOT, "bin", "llmx"), "perplexity", model_folder(name), "7"], capture_output=True, text=True, timeout=120)
     assert bad.returncode == 2 and "at least 2" in bad.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_requests_through_a_small_pool_equal_their_runs_alone(dtype):
+    """Thirty requests of drawn lengths, counts and settings, through pages for about three of them: requests wait for
+    pages, portions of prompts run beside decoded tokens, freed pages are used again.  Logits do not depend on the
+    batch or the pages and every request owns its generator, so each gets the tokens of its run alone, bit for bit,
+    in both dtypes."""
+    import random
+    from llmx_amd import SamplingParams, generate
+    name = "B"
+    rng = random.Random(5)
+    prompts = [tokens_for(name, rng.randrange(1, 90), 200 + i) for i in range(30)]
+    params = []
+    for i in range(30):
+        kind = i % 3
+        params.append(SamplingParams(max_tokens=rng.randrange(1, 20), seed=77 + i, temp=(0.0, 0.8, 1.2)[kind],
+                                     top_k=(0, 0, 12)[kind], top_p=(1.0, 1.0, 0.9)[kind],
+                                     penalty=1.2 if i % 5 == 0 else 1.0, ignore_eos=True))
+    small = engine_for(name, dtype, kv_tokens=3 * 112, max_requests=4)
+    together = generate(small, prompts, params, max_seqs=4, max_step_tokens=48)
+    assert small.cache.pages_in_use() == 0
+    assert [len(t) for t in together] == [p.max_tokens for p in params]
+    roomy = engine_for(name, dtype, kv_tokens=512, max_requests=2)
+    for i, (prompt, sp) in enumerate(zip(prompts, params)):
+        assert generate(roomy, [prompt], sp)[0] == together[i], f"request {i} ({len(prompt)} prompt tokens, {sp})"
