@@ -11,7 +11,8 @@ step, one new token each, logits -> greedy token on the device -> ids read back 
 record's `frac` is its flops over the bf16 peak; beside it `hbm_frac` is the weights it has to read (the experts its
 tokens picked, counted in the warm-up run) over its time against 8 TB/s: few rows an expert make the step a
 weight-streaming one.
-Token ids are a fixed LCG sequence; weights are N(0, 0.02) generated on the device.
+Token ids are a fixed LCG sequence; weights are N(0, 0.02) generated on the device.  The context before the timed
+steps is built by running each request's prompt through the model (`context_fill` gives its rate).
 """
 
 from __future__ import annotations
@@ -45,9 +46,9 @@ def parse():
     ap.add_argument("--no-logits-to-host", action="store_true",
                     help="skip the extra point: the default batch with every step's logits copied to the host")
     ap.add_argument("--only-prefill", action="store_true", help="for profiling: measure the prefill alone and print its record")
-    ap.add_argument("--context-fill", choices=["synthetic", "prefill"], default="synthetic",
-                    help="how the context before the timed steps gets into the cache: random keys and values written "
-                         "directly, or prompts run through the model")
+    ap.add_argument("--context-fill", choices=["prefill", "synthetic"], default="prefill",
+                    help="how the context before the timed steps gets into the cache: prompts run through the model in "
+                         "portions of 2,048 tokens, or (for quick profiling runs) random keys and values written directly")
     return ap.parse_args()
 
 
