@@ -19,6 +19,81 @@ __device__ __forceinline__ float sum_slices(const float* __restrict__ p, int sli
     return x;
 }
 
+// A row of at most 256 experts in one wave's registers (slot i of a lane: expert lane + 64 i): the logits, from the row
+// or from `slices` partial sums added in slice order (then also written to the row).  All loads are asked for before
+// the first is used, also those of lanes and slices that do not count (their addresses are clamped).
+__device__ __forceinline__ void load_row_256(float* __restrict__ row, const float* __restrict__ parts, int slices, long slice_stride,
+                                             const float* __restrict__ bias, int n_experts, int lane, float (&x)[4], float (&bias_v)[4]) {
+    float v[4][ROUTE_MAX_SLICES];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = min(lane + 64 * i, n_experts - 1);
+        if (parts) {
+#pragma unroll
+            for (int sl = 0; sl < ROUTE_MAX_SLICES; ++sl) v[i][sl] = parts[(size_t)min(sl, slices - 1) * slice_stride + e];
+        } else {
+            v[i][0] = row[e];
+        }
+        bias_v[i] = bias ? bias[e] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[i] = v[i][0];
+        if (parts) {
+#pragma unroll
+            for (int sl = 1; sl < ROUTE_MAX_SLICES; ++sl)
+                if (sl < slices) x[i] += v[i][sl];
+            if (lane + 64 * i < n_experts) row[lane + 64 * i] = x[i];
+        }
+    }
+}
+
+// Sigmoid scores and the k <= 64 picks of such a row: lane j < k ends with pick j's id and weight (-1 and 0 for a row with
+// a non-finite key).  A pick is the largest key not yet taken, the lowest id among equal keys: the wave's maximum of
+// the keys (exact, so its order does not matter), then the first slot and in it the first lane that holds it.  The
+// formulas and the order of the picks' sum are those of route_topk_kernel's general path.
+__device__ __forceinline__ void route_row_256(const float (&x)[4], const float (&bias_v)[4], bool has_bias, int n_experts, int k, int normalize,
+                                              float scale, int lane, int& pick_id, float& pick_weight) {
+    float s[4], b[4];
+    int finite = 1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        s[i] = 0.0f;
+        b[i] = -INFINITY;   // no expert, or taken: below every finite key
+        if (lane + 64 * i < n_experts) {
+            s[i] = 1.0f / (1.0f + expf(-x[i]));
+            b[i] = has_bias ? s[i] + bias_v[i] : s[i];
+            if (!isfinite(b[i])) finite = 0;
+        }
+    }
+    pick_id = -1;
+    pick_weight = 0.0f;
+    if (!__all(finite)) return;
+    float mine = 0.0f;
+    for (int j = 0; j < k; ++j) {
+        const float best = wave_max(fmaxf(fmaxf(b[0], b[1]), fmaxf(b[2], b[3])));
+        const unsigned long long m0 = __ballot(b[0] == best), m1 = __ballot(b[1] == best), m2 = __ballot(b[2] == best),
+                                 m3 = __ballot(b[3] == best);
+        const int slot = m0 ? 0 : m1 ? 1 : m2 ? 2 : 3;
+        const unsigned long long m = m0 ? m0 : m1 ? m1 : m2 ? m2 : m3;
+        const int ln = __builtin_amdgcn_readfirstlane(__ffsll((long long)m) - 1);
+        const float picked = slot == 0 ? s[0] : slot == 1 ? s[1] : slot == 2 ? s[2] : s[3];
+        const float score = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(picked), ln));
+        if (lane == ln) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (i == slot) b[i] = -INFINITY;
+        }
+        if (lane == j) {
+            mine = score;
+            pick_id = ln + 64 * slot;
+        }
+    }
+    float total = 0.0f;
+    for (int j = 0; j < k; ++j) total += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mine), j));
+    pick_weight = (normalize ? mine / total : mine) * scale;
+}
+
 // One wave per row.  score s_e = sigmoid(z_e) (or softmax over the row); the pick key is b_e = s_e + bias_e; k times
 // the largest key not yet taken is picked, the lowest id on ties; the weight is the unbiased s_e, divided by the
 // picks' sum (added in pick order) when `normalize`, then times `scale`.  A row with a non-finite key gets ids -1 and
@@ -34,6 +109,17 @@ __global__ void __launch_bounds__(64) route_topk_kernel(float* __restrict__ z, c
     __shared__ float chosen[ROUTE_MAX_K];
     const int r = blockIdx.x, lane = threadIdx.x;
     float* row = z + (size_t)r * n_experts;
+    if (score == SCORE_SIGMOID && n_experts <= 256 && k <= 64) {   // the row fits the wave's registers
+        float x[4], bias_v[4], weight;
+        int id;
+        load_row_256(row, parts ? parts + (size_t)r * n_experts : nullptr, slices, slice_stride, bias, n_experts, lane, x, bias_v);
+        route_row_256(x, bias_v, bias != nullptr, n_experts, k, normalize, scale, lane, id, weight);
+        if (lane < k) {
+            ids[(size_t)r * k + lane] = id;
+            weights[(size_t)r * k + lane] = weight;
+        }
+        return;
+    }
     if (parts) {
         for (int e = lane; e < n_experts; e += 64) {   // the thread reads back only what it wrote
             row[e] = sum_slices(parts + (size_t)r * n_experts + e, slices, slice_stride);
@@ -348,8 +434,8 @@ extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* c
 
 // ---------------------------------------------------------------------------
 // A decode step's routing in one launch: top-k of every row (one wave a row, values in registers: at most 256 experts,
-// at most 64 picks), then the pairs grouped by expert as moe_align_small_kernel does.  Same formulas and the same
-// orders as route_topk_kernel, so the picks and weights are the same bits.
+// at most 64 picks), then the pairs grouped by expert as moe_align_small_kernel does.  The rows go through the same
+// functions as in route_topk_kernel, so the picks and weights are the same bits.
 __global__ void __launch_bounds__(1024) route_topk_align_kernel(float* __restrict__ z, const float* __restrict__ parts, int slices,
                                                                long slice_stride, const float* __restrict__ bias,
                                                                int* __restrict__ ids, float* __restrict__ weights, int rows, int n_experts,
@@ -361,71 +447,15 @@ __global__ void __launch_bounds__(1024) route_topk_align_kernel(float* __restric
     __shared__ int offs[1024];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     for (int r = wave; r < rows; r += 16) {
-        float* row = z + (size_t)r * n_experts;
-        float s[4], b[4];
-        bool taken[4];
-        int finite = 1;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int e = lane + 64 * i;
-            s[i] = 0.0f;
-            b[i] = -INFINITY;
-            taken[i] = true;
-            if (e < n_experts) {
-                float x;
-                if (parts) {   // the slices' loads are in flight together; they are added in slice order
-                    x = sum_slices(parts + (size_t)r * n_experts + e, slices, slice_stride);
-                    row[e] = x;
-                } else {
-                    x = row[e];
-                }
-                s[i] = 1.0f / (1.0f + expf(-x));
-                b[i] = bias ? s[i] + bias[e] : s[i];
-                taken[i] = false;
-                if (!isfinite(b[i])) finite = 0;
-            }
-        }
-        finite = __all(finite);
-        if (!finite) {
-            if (lane < k) {
-                ids[(size_t)r * k + lane] = -1;
-                weights[(size_t)r * k + lane] = 0.0f;
-                pair_expert[r * k + lane] = -1;
-            }
-            continue;
-        }
-        float mine = 0.0f;
-        int mine_id = -1;
-        for (int j = 0; j < k; ++j) {
-            float best = -INFINITY;
-            int at = 0x7fffffff;
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (!taken[i] && b[i] > best) {
-                    best = b[i];
-                    at = lane + 64 * i;
-                }
-            wave_best(best, at);
-            at = __builtin_amdgcn_readfirstlane(at);
-            const int slot = at >> 6;
-            const float picked = slot == 0 ? s[0] : slot == 1 ? s[1] : slot == 2 ? s[2] : s[3];
-            const float score = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(picked), at & 63));
-            if (lane == (at & 63)) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (i == slot) taken[i] = true;
-            }
-            if (lane == j) {
-                mine = score;
-                mine_id = at;
-            }
-        }
-        float total = 0.0f;
-        for (int j = 0; j < k; ++j) total += __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mine), j));
+        float x[4], bias_v[4], weight;
+        int id;
+        load_row_256(z + (size_t)r * n_experts, parts ? parts + (size_t)r * n_experts : nullptr, slices, slice_stride, bias, n_experts, lane, x,
+                     bias_v);
+        route_row_256(x, bias_v, bias != nullptr, n_experts, k, normalize, scale, lane, id, weight);
         if (lane < k) {
-            ids[(size_t)r * k + lane] = mine_id;
-            weights[(size_t)r * k + lane] = (normalize ? mine / total : mine) * scale;
-            pair_expert[r * k + lane] = mine_id;
+            ids[(size_t)r * k + lane] = id;
+            weights[(size_t)r * k + lane] = weight;
+            pair_expert[r * k + lane] = id;
         }
     }
     __syncthreads();
