@@ -92,6 +92,128 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
     }
 }
 
+// The form for many rows (prompt portions): one block norms and rotates a row's q, another its k and writes k and v.
+// A thread keeps its share of the projection (elements threadIdx.x + 256 j, at most KEPT of them) in registers from
+// the one pass that asks for everything the block reads (values, norm weights, the position's cosines and sines);
+// the rotation's partners come from a copy of the normed row in LDS, and all results are formed before the first is
+// stored.
+// The sum of squares takes the elements in the order of strided_squares and every result is formed by the expressions
+// of normed_rotated, so a row gets the bits of the kernel above; no element is divided to find its head and dim.
+template <int KEPT>
+struct KeptRow {
+    float x[KEPT];   // after norm_rotate_kept: the normed and rotated values
+};
+
+// (head, dim) of element threadIdx.x + 256 j, stepped from j to j + 1
+struct HeadDim {
+    int h, d, step_h, step_d, D;
+    __device__ __forceinline__ HeadDim(int tid, int D_) : h(tid / D_), d(tid % D_), step_h(256 / D_), step_d(256 % D_), D(D_) {}
+    __device__ __forceinline__ void next() {
+        h += step_h;
+        d += step_d;
+        if (d >= D) {
+            d -= D;
+            ++h;
+        }
+    }
+};
+
+template <int KEPT>
+__device__ __forceinline__ void norm_rotate_kept(const float* __restrict__ src, const float* __restrict__ weight, int width,
+                                                 const float* __restrict__ cs, int D, int rotary_dim, int norm_mode, float eps,
+                                                 float* __restrict__ row_lds, float* __restrict__ scratch, KeptRow<KEPT>& out) {
+    const int tid = threadIdx.x, half = rotary_dim / 2;
+    const bool normed = norm_mode != QKNORM_NONE;
+    float* cs_lds = row_lds + width;
+    float w[KEPT];
+#pragma unroll
+    for (int j = 0; j < KEPT; ++j) {
+        const bool in = tid + 256 * j < width;
+        out.x[j] = in ? src[tid + 256 * j] : 0.0f;
+        w[j] = (in && normed) ? weight[tid + 256 * j] : 0.0f;
+    }
+    for (int i = tid; i < rotary_dim; i += 256) cs_lds[i] = cs[i];
+    float r = 1.0f;
+    if (norm_mode == QKNORM_PROJECTION) {
+        float sq = 0.0f;
+#pragma unroll
+        for (int j = 0; j < KEPT; ++j) sq = fmaf(out.x[j], out.x[j], sq);   // an element past the end adds fmaf(0, 0, s) = s
+        r = 1.0f / sqrtf(block_sum<4>(sq, scratch) / (float)width + eps);
+    }
+    // the normed values go to LDS: an element's partner in the rotation is another thread's
+#pragma unroll
+    for (int j = 0; j < KEPT; ++j) {
+        if (normed) out.x[j] = out.x[j] * (r * w[j]);
+        if (tid + 256 * j < width) row_lds[tid + 256 * j] = out.x[j];
+    }
+    __syncthreads();
+    HeadDim at(tid, D);
+#pragma unroll
+    for (int j = 0; j < KEPT; ++j) {
+        const int i = tid + 256 * j;
+        if (i < width && at.d < rotary_dim) {
+            const bool low = at.d < half;
+            const int pair = low ? at.d : at.d - half;
+            const float y = row_lds[low ? i + half : i - half];
+            const float c = cs_lds[pair], sn = cs_lds[half + pair];
+            out.x[j] = low ? fmaf(-y, sn, out.x[j] * c) : fmaf(y, sn, out.x[j] * c);
+        }
+        at.next();
+    }
+}
+
+template <typename TQ, typename TKV, int KQ, int KK>
+__global__ void __launch_bounds__(256) qknorm_rope_kvwrite_rows_kernel(QkvArgs a) {
+    extern __shared__ float row_lds[];
+    __shared__ float scratch[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int D = a.head_dim;
+    const int qw = a.n_heads * D, kw = a.n_kv_heads * D;
+    const float* row = a.qkv + (size_t)t * (qw + 2 * kw);
+    const int p = a.pos[t];
+    const float* cs = a.cos_sin + (size_t)p * a.rotary_dim;
+    if (blockIdx.y == 0) {
+        KeptRow<KQ> q;
+        norm_rotate_kept<KQ>(row, a.q_weight, qw, cs, D, a.rotary_dim, a.norm_mode, a.eps, row_lds, scratch, q);
+        TQ* q_out = (TQ*)a.q_out + (size_t)t * qw;
+#pragma unroll
+        for (int j = 0; j < KQ; ++j)
+            if (tid + 256 * j < qw) st(q_out + tid + 256 * j, q.x[j]);
+        return;
+    }
+    if (!a.write_kv) return;
+    const int page = a.tables[(size_t)a.row_entry[t] * a.max_blocks + p / a.page_tokens];
+    const int slot = p % a.page_tokens;
+    float vals[KK];
+#pragma unroll
+    for (int j = 0; j < KK; ++j) vals[j] = tid + 256 * j < kw ? row[qw + kw + tid + 256 * j] : 0.0f;
+    KeptRow<KK> k;
+    norm_rotate_kept<KK>(row + qw, a.k_weight, kw, cs, D, a.rotary_dim, a.norm_mode, a.eps, row_lds, scratch, k);
+    TKV* kc = (TKV*)a.k_cache;
+    TKV* vc = (TKV*)a.v_cache;
+    HeadDim at(tid, D);
+#pragma unroll
+    for (int j = 0; j < KK; ++j) {
+        if (tid + 256 * j < kw) {
+            const size_t head_at = (size_t)page * a.n_kv_heads + at.h;
+            st(kc + (head_at * a.page_tokens + slot) * D + at.d, k.x[j]);
+            st(vc + (head_at * D + at.d) * a.page_tokens + slot, vals[j]);
+        }
+        at.next();
+    }
+}
+
+template <typename TQ, typename TKV>
+static void launch_qkv_rows(const QkvArgs& a, int rows, int qw, int kw, hipStream_t stream) {
+    const dim3 grid(rows, 2);
+    const size_t lds = sizeof(float) * (size_t)((qw > kw ? qw : kw) + a.rotary_dim);
+    const bool q16 = qw <= 16 * 256, k8 = kw <= 8 * 256;
+    if (q16 && k8) hipLaunchKernelGGL((qknorm_rope_kvwrite_rows_kernel<TQ, TKV, 16, 8>), grid, dim3(256), lds, stream, a);
+    else if (q16) hipLaunchKernelGGL((qknorm_rope_kvwrite_rows_kernel<TQ, TKV, 16, 32>), grid, dim3(256), lds, stream, a);
+    else if (k8) hipLaunchKernelGGL((qknorm_rope_kvwrite_rows_kernel<TQ, TKV, 32, 8>), grid, dim3(256), lds, stream, a);
+    else hipLaunchKernelGGL((qknorm_rope_kvwrite_rows_kernel<TQ, TKV, 32, 32>), grid, dim3(256), lds, stream, a);
+}
+
 extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight, const float* k_weight, const float* cos_sin, const int* pos,
                                         const int* row_entry, const int* tables, void* q_out, void* k_cache, void* v_cache, int dtype,
                                         float eps, int rows, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int norm_mode,
@@ -109,6 +231,11 @@ extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight,
     }
     QkvArgs a{qkv, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
               n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, q_slices, k_slices};
+    if (rows > 256 && qw <= 32 * 256 && kw <= 32 * 256 && head_dim <= 256) {   // rows kept in registers
+        if (dtype == LLMX_F32) launch_qkv_rows<float, float>(a, rows, qw, kw, stream);
+        else launch_qkv_rows<bf16_t, bf16_t>(a, rows, qw, kw, stream);
+        return LLMX_CHECK_LAUNCH();
+    }
     const dim3 grid(rows, q_slices + k_slices);
     if (dtype == LLMX_F32)
         hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<float, float>), grid, dim3(256), 0, stream, a);

@@ -332,6 +332,62 @@ def test_routed_products(T, X, k, E, F, dtype):
 
 
 # ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,D,R,norm", [(48, 8, 128, 64, True), (6, 2, 80, 80, True), (20, 20, 160, 34, True), (5, 1, 48, 0, True),
+                                              (30, 30, 256, 256, False), (12, 3, 16, 8, True)])
+def test_qknorm_rope_kvwrite_of_many_rows_keeps_the_bits_of_few_rows(Hq, Hkv, D, R, norm, dtype):
+    """More than 256 rows in one launch take the form that keeps a row in registers; it must give every row the bits of
+    the launches of few rows (q, the key pages and the transposed value pages), and agree with the plain formulas
+    (norm over the whole projection, NeoX halves over the first R dims).  The shapes reach all four register budgets
+    of the form: projections up to 4,096 and above, key widths up to 2,048 and above."""
+    o = ops()
+    rows, page, eps = 300, 16, 1e-5
+    qw, kw = Hq * D, Hkv * D
+    qkv = rnd(rows, qw + 2 * kw, scale=1.5, seed=D)
+    wq, wk = 1.0 + 0.2 * rnd(qw, seed=1), 1.0 + 0.2 * rnd(kw, seed=2)
+    # two requests: rows 0..179 at positions 7.., rows 180..299 at positions 0..
+    pos = torch.tensor([7 + i for i in range(180)] + list(range(120)), dtype=torch.int32, device=DEV)
+    ent = torch.tensor([0] * 180 + [1] * 120, dtype=torch.int32, device=DEV)
+    cos, sin = plain_model.rope_tables(list(range(256)), R, 1e4) if R else (torch.zeros(256, 0), torch.zeros(256, 0))
+    cos_sin = torch.cat([cos, sin], dim=1).contiguous().to(DEV)
+    blocks = 12
+    perm = torch.randperm(2 * blocks, generator=torch.Generator().manual_seed(3)).to(torch.int32)
+    tables = perm.reshape(2, blocks).to(DEV)
+    mode = o.QKNORM_PROJECTION if norm else o.QKNORM_NONE
+
+    def run(chunks):
+        q = torch.zeros(rows, qw, dtype=dtype, device=DEV)
+        kc = torch.zeros(2 * blocks, Hkv, page, D, dtype=dtype, device=DEV)
+        vc = torch.zeros(2 * blocks, Hkv, D, page, dtype=dtype, device=DEV)
+        for a, b in chunks:
+            o.qknorm_rope_kvwrite(qkv[a:b], wq if norm else None, wk if norm else None, cos_sin, pos[a:b], ent[a:b], tables, q[a:b], kc, vc,
+                                  eps, Hq, Hkv, D, R, mode)
+        return q, kc, vc
+
+    many = run([(0, rows)])
+    few = run([(0, 100), (100, 117), (117, 300 - 1), (299, 300)])
+    for got, want, what in zip(many, few, ("q", "key pages", "value pages")):
+        assert torch.equal(got, want), f"{what} differ between one launch of {rows} rows and launches of few rows"
+    # the plain formulas, on q and on what the pages hold
+    x = qkv.double().cpu()
+    qp, kp, vp = x[:, :qw], x[:, qw:qw + kw], x[:, qw + kw:]
+    if norm:
+        qp, kp = plain_model.rms_norm(qp, wq.double().cpu(), eps), plain_model.rms_norm(kp, wk.double().cpu(), eps)
+    cs_rows = cos_sin.double().cpu()[pos.long().cpu()]
+    half = R // 2
+    qp = plain_model.apply_partial_rope(qp.reshape(rows, Hq, D), cs_rows[:, :half], cs_rows[:, half:], R)
+    kp = plain_model.apply_partial_rope(kp.reshape(rows, Hkv, D), cs_rows[:, :half], cs_rows[:, half:], R)
+    tol = 3e-6 if dtype == torch.float32 else 2.0 ** -8
+    assert (many[0].double().cpu().reshape(rows, Hq, D) - qp).abs().max() <= tol * qp.abs().max()
+    tab = tables.cpu()
+    for t in (0, 9, 179, 180, 299):
+        e, pp = int(ent[t]), int(pos[t])
+        pg = int(tab[e, pp // page])
+        assert (many[1][pg, :, pp % page, :].double().cpu() - kp[t]).abs().max() <= tol * kp.abs().max()
+        assert (many[2][pg, :, :, pp % page].double().cpu() - vp[t].reshape(Hkv, D)).abs().max() <= tol * vp.abs().max()
+
+
+# ---------------------------------------------------------------------------
 def attention_case(T_lens, Hq, Hkv, D, R, page, dtype, window=0, shuffle_seed=0, norm=True, planned=True, second_single=False):
     """Runs qknorm_rope_kvwrite + paged_attention for sequences of the given lengths, each cut into two steps, with
     shuffled page tables, and returns (got, want) attention outputs in float64."""
