@@ -215,7 +215,8 @@ def test_routed_products_choose_their_tiles_on_the_device(T, X, k, E, F, full):
             assert torch.equal(y1[0], y[p]), f"expert {e}, row {at} of {n}"
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 8, 64), (3, 16, 96), (8, 256, 3072), (17, 24, 100), (70, 40, 72), (2048, 256, 3072), (5, 13, 30)])
+@pytest.mark.parametrize("M,N,K", [(1, 8, 64), (3, 16, 96), (8, 256, 3072), (17, 24, 100), (70, 40, 72), (2048, 256, 3072), (5, 13, 30),
+                                   (130, 100, 200), (97, 64, 1000), (1000, 72, 520), (65, 640, 4096)])
 def test_gemm_f32_matrix_cores(M, N, K):
     """The router's product: true float32 on the float32 matrix instruction; a row's bits do not depend on the batch."""
     o = ops()
@@ -674,7 +675,8 @@ def test_fused_route_and_align_equals_the_two_kernels(T, X, k):
             assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("M,N,K,k", [(1, 256, 3072, 8), (8, 256, 3072, 8), (64, 256, 3072, 8), (300, 256, 3072, 8), (5, 64, 1024, 3)])
+@pytest.mark.parametrize("M,N,K,k", [(1, 256, 3072, 8), (8, 256, 3072, 8), (64, 256, 3072, 8), (300, 256, 3072, 8), (5, 64, 1024, 3),
+                                     (130, 64, 1024, 3), (777, 1024, 1024, 5), (100, 512, 776, 2)])
 def test_router_logits_as_partial_sums(M, N, K, k):
     """The router's product spread over more workgroups: K's runs are written as partial sums and the routing kernels add
     them in run order.  The logits they leave are that sum exactly, the picks are those of routing the summed logits, and
