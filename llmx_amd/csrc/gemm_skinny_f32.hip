@@ -197,6 +197,128 @@ __global__ void __launch_bounds__(64 * KS) gemm_rows_f32_kernel(SkinnyF32Args g)
     }
 }
 
+// Many rows and at least 128 features, operands staged through LDS: a workgroup of 8 waves takes 64 rows, 256
+// features and one of K's slices; the slice's steps come in chunks of two (a row's 128 bytes, read whole by 8
+// neighbouring lanes), the next chunk travelling while this one is multiplied.  A wave holds 64 features x 32 rows (two
+// waves a SIMD: one's sums and operand reads hide behind the other's multiplications) and
+// walks the slice's steps in order; where one of the `ks` wave ranges of the kernels above ends, its sum joins the
+// ranges before it, in order: the same bits (the steps that those kernels mask add products of zeros and are left out).
+#define RL_ROWS 64
+#define RL_FEATS 256
+#define RL_PITCH 36   // floats a staged row takes: 32 of k and 4 of padding, so 8 rows' 16-byte pieces fall into different banks
+__global__ void __launch_bounds__(512) gemm_rows_f32_lds_kernel(SkinnyF32Args g, int ks) {
+    __shared__ __attribute__((aligned(16))) float Ws[2][RL_FEATS * RL_PITCH];
+    __shared__ __attribute__((aligned(16))) float As[2][RL_ROWS * RL_PITCH];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, kg = lane >> 4;
+    const int wn = wave & 3, wm = wave >> 2;   // the wave's 64 features and 32 rows
+    const int n0 = blockIdx.x * RL_FEATS, m0 = blockIdx.y * RL_ROWS;
+    const int K = g.K;
+    const int steps_total = (K + 15) >> 4;
+    const int per_slice = (steps_total + gridDim.z - 1) / gridDim.z;
+    const int slice_begin = blockIdx.z * per_slice, slice_end = min(steps_total, slice_begin + per_slice);
+    const int per = (per_slice + ks - 1) / ks;
+    const int n_chunks = (max(slice_end - slice_begin, 0) + 1) / 2;
+
+    // piece p = tid + 512 j of a chunk: row p / 8, 16 bytes p % 8 of the row's 128
+    const int piece = tid & 7, prow = tid >> 3;   // rows prow, prow + 64, ...
+    struct Fetched {
+        f32x4_t w[4], a;
+    };
+    auto fetch = [&](int c, Fetched& f) {
+        // K is a multiple of 16 here, so a step inside the slice is whole; a chunk's second step past the slice's end is
+        // fetched from a clamped place and never multiplied.  Nothing is done to the values before they are staged, so
+        // the loads stay out while the chunk before is multiplied.
+        const int kk = min((slice_begin + 2 * c) * 16 + piece * 4, K - 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) f.w[j] = *reinterpret_cast<const f32x4_t*>(g.W + (size_t)min(n0 + prow + 64 * j, g.N - 1) * K + kk);
+        f.a = *reinterpret_cast<const f32x4_t*>(g.A + (size_t)min(m0 + prow, g.M - 1) * g.lda + kk);
+    };
+    auto stage = [&](const Fetched& f, int buf) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<f32x4_t*>(&Ws[buf][(prow + 64 * j) * RL_PITCH + piece * 4]) = f.w[j];
+        *reinterpret_cast<f32x4_t*>(&As[buf][prow * RL_PITCH + piece * 4]) = f.a;
+    };
+
+    f32x4_t total[4][2], acc[4][2];
+#pragma unroll
+    for (int ns = 0; ns < 4; ++ns)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) acc[ns][t] = total[ns][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    bool first_range = true;
+    int in_range = 0;   // steps of the current wave range done
+
+    // a chunk's values are asked for before the chunk ahead of it is multiplied and staged after it (asking two chunks
+    // ahead with a second set of registers was measured and gave nothing)
+    auto multiply_chunk = [&](int c, int buf) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int s = slice_begin + 2 * c + u;
+            if (s < slice_end) {
+                f32x4_t wf[4], af[2];
+#pragma unroll
+                for (int ns = 0; ns < 4; ++ns)
+                    wf[ns] = *reinterpret_cast<const f32x4_t*>(&Ws[buf][(64 * wn + 16 * ns + r) * RL_PITCH + 16 * u + 4 * kg]);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) af[t] = *reinterpret_cast<const f32x4_t*>(&As[buf][(32 * wm + 16 * t + r) * RL_PITCH + 16 * u + 4 * kg]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int ns = 0; ns < 4; ++ns)
+#pragma unroll
+                        for (int t = 0; t < 2; ++t) acc[ns][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf[ns][i], af[t][i], acc[ns][t], 0, 0, 0);
+                if (++in_range == per || s + 1 == slice_end) {   // a wave range ends
+#pragma unroll
+                    for (int ns = 0; ns < 4; ++ns)
+#pragma unroll
+                        for (int t = 0; t < 2; ++t) {
+                            if (first_range) total[ns][t] = acc[ns][t];
+                            else total[ns][t] = f32x4_t{total[ns][t][0] + acc[ns][t][0], total[ns][t][1] + acc[ns][t][1],
+                                                        total[ns][t][2] + acc[ns][t][2], total[ns][t][3] + acc[ns][t][3]};
+                            acc[ns][t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+                        }
+                    first_range = false;
+                    in_range = 0;
+                }
+            }
+        }
+    };
+    Fetched f;
+    if (n_chunks > 0) {
+        fetch(0, f);
+        stage(f, 0);
+    }
+    __syncthreads();
+    for (int c = 0; c < n_chunks; ++c) {
+        if (c + 1 < n_chunks) fetch(c + 1, f);
+        multiply_chunk(c, c & 1);
+        if (c + 1 < n_chunks) stage(f, (c & 1) ^ 1);
+        __syncthreads();
+    }
+
+    float* C = g.C + (size_t)blockIdx.z * g.slice_stride;
+    const bool quad = !g.add && g.ldc % 4 == 0 && ((uintptr_t)C & 15) == 0;
+#pragma unroll
+    for (int ns = 0; ns < 4; ++ns)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int m = m0 + 32 * wm + 16 * t + r;
+            if (m >= g.M) continue;
+            const int n = n0 + 64 * wn + 16 * ns + 4 * kg;
+            float* c = C + (size_t)m * g.ldc + n;
+            const f32x4_t v = total[ns][t];
+            if (quad && n + 3 < g.N) {
+                *reinterpret_cast<f32x4_t*>(c) = v;     // a lane's four neighbouring features in one access
+                continue;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (n + i >= g.N) continue;
+                c[i] = g.add ? c[i] + v[i] : v[i];
+            }
+        }
+}
+
 // K a multiple of 4, rows 16-byte aligned.  ks: 1, 2, 4, 8 or 16 waves share a strip's K.  slices > 1: K's steps are
 // cut into `slices` runs first, run z written to C + z * slice_stride (no add then); the caller adds the runs in order.
 extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, int M, int N, int K, int lda, int ldc, int add, int ks,
@@ -207,6 +329,12 @@ extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, in
     int chunks = (M + 63) / 64;
     if (chunks > 1024) chunks = 1024;
     const dim3 grid((N + 15) / 16, M <= 64 ? 1 : chunks, slices);
+    if (M > 64 && N >= 128 && K % 16 == 0 && ks >= 1 && ks <= 16) {
+        const dim3 staged((N + RL_FEATS - 1) / RL_FEATS, (M + RL_ROWS - 1) / RL_ROWS, slices);
+        if (staged.y > 65535) return -2;
+        hipLaunchKernelGGL(gemm_rows_f32_lds_kernel, staged, dim3(512), 0, stream, g, ks);
+        return LLMX_CHECK_LAUNCH();
+    }
     if (M > 64 && N >= 64 && ks <= 8) {
         const dim3 wide((N + 63) / 64, (M + 63) / 64, slices);
         if (wide.y > 65535) return -2;
