@@ -108,11 +108,11 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     __shared__ __attribute__((aligned(1024))) bf16_t Ws[FAST ? STAGES * TL_BN * TL_BK : TL_BN * TL_LD];
     __shared__ int rows_a[BM];
     __shared__ int rows_c[BM];
-    __shared__ int tile_info[2];
+    __shared__ int tile_info[4];
     __shared__ int scan_waves[4];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    if (GROUPED && !tile_launch_runs(g)) return;
+    const bool runs = !GROUPED || tile_launch_runs(g);   // looked at below, once the first offsets are asked for too
     constexpr int FEATS = (EPI == TL_SWIGLU) ? 64 : 128;  // output features a workgroup covers
     const int n0 = blockIdx.x * FEATS;
     const bf16_t* W = g.W;
@@ -125,7 +125,9 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         for (int e0 = 0; e0 < g.n_groups; e0 += 256) {
             const int e = e0 + tid;
             const int begin = e < g.n_groups ? g.group_offsets[e] : 0;
-            const int tiles = e < g.n_groups ? (g.group_offsets[e + 1] - begin + BM - 1) / BM : 0;
+            const int end = e < g.n_groups ? g.group_offsets[e + 1] : 0;
+            if (!runs) return;   // the whole workgroup: the other tile size has this product
+            const int tiles = (end - begin + BM - 1) / BM;
             int incl = tiles;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
@@ -140,7 +142,8 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
             const int first = before + incl - tiles;
             if ((int)blockIdx.y >= first && (int)blockIdx.y < first + tiles) {
                 tile_info[0] = e;
-                tile_info[1] = (int)blockIdx.y - first;
+                tile_info[1] = begin + ((int)blockIdx.y - first) * BM;
+                tile_info[2] = end;
             }
             base += round_total;
             __syncthreads();
@@ -149,8 +152,8 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         __syncthreads();
         const int e = tile_info[0];
         if (e < 0) return;
-        row_begin = g.group_offsets[e] + tile_info[1] * BM;
-        row_end = min(g.group_offsets[e + 1], row_begin + BM);
+        row_begin = tile_info[1];
+        row_end = min(tile_info[2], row_begin + BM);
         W += (size_t)e * g.w_group_stride;
     } else {
         row_begin = blockIdx.y * BM;
@@ -472,11 +475,11 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
     __shared__ __attribute__((aligned(1024))) bf16_t Ws[WD_STAGES * WD_BN * TL_BK];
     __shared__ int rows_a[WD_BM];
     __shared__ int rows_c[WD_BM];
-    __shared__ int tile_info[2];
+    __shared__ int tile_info[4];
     __shared__ int scan_waves[8];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    if (GROUPED && !tile_launch_runs(g)) return;
+    const bool runs = !GROUPED || tile_launch_runs(g);   // looked at below, once the first offsets are asked for too
     constexpr int HALF = WD_BN / 2;                               // SwiGLU: gate rows, then the up rows of the same features
     constexpr int FEATS = (EPI == TL_SWIGLU) ? HALF : WD_BN;      // output features a workgroup covers
     const int n0 = blockIdx.x * FEATS;
@@ -489,7 +492,9 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
         for (int e0 = 0; e0 < g.n_groups; e0 += 512) {
             const int e = e0 + tid;
             const int begin = e < g.n_groups ? g.group_offsets[e] : 0;
-            const int tiles = e < g.n_groups ? (g.group_offsets[e + 1] - begin + WD_BM - 1) / WD_BM : 0;
+            const int end = e < g.n_groups ? g.group_offsets[e + 1] : 0;
+            if (!runs) return;   // the whole workgroup: the other tile size has this product
+            const int tiles = (end - begin + WD_BM - 1) / WD_BM;
             int incl = tiles;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
@@ -506,7 +511,8 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
             const int first = before + incl - tiles;
             if ((int)blockIdx.y >= first && (int)blockIdx.y < first + tiles) {
                 tile_info[0] = e;
-                tile_info[1] = (int)blockIdx.y - first;
+                tile_info[1] = begin + ((int)blockIdx.y - first) * WD_BM;
+                tile_info[2] = end;
             }
             base += round_total;
             __syncthreads();
@@ -515,8 +521,8 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
         __syncthreads();
         const int e = tile_info[0];
         if (e < 0) return;
-        row_begin = g.group_offsets[e] + tile_info[1] * WD_BM;
-        row_end = min(g.group_offsets[e + 1], row_begin + WD_BM);
+        row_begin = tile_info[1];
+        row_end = min(tile_info[2], row_begin + WD_BM);
         W += (size_t)e * g.w_group_stride;
     } else {
         row_begin = blockIdx.y * WD_BM;
