@@ -5,6 +5,9 @@
 // exp((score - best) / temp); sums are double; the draw r * sum walks ids in increasing order and returns the first id
 // whose running sum exceeds it, else the best id.  `skip` (>= n for none) is an id no path gives.
 #include "common.h"
+#include "no_alloc.h"
+#include <cstdio>
+#include <mutex>
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_WAVES (SAMPLE_THREADS / 64)
@@ -116,8 +119,80 @@ extern "C" int llmx_argmax_rows(const float* scores, const int* skip, int* out, 
         hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, skip, out, n);
         return LLMX_CHECK_LAUNCH();
     }
+    if (rows > 65535) return -2;   // the slices' grid holds the rows in its second dimension
     const int n_slices = (n + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
     hipLaunchKernelGGL(argmax_slices_kernel, dim3(n_slices, rows), dim3(256), 0, stream, scores, skip, (Leader*)partial, n, n_slices);
+    hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(64), 0, stream, scores, skip, (const Leader*)partial, out, n, n_slices);
+    return LLMX_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------------------
+// The same arg-max for callers that cannot allocate (no_alloc.h): the slices' leaders go through a fixed array in the
+// library's device image.  In host code the array's name is only a stand-in; its device address is asked for once per
+// device with hipGetSymbolAddress and that pointer is what the kernels get.
+static __device__ __align__(256) Leader argmax_static_scratch[LLMX_ARGMAX_STATIC_LEADERS];
+
+#define NO_ALLOC_MAX_DEVICES 64
+static std::mutex no_alloc_lock;
+static Leader* no_alloc_scratch_of[NO_ALLOC_MAX_DEVICES];   // the array's address on each device, 0 until resolved
+static thread_local char no_alloc_error[256];
+
+extern "C" const char* llmx_no_alloc_last_error(void) { return no_alloc_error; }
+
+// The static array's address on the current device, resolved at the first call there; null with the reason recorded.
+static Leader* no_alloc_scratch(int* rc) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess || device < 0 || device >= NO_ALLOC_MAX_DEVICES) {
+        snprintf(no_alloc_error, sizeof no_alloc_error, "no current device below %d (%s)", NO_ALLOC_MAX_DEVICES, hipGetErrorString(e));
+        *rc = e != hipSuccess ? (int)e : -2;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(no_alloc_lock);
+    if (!no_alloc_scratch_of[device]) {
+        void* at = nullptr;
+        e = hipGetSymbolAddress(&at, HIP_SYMBOL(argmax_static_scratch));
+        if (e != hipSuccess || !at) {
+            snprintf(no_alloc_error, sizeof no_alloc_error, "hipGetSymbolAddress of the static scratch failed on device %d (%s)", device,
+                     hipGetErrorString(e));
+            *rc = e != hipSuccess ? (int)e : -1;
+            return nullptr;
+        }
+        no_alloc_scratch_of[device] = (Leader*)at;
+    }
+    *rc = 0;
+    return no_alloc_scratch_of[device];
+}
+
+extern "C" int llmx_no_alloc_init(void) {
+    no_alloc_error[0] = 0;
+    int rc = 0;
+    no_alloc_scratch(&rc);
+    return rc;
+}
+
+extern "C" int llmx_argmax_rows_static(const float* scores, const int* skip, int* out, int rows, int n, hipStream_t stream) {
+    no_alloc_error[0] = 0;
+    if (rows <= 0) return 0;
+    if (n <= 0) {
+        snprintf(no_alloc_error, sizeof no_alloc_error, "llmx_argmax_rows_static: rows of %d scores", n);
+        return -2;
+    }
+    if (n <= 2 * ARGMAX_SLICE) {   // narrow rows need no scratch
+        hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, skip, out, n);
+        return LLMX_CHECK_LAUNCH();
+    }
+    const int n_slices = (n + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
+    if ((long)rows * n_slices > LLMX_ARGMAX_STATIC_LEADERS || rows > 65535) {
+        snprintf(no_alloc_error, sizeof no_alloc_error,
+                 "llmx_argmax_rows_static: %d rows x %d slices of %d scores need %ld leaders, the static scratch holds %d (and at most 65535 rows)",
+                 rows, n_slices, ARGMAX_SLICE, (long)rows * n_slices, LLMX_ARGMAX_STATIC_LEADERS);
+        return -2;
+    }
+    int rc = 0;
+    Leader* partial = no_alloc_scratch(&rc);
+    if (!partial) return rc;
+    hipLaunchKernelGGL(argmax_slices_kernel, dim3(n_slices, rows), dim3(256), 0, stream, scores, skip, partial, n, n_slices);
     hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(64), 0, stream, scores, skip, (const Leader*)partial, out, n, n_slices);
     return LLMX_CHECK_LAUNCH();
 }
