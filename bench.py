@@ -1,18 +1,28 @@
 """Decode and prefill throughput of MiniMax-M3 at real layer sizes with random weights, on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--points 1,64] [--sweep] [--long]
 
 A step is one decode step of the whole batch: B requests, each at a context that reaches C tokens at the last timed
 step, one new token each, logits -> greedy token on the device -> ids read back (the reference's batched `tg`,
-/root/reference/src/cli/main.cpp:1246-1254, reads each pass's results before the next).  Prints one JSON line:
-`value` = decoded tokens a second at the default batch; `points` = the same at batch 1 and 64; `prefill` = one
-2,048-token prompt from an empty cache; `roofline` = bytes the decode step has to read / its time against HBM's 8 TB/s;
-`calibration` = what a device copy, a read-only pass and a square bf16 library product reach on this card.  The prefill
-record's `frac` is its flops over the bf16 peak; beside it `hbm_frac` is the weights it has to read (the experts its
-tokens picked, counted in the warm-up run) over its time against 8 TB/s: few rows an expert make the step a
-weight-streaming one.
-Token ids are a fixed LCG sequence; weights are N(0, 0.02) generated on the device.  The context before the timed
-steps is built by running each request's prompt through the model (`context_fill` gives its rate).
+/root/reference/src/cli/main.cpp:1246-1254, reads each pass's results before the next; it reports every test it times,
+:1192-1287, and so does this line).  Prints one JSON line:
+  value, ms_per_step   decoded tokens a second and the step's time at the default batch;
+  roofline             bytes the decode step has to read (every weight it uses once, with the measured number of
+                       distinct experts a layer, and the cache of the live requests) / its time, against HBM's 8 TB/s;
+  points               the same for every measured batch, flat: decode_b<B> (tok/s), decode_b<B>_ms, _gb (bytes to read),
+                       _experts (distinct a layer) and _frac (of 8 TB/s); decode_b<B>_logits_to_host is the default batch
+                       with every step's logits copied to pinned host memory, as the reference's bench reads them;
+  prefill              one 2,048-token prompt from an empty cache: tok/s, ms, `frac` = flops / time / the bf16 peak,
+                       `hbm_frac` = the weights it has to read (the experts its tokens picked) / time / 8 TB/s, and the
+                       first layer's feed-forward alone (first_layer_*): its rows are all different, so it touches every
+                       expert and streams all their weights;
+  sweep (--sweep)      further sizes: batch 8 at 16k and 32k tokens of context, batch 16 and 32 at 4k, and the mixed step
+                       a scheduler issues: a 512-token prompt portion beside 8 decoding requests;
+  long (--long)        the long-context configuration: 30 layers, 2 requests of 65,536 prompt tokens in portions of
+                       2,048, then 256 decoded tokens each (the engine is freed and built again for it);
+  calibration          what a device copy, a read-only pass and a square bf16 library product reach on this card.
+Token ids are a fixed LCG sequence; weights are N(0, 0.02) generated on the device.  The context before the timed steps
+is built by running each request's prompt through the model in portions of 2,048 tokens (`context_fill` gives its rate).
 """
 
 from __future__ import annotations
@@ -30,6 +40,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 PREFILL_TOKENS = 2048
+FULL_LAYERS, CONTEXT = 24, 4096                     # the benchmark's configuration: 24 of the model's 62 layers, 4,096 tokens
+LONG_LAYERS, LONG_PROMPT, LONG_DECODE = 30, 65536, 256
 
 
 def parse():
@@ -37,28 +49,28 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=32)
     ap.add_argument("--warmup", type=int, default=4, help="untimed steps before the timed ones (at least 1)")
-    ap.add_argument("--layers", type=int, default=0, help="layers to run (0: as many of the configuration's as fit)")
+    ap.add_argument("--layers", type=int, default=0, help="layers to run (0: the configuration's 24)")
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--context", type=int, default=0, help="tokens each sequence holds at the last timed step (0: the configuration's)")
+    ap.add_argument("--context", type=int, default=0, help="tokens each sequence holds at the last timed step (0: the configuration's 4,096)")
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
+    ap.add_argument("--sweep", action="store_true", help="also measure further contexts and batches and the mixed prompt + decode step")
+    ap.add_argument("--long", action="store_true", help="also run the long-context configuration (30 layers, 2 x 65,536 tokens, 256 decoded)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-calibration", action="store_true", help="skip the copy, read and library-product rates of the card")
     ap.add_argument("--no-logits-to-host", action="store_true",
                     help="skip the extra point: the default batch with every step's logits copied to the host")
     ap.add_argument("--only-prefill", action="store_true", help="for profiling: measure the prefill alone and print its record")
-    ap.add_argument("--context-fill", choices=["prefill", "synthetic"], default="prefill",
-                    help="how the context before the timed steps gets into the cache: prompts run through the model in "
-                         "portions of 2,048 tokens, or (for quick profiling runs) random keys and values written directly")
+    ap.add_argument("--only-long", action="store_true", help="for profiling: run the long-context configuration alone and print its record")
     return ap.parse_args()
 
 
-# The real layer sizes: 24 layers of the 62-layer model's widths (the third configuration of the benchmark's list).
-def real_config(layers: int, context: int):
+def real_config(layers: int, positions: int):
+    """The real layer sizes (the third configuration of the benchmark's list) with `layers` layers."""
     from llmx_amd import MiniMaxM3Config
     return MiniMaxM3Config(vocab_size=200064, hidden_size=3072, num_hidden_layers=layers, num_attention_heads=48,
                            num_key_value_heads=8, head_dim=128, rotary_dim=64, rope_theta=5e6, rms_norm_eps=1e-6,
                            num_local_experts=256, num_experts_per_tok=8, intermediate_size=1536, routed_scaling_factor=1.0,
-                           norm_topk_prob=True, tie_word_embeddings=False, max_position_embeddings=max(context, PREFILL_TOKENS))
+                           norm_topk_prob=True, tie_word_embeddings=False, max_position_embeddings=max(positions, PREFILL_TOKENS))
 
 
 def lcg_ids(n, vocab, seed):
@@ -106,6 +118,10 @@ class DistinctExperts:
             import torch
             self.counts.append(int(torch.unique(tensors["ids"]).numel()))
 
+    @property
+    def mean(self):
+        return sum(self.counts) / max(1, len(self.counts))
+
 
 def calibrate(torch, device):
     """What this card gives a plain program: a device-to-device copy (bytes read plus written), a read-only pass
@@ -137,7 +153,24 @@ def calibrate(torch, device):
     return {"copy_gbs": round(copy_gbs, 1), "read_gbs": round(read_gbs, 1), "bf16_gemm_tflops": round(tflops, 1)}
 
 
-def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch, read_logits=False):
+def fill_context(engine, rids, tokens_each, torch):
+    """Runs each request's prompt of `tokens_each` tokens through the model in portions of 2,048; returns the seconds it took."""
+    from llmx_amd.engine import StepEntry
+    c = engine.config
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i, rid in enumerate(rids):
+        engine.add_request(rid)
+        ids = lcg_ids(tokens_each, c.vocab_size, 100 + i)
+        for s in range(0, tokens_each, PREFILL_TOKENS):
+            engine.step([StepEntry(rid, ids[s:s + PREFILL_TOKENS], [])])
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def run_decode(engine, sampler_out, batch, context, steps, warmup, torch, read_logits=False):
+    """`steps` timed decode steps of `batch` requests that end at `context` tokens each.  Returns a record: seconds of the
+    timed steps, of the context fill, and the distinct experts a layer that the first warm-up step touched."""
     from llmx_amd import ops
     from llmx_amd.engine import StepEntry
     c = engine.config
@@ -145,18 +178,7 @@ def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch, 
     if start < 1:
         raise SystemExit(f"bench: context {context} is shorter than the {steps + warmup} steps")
     rids = [f"b{batch}_{i}" for i in range(batch)]
-    torch.cuda.synchronize()
-    t_fill = time.perf_counter()
-    for i, rid in enumerate(rids):
-        engine.add_request(rid)
-        if fill == "synthetic":
-            engine.assume_context(rid, start)
-        else:
-            ids = lcg_ids(start, c.vocab_size, 100 + i)
-            for s in range(0, start, PREFILL_TOKENS):
-                engine.step([StepEntry(rid, ids[s:s + PREFILL_TOKENS], [])])
-    torch.cuda.synchronize()
-    run_decode.fill_s = time.perf_counter() - t_fill
+    fill_s = fill_context(engine, rids, start, torch)
     last = [lcg_ids(1, c.vocab_size, 7 + i)[0] for i in range(batch)]
     out = sampler_out[:batch]
     host_logits = torch.empty(batch, c.vocab_size, dtype=torch.float32, pin_memory=True) if read_logits else None
@@ -174,7 +196,6 @@ def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch, 
     engine.observer = watcher
     one()
     engine.observer = None
-    distinct = sum(watcher.counts) / max(1, len(watcher.counts))
     for _ in range(warmup - 1):
         one()
     torch.cuda.synchronize()
@@ -185,38 +206,138 @@ def run_decode(engine, sampler_out, batch, context, steps, warmup, fill, torch, 
     dt = time.perf_counter() - t0
     for rid in rids:
         engine.end_request(rid)
-    return dt, distinct
+    return {"s": dt, "fill_s": fill_s, "fill_tokens": batch * start, "distinct": watcher.mean}
+
+
+def decode_record(cfg, batch, context, steps, run):
+    """tok/s, ms a step, the bytes the step has to read and their share of the HBM peak."""
+    step_s = run["s"] / steps
+    need = decode_bytes(cfg, batch, context - steps / 2, run["distinct"])
+    return {"tok_s": round(batch * steps / run["s"], 2), "ms": round(step_s * 1e3, 4), "gb": round(need / 1e9, 2),
+            "experts": round(run["distinct"], 1), "gbs": round(need / step_s / 1e9, 1), "frac": round(need / step_s / 1e9 / HBM_PEAK_GBS, 4)}
 
 
 def run_prefill(engine, cfg, sampler_out, torch):
-    """One prompt of 2,048 tokens from an empty cache, in one step, to its first sampled token; best of two after a warm-up."""
+    """One prompt of 2,048 tokens from an empty cache, in one step, to its first sampled token; best of two after a
+    warm-up.  The first layer's feed-forward (router, routing, both routed products, combine) is timed by events of its own."""
     from llmx_amd import ops
     from llmx_amd.engine import StepEntry
     T = PREFILL_TOKENS
-    times = []
+    times, first_ms = [], []
     watcher = DistinctExperts()
-    for rep in range(3):   # the first is the warm-up; it also counts the experts the prompt touches per layer
-        rid = f"p{rep}"
-        engine.add_request(rid)
-        ids = lcg_ids(T, cfg.vocab_size, 500 + rep)
-        engine.observer = watcher if rep == 0 else None
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        logits = engine.step([StepEntry(rid, ids, [T - 1])])
-        ops.argmax_rows(logits, sampler_out[:1])
-        sampler_out[:1].tolist()
-        torch.cuda.synchronize()
-        times.append(time.perf_counter() - t0)
-        engine.end_request(rid)
-    engine.observer = None
+    ffn = engine.model.blocks[0].ffn
+    plain_forward = ffn.forward
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+
+    def timed_forward(*args, **kwargs):
+        marks[0].record()
+        plain_forward(*args, **kwargs)
+        marks[1].record()
+
+    ffn.forward = timed_forward
+    try:
+        for rep in range(3):   # the first is the warm-up; it also counts the experts the prompt touches per layer
+            rid = f"p{rep}"
+            engine.add_request(rid)
+            ids = lcg_ids(T, cfg.vocab_size, 500 + rep)
+            engine.observer = watcher if rep == 0 else None
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = engine.step([StepEntry(rid, ids, [T - 1])])
+            ops.argmax_rows(logits, sampler_out[:1])
+            sampler_out[:1].tolist()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            first_ms.append(marks[0].elapsed_time(marks[1]))
+            engine.end_request(rid)
+    finally:
+        ffn.forward = plain_forward
+        engine.observer = None
     t = min(times[1:])
     flops = prefill_flops(cfg, T)
     # what the step has to read: every weight it uses once (the experts the prompt's tokens picked), as for decode
-    distinct = sum(watcher.counts) / max(1, len(watcher.counts))
-    need = decode_bytes(cfg, 0, 0, distinct)
+    need = decode_bytes(cfg, 0, 0, watcher.mean)
+    first_experts = watcher.counts[0] if watcher.counts else 0
+    _, small, expert = layer_weight_bytes(cfg, 2)
+    first_bytes = first_experts * expert + small
+    first = min(first_ms[1:]) * 1e-3
     return {"value": round(T / t, 1), "tokens": T, "ms": round(t * 1e3, 3), "frac": round(flops / t / PEAK_FLOPS["bf16"], 5),
-            "tflop": round(flops / 1e12, 2), "distinct_experts_per_layer": round(distinct, 1), "weights_read_gb": round(need / 1e9, 1),
-            "hbm_frac": round(need / t / 1e9 / HBM_PEAK_GBS, 4)}
+            "tflop": round(flops / 1e12, 2), "distinct_experts_per_layer": round(watcher.mean, 1), "weights_read_gb": round(need / 1e9, 1),
+            "hbm_frac": round(need / t / 1e9 / HBM_PEAK_GBS, 4),
+            "first_layer_ffn_ms": round(first * 1e3, 3), "first_layer_experts": first_experts, "first_layer_gb": round(first_bytes / 1e9, 2),
+            "first_layer_hbm_frac": round(first_bytes / first / 1e9 / HBM_PEAK_GBS, 4)}
+
+
+def run_mixed_step(engine, cfg, sampler_out, context, portion, decoding, reps, torch):
+    """The step a scheduler issues while a prompt arrives: `decoding` requests at `context` tokens take one token each
+    beside a `portion`-token portion of another request's prompt.  Returns ms a step (mean of `reps`) and tokens a second."""
+    from llmx_amd import ops
+    from llmx_amd.engine import StepEntry
+    rids = [f"m{i}" for i in range(decoding)]
+    fill_context(engine, rids, context - reps - 1, torch)
+    engine.add_request("prompt")
+    ids = lcg_ids(portion * (reps + 1), cfg.vocab_size, 900)
+    last = [lcg_ids(1, cfg.vocab_size, 7 + i)[0] for i in range(decoding)]
+    out = sampler_out[:decoding]
+
+    def one(k):
+        nonlocal last
+        entries = [StepEntry(rid, [t], [0]) for rid, t in zip(rids, last)] + [StepEntry("prompt", ids[k * portion:(k + 1) * portion], [])]
+        ops.argmax_rows(engine.step(entries), out)
+        last = out.tolist()
+
+    one(0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(1, reps + 1):
+        one(k)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    for rid in rids + ["prompt"]:
+        engine.end_request(rid)
+    return {"ms": round(dt * 1e3, 3), "tok_s": round((decoding + portion) / dt, 1), "decoding": decoding, "portion": portion, "context": context}
+
+
+def run_long(torch, steps_warm=4):
+    """The long-context configuration: 30 layers, 2 requests of 65,536 prompt tokens fed in portions of 2,048, then 256
+    decoded tokens each.  Returns its record."""
+    from llmx_amd import Engine, RandomInit, ops
+    from llmx_amd.engine import StepEntry
+    batch, context = 2, LONG_PROMPT + LONG_DECODE
+    cfg = real_config(LONG_LAYERS, context)
+    engine = Engine.from_random(cfg, RandomInit(seed=0, std=0.02), dtype="bfloat16", kv_tokens=batch * context, page_tokens=16, max_requests=batch)
+    rids = [f"long{i}" for i in range(batch)]
+    fill_s = fill_context(engine, rids, LONG_PROMPT, torch)
+    out = torch.empty(batch, dtype=torch.int32, device=engine.device)
+    last = [lcg_ids(1, cfg.vocab_size, 7 + i)[0] for i in range(batch)]
+    watcher = DistinctExperts()
+
+    def one():
+        nonlocal last
+        ops.argmax_rows(engine.step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, last)]), out)
+        last = out.tolist()
+
+    engine.observer = watcher
+    one()
+    engine.observer = None
+    for _ in range(steps_warm - 1):
+        one()
+    torch.cuda.synchronize()
+    timed = LONG_DECODE - steps_warm
+    t0 = time.perf_counter()
+    for _ in range(timed):
+        one()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    record = decode_record(cfg, batch, context, timed, {"s": dt, "distinct": watcher.mean})
+    for rid in rids:
+        engine.end_request(rid)
+    weights_gb = engine.weight_bytes() / 1e9
+    del engine
+    torch.cuda.empty_cache()
+    return {"layers": LONG_LAYERS, "batch": batch, "prompt_tokens": LONG_PROMPT, "portion": PREFILL_TOKENS, "decoded": LONG_DECODE,
+            "weights_gb": round(weights_gb, 1), "prompt_s": round(fill_s, 2), "prompt_tok_s": round(batch * LONG_PROMPT / fill_s, 1),
+            "decode_tok_s": record["tok_s"], "decode_ms": record["ms"], "decode_gb": record["gb"], "decode_frac": record["frac"]}
 
 
 def main():
@@ -226,20 +347,20 @@ def main():
         print(f"bench: this engine runs on one GPU; --gpus {a.gpus} is not built")
         sys.exit(2)
     import torch
-    from llmx_amd import Engine, RandomInit, ops
-    from llmx_amd.engine import StepEntry
+    from llmx_amd import Engine, RandomInit
 
-    full_layers, context = 24, 4096
-    context = a.context or context
-    layers = a.layers or full_layers
+    if a.only_long:
+        print(json.dumps({"long": run_long(torch)}))
+        return
+    context = a.context or CONTEXT
+    layers = a.layers or FULL_LAYERS
     points = [int(p) for p in a.points.split(",") if p.strip()]
-    max_batch = max([a.batch] + points)
-    cfg = real_config(layers, context)
+    sweep = [(8, 16384), (8, 32768), (16, context), (32, context)] if a.sweep else []
+    kv_tokens = max([a.batch * context] + [b * context for b in points] + [b * c for b, c in sweep] + ([9 * context] if a.sweep else []))
+    max_batch = max([a.batch] + points + [b for b, _ in sweep] + ([9] if a.sweep else []))
+    cfg = real_config(layers, max([context] + [c for _, c in sweep]))
     t_setup = time.perf_counter()
-    engine = Engine.from_random(cfg, RandomInit(seed=0, std=0.02), dtype="bfloat16", kv_tokens=max_batch * context,
-                                page_tokens=16, max_requests=max_batch)
-    if a.context_fill == "synthetic":
-        engine.fill_cache_random(seed=1)
+    engine = Engine.from_random(cfg, RandomInit(seed=0, std=0.02), dtype="bfloat16", kv_tokens=kv_tokens, page_tokens=16, max_requests=max_batch)
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t_setup
     sampler_out = torch.empty(max_batch, dtype=torch.int32, device=engine.device)
@@ -247,52 +368,65 @@ def main():
     if a.only_prefill:
         print(json.dumps({"prefill": run_prefill(engine, cfg, sampler_out, torch)}))
         return
-    dt, distinct = run_decode(engine, sampler_out, a.batch, context, a.steps, a.warmup, a.context_fill, torch)
-    fill_s = run_decode.fill_s
-    ms_per_step = dt / a.steps * 1e3
-    value = a.batch * a.steps / dt
-    mean_context = context - a.steps / 2
-    need = decode_bytes(cfg, a.batch, mean_context, distinct)
-    achieved = need / (dt / a.steps) / 1e9
+    run = run_decode(engine, sampler_out, a.batch, context, a.steps, a.warmup, torch)
+    head = decode_record(cfg, a.batch, context, a.steps, run)
 
     result = {
         "metric": "decode tok/s (MiniMax-M3 real layer sizes, batch %d, context %d)" % (a.batch, context),
-        "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": head["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": head["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic: LCG token ids, N(0,0.02) weights generated on the device; context before the timed steps: "
-                + ("random keys and values written to the cache" if a.context_fill == "synthetic" else "prompts run through the model"),
+        "data": "synthetic: LCG token ids, N(0,0.02) weights generated on the device; context before the timed steps: prompts run through the model",
         "config": {
-            "model": "MiniMax-M3 slice (real layer sizes, configs[2])", "layers": layers, "layers_of_config": full_layers, "layers_full_model": 62,
+            "model": "MiniMax-M3 slice (real layer sizes, configs[2])", "layers": layers, "layers_of_config": FULL_LAYERS, "layers_full_model": 62,
             "hidden": cfg.hidden_size, "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "rotary_dim": cfg.rotary_dim, "experts": cfg.num_local_experts, "top_k": cfg.num_experts_per_tok,
             "expert_intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "global_batch": a.batch, "seq_len": context,
             "page_tokens": 16, "parallelism": "single GPU", "weights_gb": round(engine.weight_bytes() / 1e9, 1),
         },
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "bytes_gb": round(need / 1e9, 2),
-                     "distinct_experts_per_layer": round(distinct, 1)},
+        "roofline": {"bound": "hbm", "achieved": head["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": head["frac"],
+                     "bytes_gb": head["gb"], "distinct_experts_per_layer": head["experts"]},
         "setup_s": round(setup_s, 1),
-        **({"context_fill": {"tokens": a.batch * (context - a.steps - a.warmup), "s": round(fill_s, 2),
-                             "tok_s": round(a.batch * (context - a.steps - a.warmup) / fill_s, 1), "portion": PREFILL_TOKENS}}
-           if a.context_fill == "prefill" else {}),
+        "context_fill": {"tokens": run["fill_tokens"], "s": round(run["fill_s"], 2), "tok_s": round(run["fill_tokens"] / run["fill_s"], 1),
+                         "portion": PREFILL_TOKENS},
     }
 
     pts = {}
+
+    def add_point(name, rec):
+        pts[name] = rec["tok_s"]
+        for key in ("ms", "gb", "experts", "frac"):
+            pts[f"{name}_{key}"] = rec[key]
+
+    add_point(f"decode_b{a.batch}", head)
     if points and not a.no_logits_to_host:
-        dtb, _ = run_decode(engine, sampler_out, a.batch, context, a.steps, a.warmup, a.context_fill, torch, read_logits=True)
-        pts[f"decode_b{a.batch}_logits_to_host"] = round(a.batch * a.steps / dtb, 2)
+        r = run_decode(engine, sampler_out, a.batch, context, a.steps, a.warmup, torch, read_logits=True)
+        pts[f"decode_b{a.batch}_logits_to_host"] = round(a.batch * a.steps / r["s"], 2)
     for b in points:
-        steps = a.steps
-        dtb, _ = run_decode(engine, sampler_out, b, context, steps, a.warmup, a.context_fill, torch)
-        pts[f"decode_b{b}"] = round(b * steps / dtb, 2)
-    if pts:
-        result["points"] = pts
+        add_point(f"decode_b{b}", decode_record(cfg, b, context, a.steps, run_decode(engine, sampler_out, b, context, a.steps, a.warmup, torch)))
+    result["points"] = pts
+
+    if a.sweep:
+        sw = {}
+        for b, c in sweep:
+            rec = decode_record(cfg, b, c, a.steps, run_decode(engine, sampler_out, b, c, a.steps, a.warmup, torch))
+            name = f"decode_b{b}_ctx{c}"
+            sw[name] = rec["tok_s"]
+            for key in ("ms", "gb", "experts", "frac"):
+                sw[f"{name}_{key}"] = rec[key]
+        mixed = run_mixed_step(engine, cfg, sampler_out, context, 512, 8, 8, torch)
+        sw["mixed_512_beside_8_ms"] = mixed["ms"]
+        sw["mixed_512_beside_8_tok_s"] = mixed["tok_s"]
+        result["sweep"] = sw
 
     if not a.no_prefill:
         result["prefill"] = run_prefill(engine, cfg, sampler_out, torch)
     if not a.no_calibration:
         result["calibration"] = calibrate(torch, sampler_out.device)
+    if a.long:
+        del engine
+        torch.cuda.empty_cache()
+        result["long"] = run_long(torch)
     print(json.dumps(result))
 
 

@@ -5,8 +5,10 @@ Flags keep the reference's names and meanings where it has them (main.cpp:2018-2
 --ignore-eos, --stop, --dtype, --ubatch, --kv-tokens, --verbose; logits: --then-ids, --last, --per-token, --top;
 perplexity: --ctx-size/-c, --chunks, --per-token.  There is no tokenizer here: a prompt is a list of token ids
 (comma or space separated), given on the line, with --file, or made up with --prompt-len; a stop text is a sequence
-of token ids.  A usage error exits with
-status 2 (main.cpp:100-103); a flag given twice is refused (:129-159).
+of token ids.  Instead of a model folder, `--config JSON --random SEED` runs the configuration with weights generated
+on the device from the seed (the reference builds its file-less model the same way for its bench,
+/root/reference/src/model/arch/registry.hpp:144-152): `llmx generate --config cfg.json --random 0 "1 2 3"`.
+A usage error exits with status 2 (main.cpp:100-103); a flag given twice is refused (:129-159).
 """
 
 from __future__ import annotations
@@ -55,6 +57,44 @@ def _add_exec(p):
     p.add_argument("--page-tokens", type=int, default=16, action=_Once, help="tokens a cache page holds (default %(default)s)")
     p.add_argument("--max-seqs", type=int, default=8, action=_Once, help="requests running together at most (default %(default)s)")
     p.add_argument("--verbose", nargs=0, default=False, action=_Once)
+    p.add_argument("--config", default=None, action=_Once, help="a config.json to run with random weights instead of a model folder (needs --random)")
+    p.add_argument("--random", type=int, default=None, action=_Once, help="seed of the weights generated on the device for --config")
+    p.add_argument("--std", type=float, default=0.02, action=_Once, help="standard deviation of the random matrices (default %(default)s)")
+
+
+def _model_and_prompt(a, command: str):
+    """The positionals are MODEL [PROMPT], or [PROMPT] alone when --config names the model."""
+    words = list(a.words)
+    if (a.config is None) != (a.random is None):
+        raise SystemExit2(f"{command}: --config and --random go together")
+    if a.config is None:
+        if not words:
+            raise SystemExit2(f"{command} needs a model folder, or --config JSON --random SEED")
+        a.model, words = words[0], words[1:]
+    else:
+        a.model = None
+    if len(words) > 1:
+        raise SystemExit2(f"{command}: unexpected argument {words[1]!r}")
+    a.prompt = words[0] if words else None
+
+
+def _config_of(a):
+    from .models import read_config, read_model_dir
+    if a.model is not None:
+        return read_model_dir(a.model)[0]
+    try:
+        return read_config(json.loads(Path(a.config).read_text()))
+    except (OSError, json.JSONDecodeError) as e:
+        raise SystemExit2(f"--config {a.config}: {e}")
+
+
+def _engine(a, cfg, **options):
+    """The engine of the model folder, or of the configuration with weights generated on the device."""
+    from .engine import Engine
+    if a.model is not None:
+        return Engine.load(a.model, dtype=a.dtype, **options)
+    from .weights import RandomInit
+    return Engine.from_random(cfg, RandomInit(seed=a.random, std=a.std), dtype=a.dtype, **options)
 
 
 def _ids(text: str):
@@ -86,12 +126,11 @@ def _lcg_ids(n: int, vocab: int, seed: int = 1):
 
 
 def cmd_generate(a) -> int:
-    from .engine import Engine
     from .engine.generation import Generator
     from .engine.scheduler import Request
-    from .models import read_model_dir
+    _model_and_prompt(a, "generate")
     params = _params(a)
-    cfg, _ = read_model_dir(a.model)
+    cfg = _config_of(a)
     if a.file:
         prompts = [_ids(line) for line in Path(a.file).read_text().splitlines() if line.strip()]
     elif a.prompt is not None:
@@ -104,7 +143,7 @@ def cmd_generate(a) -> int:
         raise SystemExit2("generate: empty prompt")
     need = sum(len(p) + params.max_tokens for p in prompts[:a.max_seqs]) if len(prompts) > 1 else len(prompts[0]) + params.max_tokens
     kv_tokens = a.kv_tokens or max(need + a.page_tokens * a.max_seqs, max(len(p) for p in prompts) + params.max_tokens)
-    engine = Engine.load(a.model, dtype=a.dtype, kv_tokens=kv_tokens, page_tokens=a.page_tokens, max_requests=a.max_seqs)
+    engine = _engine(a, cfg, kv_tokens=kv_tokens, page_tokens=a.page_tokens, max_requests=a.max_seqs)
     gen = Generator(engine, a.max_seqs, a.ubatch)
     for i, p in enumerate(prompts):
         import copy
@@ -129,13 +168,14 @@ def cmd_generate(a) -> int:
 
 def cmd_logits(a) -> int:
     """Top-N logits of the last positions, whole or token by token (the reference's `llmx logits`, main.cpp:934-980)."""
-    from .engine import Engine, StepEntry
+    from .engine import StepEntry
+    _model_and_prompt(a, "logits")
     ids = _prompt_ids(a, "logits")
     if a.then_ids:
         ids = ids + _ids(Path(a.then_ids).read_text())
     if not ids:
         raise SystemExit2("logits: empty prompt")
-    engine = Engine.load(a.model, dtype=a.dtype, kv_tokens=a.kv_tokens or len(ids) + a.page_tokens, page_tokens=a.page_tokens, max_requests=1)
+    engine = _engine(a, _config_of(a), kv_tokens=a.kv_tokens or len(ids) + a.page_tokens, page_tokens=a.page_tokens, max_requests=1)
     engine.add_request(0)
     last = min(a.last or 1, len(ids))
     rows = []
@@ -175,13 +215,13 @@ def _prompt_ids(a, command: str):
 
 def cmd_perplexity(a) -> int:
     """Mean negative log-likelihood over windows of token ids (the reference's `llmx perplexity`, main.cpp:982-1008)."""
-    from .engine import Engine
     from .engine.perplexity import MIN_WINDOW, perplexity
+    _model_and_prompt(a, "perplexity")
     ids = _prompt_ids(a, "perplexity")
     if len(ids) < MIN_WINDOW:
         raise SystemExit2(f"perplexity: need at least {MIN_WINDOW} tokens")
     window = min(a.ctx_size or len(ids), len(ids))
-    engine = Engine.load(a.model, dtype=a.dtype, kv_tokens=a.kv_tokens or window + a.page_tokens, page_tokens=a.page_tokens, max_requests=1)
+    engine = _engine(a, _config_of(a), kv_tokens=a.kv_tokens or window + a.page_tokens, page_tokens=a.page_tokens, max_requests=1)
     window = min(window, engine.max_positions)
     r = perplexity(engine, ids, window, a.chunks, a.per_token, a.ubatch)
     if a.verbose:
@@ -232,16 +272,15 @@ def build_parser():
     ap = argparse.ArgumentParser(prog="llmx", description="MiniMax-M3 on one MI355X: generate, logits, perplexity, replay, random, bench")
     sub = ap.add_subparsers(dest="command", required=True)
     g = sub.add_parser("generate", help="generate tokens after a prompt of token ids")
-    g.add_argument("model", help="model folder (config.json + model.safetensors)")
-    g.add_argument("prompt", nargs="?", default=None, help="token ids, comma or space separated")
+    g.add_argument("words", nargs="*", metavar="MODEL [PROMPT]",
+                   help="model folder (config.json + model.safetensors), then token ids, comma or space separated; with --config the prompt alone")
     g.add_argument("--file", "-f", default=None, help="a file with one prompt of token ids per line")
     g.add_argument("--prompt-len", type=int, default=0, help="make up a prompt of this many fixed token ids")
     _add_sampling(g)
     _add_exec(g)
     g.set_defaults(run=cmd_generate)
     l = sub.add_parser("logits", help="top logits of the last positions of a prompt")
-    l.add_argument("model")
-    l.add_argument("prompt", nargs="?", default=None)
+    l.add_argument("words", nargs="*", metavar="MODEL [PROMPT]")
     l.add_argument("--file", "-f", default=None)
     l.add_argument("--then-ids", default=None, help="a file of token ids appended to the prompt")
     l.add_argument("--last", type=int, default=0, help="report this many final positions")
@@ -250,8 +289,7 @@ def build_parser():
     _add_exec(l)
     l.set_defaults(run=cmd_logits)
     x = sub.add_parser("perplexity", help="mean negative log-likelihood of token ids, in windows from an empty history")
-    x.add_argument("model")
-    x.add_argument("prompt", nargs="?", default=None)
+    x.add_argument("words", nargs="*", metavar="MODEL [PROMPT]")
     x.add_argument("--file", "-f", default=None, help="a file of token ids")
     x.add_argument("--ctx-size", "-c", type=int, default=0, action=_Once, help="window tokens (default: all the ids, at most the model's context)")
     x.add_argument("--chunks", type=int, default=0, action=_Once, help="windows at most (default: all)")

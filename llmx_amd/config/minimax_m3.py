@@ -14,6 +14,7 @@ from __future__ import annotations
 from dataclasses import dataclass, asdict
 from typing import Any, Mapping, Optional
 
+from ..limits import MAX_EXPERTS, MAX_HEAD_DIM, MAX_TOP_K
 from .reader import ConfigError, KeyReader
 
 ARCHITECTURE = "MiniMaxM3ForCausalLM"
@@ -156,7 +157,11 @@ def check(c: MiniMaxM3Config) -> None:
         raise bad("num_key_value_heads", "the head count must be divisible by the KV head count")
     if c.head_dim % 2 or c.rotary_dim % 2 or c.rotary_dim > c.head_dim or c.rotary_dim < 0:
         raise bad("rotary_dim", "the rotary width must be even and at most the head width")
-    if c.num_experts_per_tok > c.num_local_experts or c.num_experts_per_tok > 256:
-        raise bad("num_experts_per_tok", "more experts per token than the layer has, or above 256")
+    if c.num_experts_per_tok > c.num_local_experts or c.num_experts_per_tok > MAX_TOP_K:
+        raise bad("num_experts_per_tok", f"more experts per token than the layer has, or above the kernels' limit of {MAX_TOP_K}")
+    if c.num_local_experts > MAX_EXPERTS:
+        raise bad("num_local_experts", f"{c.num_local_experts} is above the routing kernels' limit of {MAX_EXPERTS}")
+    if c.head_dim > MAX_HEAD_DIM:
+        raise bad("head_dim", f"{c.head_dim} is above the attention kernels' limit of {MAX_HEAD_DIM}")
     if c.eos_token_id is not None and not 0 <= c.eos_token_id < c.vocab_size:
         raise bad("eos_token_id", "outside the vocabulary")

@@ -2,8 +2,8 @@
 
 The library is a plain shared object with a C ABI (no Python headers), built in
 the tree beside its sources so that it travels with the checkout.  `load_path`
-returns what is built and compiles only when nothing is; `build` always
-compiles.  Where the source tree cannot be written the library goes to a
+returns what is built when its stamp (a hash of sources and flags) is the
+current one and compiles otherwise; `build` always compiles.  Where the source tree cannot be written the library goes to a
 per-user folder under the system's temporary directory.
 """
 
@@ -119,13 +119,16 @@ def build(verbose: bool = True) -> Path:
 
 
 def load_path(verbose: bool = True) -> Path:
-    """The built library; compiled now if none is there."""
+    """The built library; compiled now if none is there or if what is there was built from other sources or flags."""
+    want = _stamp()
     for lib in lib_candidates():
         if lib.exists():
             stamp = lib.with_name(LIB_NAME + ".stamp")
-            if verbose and (not stamp.exists() or stamp.read_text() != _stamp()):
-                _say(f"warning: {lib} is older than its sources; build again (python -c 'import __graft_entry__ as g; g.build()')")
-            return lib
+            if stamp.exists() and stamp.read_text() == want:
+                return lib
+            if verbose:
+                _say(f"{lib} was not built from the current sources: building again")
+            break
     return build(verbose=verbose)
 
 

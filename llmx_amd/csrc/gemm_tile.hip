@@ -28,9 +28,7 @@ enum : int { TL_STORE = 0, TL_ADD = 1, TL_SWIGLU = 2 };
 #define TL_BN 128
 #define TL_BK 64
 #define TL_LD 72  // padded row length in bf16 elements (144 bytes)
-#ifndef TL_STAGES
 #define TL_STAGES 2  // tiles in LDS in the lean loop: one being multiplied, the other on its way (48 KB: three workgroups a CU; measured better than deeper stages with fewer workgroups)
-#endif
 
 // Lane l of the wave: 16 bytes from base + offset (bytes, per lane) to LDS at lds + 16 l (lds the same for the whole
 // wave).  Written as an instruction of its own so that waiting for it is the kernel's business: the loop below keeps

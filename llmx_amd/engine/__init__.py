@@ -1,7 +1,7 @@
 """The engine: step function, scheduler and generation."""
 
-from .batch import EntryView, StepEntry, StepState
-from .engine import Engine, StepError, resolve_dtype
+from .batch import EntryView, StepEntry, StepError, StepState, check_entries
+from .engine import Engine, resolve_dtype
 from .model import BuiltModel
 from .scheduler import PlannedEntry, Request, Scheduler, SchedulerError
 

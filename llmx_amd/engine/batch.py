@@ -12,6 +12,8 @@ from typing import Dict, Hashable, List, Sequence, Tuple
 import numpy as np
 import torch
 
+from ..limits import MAX_STEP_ROWS
+
 
 @dataclass(frozen=True)
 class StepEntry:
@@ -28,6 +30,45 @@ class EntryView:
     row0: int      # its first row in the step
     n: int         # its number of rows
     past: int      # tokens it held before the step
+
+
+class StepError(ValueError):
+    """A batch the step function refuses; nothing was reserved or run."""
+
+
+def check_entries(entries: Sequence[StepEntry], cache, max_positions: int, vocab: int) -> List[EntryView]:
+    """The refusals that come before anything is reserved (/root/reference/src/model/passes.hpp:271-413): an empty
+    batch, a request named twice or not open, an entry without tokens, a context that would be exceeded, a token id
+    outside the embedding's rows, a wanted place outside the entry, more rows than a step takes.  Returns the entries'
+    views (slot, first row, rows, tokens held before)."""
+    if not entries:
+        raise StepError("step: an empty batch")
+    seen = set()
+    views: List[EntryView] = []
+    row0 = 0
+    for e in entries:
+        if e.request in seen:
+            raise StepError(f"step: request {e.request!r} appears twice in one batch")
+        seen.add(e.request)
+        if not cache.is_open(e.request):
+            raise StepError(f"step: request {e.request!r} is not open")
+        n = len(e.tokens)
+        if n == 0:
+            raise StepError(f"step: request {e.request!r} brings no tokens")
+        past = cache.length(e.request)
+        if past + n > max_positions:
+            raise StepError(f"step: context length exceeded: request {e.request!r} would hold {past + n} tokens of {max_positions}")
+        for t in e.tokens:
+            if not 0 <= int(t) < vocab:
+                raise StepError(f"step: token id {t} is outside the embedding's rows")
+        for w in e.want:
+            if not 0 <= int(w) < n:
+                raise StepError(f"step: request {e.request!r} wants the logits of place {w} among {n} tokens")
+        views.append(EntryView(e.request, cache.slot(e.request), row0, n, past))
+        row0 += n
+    if row0 > MAX_STEP_ROWS:
+        raise StepError(f"step: {row0} token rows in one step; a step takes at most {MAX_STEP_ROWS}")
+    return views
 
 
 class Workspace:

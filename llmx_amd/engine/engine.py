@@ -8,6 +8,7 @@ before anything is reserved, :633-653 reserve pages, :771-830 run, :1007-1032 co
 
 from __future__ import annotations
 
+from dataclasses import replace
 from pathlib import Path
 from typing import Dict, Hashable, List, Optional, Sequence, Union
 
@@ -21,17 +22,12 @@ from ..parts.base import BuildContext, LayerCache
 from ..parts.spec import KVNeed, ModelSpec, StateNeed
 from ..weights import ModelFiles, RandomInit, load as load_weights
 from ..weights.loader import device_dtype
-from ..weights.random_init import stored_dtype
-from ..weights.device_init import fill_random
-from .batch import EntryView, RowPlanUploader, StepEntry, StepState, Workspace
+from ..weights.random_init import fill_random, stored_dtype
+from .batch import EntryView, RowPlanUploader, StepEntry, StepError, StepState, Workspace, check_entries
 from .model import BuiltModel
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
            "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
-
-
-class StepError(ValueError):
-    """A batch the step function refuses; nothing was reserved or run."""
 
 
 def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
@@ -113,8 +109,10 @@ class Engine:
             files.close()
 
     @classmethod
-    def from_random(cls, config, init: RandomInit = RandomInit(), dtype="bfloat16", **options) -> "Engine":
-        """An engine whose weights are generated on the device from (seed, tensor name); nothing is read or written."""
+    def from_random(cls, config, init: RandomInit = RandomInit(), dtype="bfloat16", tensors_out: Optional[dict] = None,
+                    **options) -> "Engine":
+        """An engine whose weights are generated on the device from (seed, tensor name); nothing is read or written.
+        `tensors_out`, when given, receives the device tensors by name as the parts were handed them."""
         def generate(eng: "Engine"):
             tensors = {}
             for s in eng.model.tensor_specs():
@@ -122,6 +120,8 @@ class Engine:
                 t = torch.empty(s.shape, dtype=dt, device=eng.device)
                 fill_random(t, s, init)
                 tensors[s.name] = t
+            if tensors_out is not None:
+                tensors_out.update(tensors)
             return tensors
 
         return cls(config, registry.assemble(config), dtype, weights=generate, **options)
@@ -147,14 +147,16 @@ class Engine:
                 self._index_in_group.append(-1)
         self.group_needs = keys
         groups = [GroupSpec(f"kv{g}", self.page_tokens, n_pages, need.window) for g, need in enumerate(keys)]
-        self.cache = CacheManager(groups, self.max_requests)
+        # a model with per-request state steps into a second slot, so that a step that fails leaves the state as it was
+        self._stateful = any(isinstance(need, StateNeed) for need in needs)
+        self.cache = CacheManager(groups, self.max_requests, shadow_slots=self._stateful)
         # [cache in group, K|V, page, kv head, token in page * head dim]; keys are [token][dim], values [dim][token]
         self._kv = [torch.zeros((counts[g], 2, n_pages, need.kv_heads, self.page_tokens * need.head_dim), dtype=self.act_dtype,
                                 device=self.device) for g, need in enumerate(keys)]
         self._state: List[Optional[torch.Tensor]] = []
         for need in needs:
             if isinstance(need, StateNeed):
-                self._state.append(torch.zeros((self.max_requests, *need.shape), dtype=getattr(torch, need.dtype), device=self.device))
+                self._state.append(torch.zeros((self.cache.slots.capacity, *need.shape), dtype=getattr(torch, need.dtype), device=self.device))
             else:
                 self._state.append(None)
         self._layer_caches: List[LayerCache] = []
@@ -182,6 +184,21 @@ class Engine:
         """The request is finished: what it holds is given back."""
         self.cache.close(request)
 
+    def truncate(self, request: Hashable, length: int) -> None:
+        """Takes the request back to its first `length` tokens (its pages beyond them are given back), so that it can go
+        on from that prefix: scoring another continuation, dropping a rejected draft.  A model that keeps fixed-size
+        state per request can only be taken back to nothing (the state is cleared) or left as it is: a state cannot be
+        unwound.  The reference's rule: /root/reference/src/model/kv_cache.hpp:126-134, history.hpp:58-59."""
+        held = self.cache.length(request)
+        if self._stateful and 0 < length < held:
+            raise StepError(f"truncate: request {request!r} keeps a state of fixed size, which cannot be taken back to {length} of {held} tokens")
+        self.cache.truncate(request, length)
+        if self._stateful and length == 0 and held > 0:
+            slot = self.cache.slot(request)
+            for s in self._state:
+                if s is not None:
+                    s[slot].zero_()
+
     def has_request(self, request: Hashable) -> bool:
         return self.cache.is_open(request)
 
@@ -201,33 +218,8 @@ class Engine:
         if not self._loaded:
             raise RuntimeError("the engine has no weights yet")
         entries = list(entries)
-        if not entries:
-            raise StepError("step: an empty batch")
-        seen = set()
-        V = self.spec.vocab_size
-        views: List[EntryView] = []
-        row0 = 0
-        for e in entries:
-            if e.request in seen:
-                raise StepError(f"step: request {e.request!r} appears twice in one batch")
-            seen.add(e.request)
-            if not self.cache.is_open(e.request):
-                raise StepError(f"step: request {e.request!r} is not open")
-            n = len(e.tokens)
-            if n == 0:
-                raise StepError(f"step: request {e.request!r} brings no tokens")
-            past = self.cache.length(e.request)
-            if past + n > self.max_positions:
-                raise StepError(f"step: context length exceeded: request {e.request!r} would hold {past + n} tokens of {self.max_positions}")
-            for t in e.tokens:
-                if not 0 <= int(t) < V:
-                    raise StepError(f"step: token id {t} is outside the embedding's rows")
-            for w in e.want:
-                if not 0 <= int(w) < n:
-                    raise StepError(f"step: request {e.request!r} wants the logits of place {w} among {n} tokens")
-            views.append(EntryView(e.request, self.cache.slot(e.request), row0, n, past))
-            row0 += n
-        T = row0
+        views = check_entries(entries, self.cache, self.max_positions, self.spec.vocab_size)
+        T = views[-1].row0 + views[-1].n
 
         prepared: List[Hashable] = []
         try:
@@ -239,6 +231,8 @@ class Engine:
                 self.cache.abort(r)
             raise
         try:
+            if self._stateful:
+                views = self._enter_shadow_slots(views)
             logits = self._run(entries, views, T)
         except BaseException:
             for r in prepared:
@@ -247,6 +241,19 @@ class Engine:
         for r in prepared:
             self.cache.commit(r)
         return logits
+
+    def _enter_shadow_slots(self, views: List[EntryView]) -> List[EntryView]:
+        """Each entry's state is copied into the slot its step writes, and the entry is pointed there; the slot it had
+        is not touched until the step commits."""
+        moved = []
+        for v in views:
+            to = self.cache.step_slot(v.request)
+            if to != v.slot:
+                for s in self._state:
+                    if s is not None:
+                        s[to].copy_(s[v.slot])
+            moved.append(replace(v, slot=to))
+        return moved
 
     # -- wrappers over step, for one request (the reference's Model::prefill / step / score, runtime.hpp:1278-1385) --
     def prefill(self, request: Hashable, tokens: Sequence[int], portion: int = 512) -> torch.Tensor:
@@ -389,19 +396,6 @@ class Engine:
         record = _StepGraph(graph, logits, plans, *before)
         self._graphs[key] = record
         return record
-
-    # -- for measurement ----------------------------------------------------------
-    def assume_context(self, request: Hashable, n: int) -> None:
-        """Marks the request's next n positions as held without computing them: their keys and values are whatever
-        the pages hold.  For measuring decode at a given depth without paying for the prompt; never for serving."""
-        self.cache.prepare(request, n)
-        self.cache.commit(request)
-
-    def fill_cache_random(self, seed: int = 1) -> None:
-        """Writes seeded N(0,1) values into every page of keys and values (see assume_context)."""
-        from ..weights.random_init import mix64
-        for g, store in enumerate(self._kv):
-            ops.fill_random(store, mix64(seed * 1315423911 + g), 0, 0.0, 1.0)
 
     # -- accounting -------------------------------------------------------------
     def weight_bytes(self) -> int:

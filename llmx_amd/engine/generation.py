@@ -30,10 +30,11 @@ class GenerationStats:
 class Generator:
     """Owns a scheduler and a sampler over one engine; `run` plays every submitted request to its end."""
 
-    def __init__(self, engine: Engine, max_seqs: Optional[int] = None, max_step_tokens: int = DEFAULT_STEP_TOKENS):
+    def __init__(self, engine: Engine, max_seqs: Optional[int] = None, max_step_tokens: int = DEFAULT_STEP_TOKENS,
+                 feed_last: bool = True):
         self.engine = engine
         self.scheduler = Scheduler(engine.cache.groups, max_seqs or engine.max_requests, max_step_tokens,
-                                   max_positions=engine.max_positions, eos_token_id=engine.spec.eos_token_id)
+                                   max_positions=engine.max_positions, eos_token_id=engine.spec.eos_token_id, feed_last=feed_last)
         if self.scheduler.max_seqs > engine.max_requests:
             raise SchedulerError(f"generation: {self.scheduler.max_seqs} seats but the engine holds {engine.max_requests} requests")
         self.sampler = Sampler(engine.vocab_size, engine.device)
@@ -47,8 +48,19 @@ class Generator:
         self.scheduler.submit(request)
 
     def step(self, on_token: Optional[Callable[[Hashable, int], None]] = None) -> List[Request]:
-        """One round: admit, plan, run, sample, advance.  Returns the requests that finished in it."""
-        import torch
+        """One round: admit, plan, run, sample, advance.  Returns the requests that finished in it.
+
+        When the round fails (a refused step, a kernel error) every running request is ended in the engine before the
+        error goes on, so that nothing stays open holding a slot and pages."""
+        try:
+            return self._round(on_token)
+        except BaseException:
+            for r in self.scheduler.running:
+                if self.engine.has_request(r.id):
+                    self.engine.end_request(r.id)
+            raise
+
+    def _round(self, on_token: Optional[Callable[[Hashable, int], None]]) -> List[Request]:
         sch = self.scheduler
         for r in sch.admit():
             self.engine.add_request(r.id)

@@ -8,7 +8,10 @@ Policy (decisions only; it owns no model and is tested with a simulated executor
   * A step takes the decoding requests first, one token each, in order of admission, then portions of prompts in order
     of admission while the step's token budget lasts; a portion wants logits only when it reaches the prompt's end.
   * A request finishes on its end token (not kept, unless ignore_eos), when its generated ids end with one of its
-    stop sequences, or at max_tokens; its pages and slot go back at once.
+    stop sequences, or at max_tokens; its pages and slot go back at once.  The last token that max_tokens allows is
+    fed in the next step, without logits, before the request ends, so that what the cache holds is the whole reply
+    (/root/reference/src/inference/generate.hpp:28-45: an end token and the token completing a stop text are not fed,
+    the last token the limit allows is); `feed_last=False` skips that step.
 The shape follows the reference's scheduler (/root/reference/src/server/scheduler.hpp:1187-1376 form, :752-766 admission,
 :2514-2571 retire; reservation: /root/reference/src/server/policy.hpp:153-158).
 """
@@ -65,7 +68,7 @@ class PlannedEntry:
 
 class Scheduler:
     def __init__(self, groups: Sequence[GroupSpec], max_seqs: int, max_step_tokens: int = DEFAULT_STEP_TOKENS,
-                 max_positions: Optional[int] = None, eos_token_id: Optional[int] = None):
+                 max_positions: Optional[int] = None, eos_token_id: Optional[int] = None, feed_last: bool = True):
         if max_seqs < 1 or max_step_tokens < 1:
             raise SchedulerError("scheduler: max_seqs and max_step_tokens must be at least 1")
         self.groups = list(groups)
@@ -73,6 +76,7 @@ class Scheduler:
         self.max_step_tokens = max_step_tokens
         self.max_positions = max_positions
         self.eos = eos_token_id
+        self.feed_last = bool(feed_last)
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []
         self.finished: Dict[Hashable, Request] = {}
@@ -126,7 +130,8 @@ class Scheduler:
         entries: List[PlannedEntry] = []
         for r in self.running:
             if r.decoding and budget > 0:
-                entries.append(PlannedEntry(r.id, [r.generated[-1]], True))
+                # a request that reached max_tokens feeds its last token and wants nothing more
+                entries.append(PlannedEntry(r.id, [r.generated[-1]], r.finish_reason is None))
                 budget -= 1
         for r in self.running:
             if budget <= 0:
@@ -146,6 +151,8 @@ class Scheduler:
             r = by_id[e.request]
             r.fed += len(e.tokens)
             if not e.wants_logits:
+                if r.finish_reason is not None:      # its last token is in the cache now
+                    done.append(r)
                 continue
             tok = sampled[e.request]
             if self.eos is not None and tok == self.eos and not r.params.ignore_eos:
@@ -156,7 +163,7 @@ class Scheduler:
                     r.finish_reason = "stop"       # the token that completes a stop sequence is kept and not fed
                 elif len(r.generated) >= r.params.max_tokens:
                     r.finish_reason = "length"
-            if r.finish_reason:
+            if r.finish_reason and not (r.finish_reason == "length" and self.feed_last):
                 done.append(r)
         for r in done:
             self.running.remove(r)

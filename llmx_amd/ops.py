@@ -15,6 +15,7 @@ from typing import Optional
 import torch
 
 from .csrc import build as _build
+from .limits import MAX_EXPERTS, MAX_HEAD_DIM, MAX_TOP_K
 
 F32, BF16 = 0, 1
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
@@ -147,15 +148,10 @@ TILE_FILL = 1024              # feature tiles of 128 from which the tiled kernel
 SKINNY_MAX_GROUPED_ROWS = 16   # routed products of at most this many token rows do (measured: beyond it the tiled kernel streams the experts faster)
 
 
-_KS_OVERRIDE = None   # set by tuning scripts only
-
-
 def _split_k(n_strips: int, K: int) -> int:
     """Runs the products cut K into (waves that share one 16-feature strip in the weight-streaming kernel; run boundaries
     in the tiled kernel): enough strips * runs to fill the chip, at least 12 steps of 32 a run.  A function of the
     product's shape only, so a row's bits do not depend on the batch."""
-    if _KS_OVERRIDE:
-        return _KS_OVERRIDE
     ks = 1
     while ks < 8 and n_strips * ks < 2048 and (K // 32) // (ks * 2) >= 12:
         ks *= 2
@@ -345,8 +341,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     n_pages, n_kv_heads, page_tokens, head_dim = k_cache.shape
     if q.shape[1] != n_heads * head_dim or out.shape != q.shape or q.dtype != k_cache.dtype or out.dtype != q.dtype:
         raise KernelError("paged_attention: shapes or dtypes do not agree")
-    if head_dim > 256 or n_heads % n_kv_heads:
-        raise KernelError(f"paged_attention: head_dim {head_dim} above 256 or heads {n_heads} not a multiple of KV heads {n_kv_heads}")
+    if head_dim > MAX_HEAD_DIM or n_heads % n_kv_heads:
+        raise KernelError(f"paged_attention: head_dim {head_dim} above {MAX_HEAD_DIM} or heads {n_heads} not a multiple of KV heads {n_kv_heads}")
     common = (_dev(q, "q"), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache", shape=(n_pages, n_kv_heads, head_dim, page_tokens)),
               _dev(pos, "pos", torch.int32, (rows,)), _dev(row_entry, "row_entry", torch.int32, (rows,)), _dev(tables, "tables", torch.int32))
     if plan is not None and plan.n_items and attention_mfma_ok(q.dtype, head_dim, page_tokens):
@@ -380,8 +376,8 @@ def route_topk(z: torch.Tensor, bias: Optional[torch.Tensor], ids: torch.Tensor,
     """`parts` [slices, rows, experts]: the logits arrive as partial sums (gemm_f32's `parts`); they are added in slice
     order into z first."""
     rows, n_experts = z.shape
-    if n_experts > 1024 or k > 256 or k > n_experts:
-        raise KernelError(f"route_topk takes at most 1024 experts and 256 picks, not {n_experts} and {k}")
+    if n_experts > MAX_EXPERTS or k > MAX_TOP_K or k > n_experts:
+        raise KernelError(f"route_topk takes at most {MAX_EXPERTS} experts and {MAX_TOP_K} picks, not {n_experts} and {k}")
     _check(lib().llmx_route_topk(_dev(z, "z", torch.float32), *_parts_args(z, parts), _dev(bias, "bias", torch.float32, (n_experts,)),
                                  _dev(ids, "ids", torch.int32, (rows, k)), _dev(weights, "weights", torch.float32, (rows, k)),
                                  rows, n_experts, k, score, 1 if normalize else 0, float(scale), _stream()), "route_topk")

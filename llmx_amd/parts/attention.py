@@ -14,6 +14,7 @@ import numpy as np
 import torch
 
 from .. import ops
+from ..limits import MAX_HEAD_DIM
 from .base import BuildContext, LayerCache, Mixer, build_part, register
 from .spec import KVNeed, PartSpec, TensorSpec
 
@@ -35,6 +36,8 @@ class Attention(Mixer):
         self.window = p.get("window")
         if self.heads % self.kv_heads:
             raise ValueError("the head count must be divisible by the KV head count")
+        if not 0 < self.head_dim <= MAX_HEAD_DIM:
+            raise ValueError(f"attention: head_dim {self.head_dim} is outside what the attention kernels take (1 to {MAX_HEAD_DIM})")
         if p.get("qk_norm", "none") not in _NORM_MODES:
             raise ValueError(f"qk_norm {p.get('qk_norm')!r} is not one of {sorted(_NORM_MODES)}")
         self.norm_mode = _NORM_MODES[p.get("qk_norm", "none")]

@@ -14,6 +14,7 @@ import re
 import torch
 
 from .. import ops
+from ..limits import MAX_EXPERTS, MAX_TOP_K
 from .base import FeedForward, register
 from .spec import TensorSpec
 
@@ -41,6 +42,9 @@ class RoutedExperts(FeedForward):
         self.scale = float(p.get("scale", 1.0))
         if not 0 < self.top_k <= self.experts:
             raise ValueError("experts per token must be between 1 and the expert count")
+        if self.experts > MAX_EXPERTS or self.top_k > MAX_TOP_K:
+            raise ValueError(f"routed experts: {self.experts} experts with {self.top_k} picks a token; the routing kernels take at most "
+                             f"{MAX_EXPERTS} experts and {MAX_TOP_K} picks")
         self.per_expert = False
         self.w_router = self.bias = self.w_gate_up = self.w_down = None
 

@@ -10,6 +10,9 @@ All entries of a step run as one batch through the engine's own step function (t
 generation uses).  For a step in which something is wanted the logits at the wanted places are written to
 OUT/<step>.f32 as little-endian float32 [wanted, vocab], in the order of the entries and of `want`.  After every step
 `done <step>` is printed and flushed.  Requests named in `end` give back what they hold after the step.
+With --routing the routed layers' expert picks and router logits of every step's rows are written beside the logits
+(OUT/<step>.picks.i32 [routed layers, rows, k], OUT/<step>.router.f32 [routed layers, rows, experts]), as the reference's
+route hook shows them (/root/reference/src/model/arch/blocks.hpp:118-138).
 Modelled on the reference's captures (/root/reference/tools/model_logits.cpp:82-109) and its replay of recorded passes
 (/root/reference/src/server/scheduler.hpp:860-868).
 """
@@ -31,6 +34,7 @@ def main(argv=None) -> int:
                     help="most tokens live requests hold at any time, each request's count rounded up to a multiple of 64")
     ap.add_argument("--page-tokens", type=int, default=16, help="tokens a cache page holds (a divisor or a multiple of 64)")
     ap.add_argument("--max-requests", type=int, default=8, help="most requests live at a time")
+    ap.add_argument("--routing", action="store_true", help="also write every step's expert picks and router logits")
     args = ap.parse_args(argv)
     if args.max_tokens <= 0:
         ap.error("--max-tokens must be positive")
@@ -48,6 +52,12 @@ def main(argv=None) -> int:
     kv_tokens = -(-args.max_tokens // unit) * unit
     engine = Engine.load(args.model, dtype=args.dtype, kv_tokens=kv_tokens, page_tokens=args.page_tokens,
                          max_requests=args.max_requests)
+    routed = []      # what the routed layers of the running step showed, in run order
+    if args.routing:
+        def observer(step, kind, **tensors):
+            if kind == "routing":
+                routed.append((tensors["ids"].cpu().numpy().copy(), tensors["logits"].cpu().numpy().copy()))
+        engine.observer = observer
     for line in sys.stdin:
         line = line.strip()
         if not line:
@@ -61,7 +71,11 @@ def main(argv=None) -> int:
                 engine.add_request(rid)
             entries.append(StepEntry(rid, [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
         if entries:
+            routed.clear()
             logits = engine.step(entries)
+            if routed:
+                np.stack([ids for ids, _ in routed]).astype("<i4").tofile(out / f"{step_no}.picks.i32")
+                np.stack([z for _, z in routed]).astype("<f4").tofile(out / f"{step_no}.router.f32")
             if logits.shape[0]:
                 host = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
                 host.tofile(out / f"{step_no}.f32")

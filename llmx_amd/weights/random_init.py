@@ -93,3 +93,11 @@ def stored_dtype(spec: TensorSpec, init: RandomInit) -> torch.dtype:
     if spec.role in ("matrix", "table"):
         return torch.bfloat16 if init.storage == "bfloat16" else torch.float32
     return torch.float32
+
+
+def fill_random(t: torch.Tensor, spec: TensorSpec, init: RandomInit) -> None:
+    """Fills the device tensor `t` in place with the values `host_values(spec, init)` computes, rounded to t's type
+    (models too large to stage on the host)."""
+    from .. import ops
+    kind, a, b = distribution(spec, init)
+    ops.fill_random(t, tensor_key(init.seed, spec.name), kind, a, b)

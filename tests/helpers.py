@@ -66,7 +66,7 @@ def routing_margin(name: str, tokens, rounded: bool = False) -> float:
     _, routing = plain_model.forward(cfg, w, tokens, torch.float64, torch.bfloat16 if rounded else None, return_routing=True)
     k = cfg["num_experts_per_tok"]
     margin = float("inf")
-    for _, _, keys in routing:
+    for _, _, keys, _ in routing:
         top = torch.sort(keys, dim=-1, descending=True).values
         margin = min(margin, float((top[:, k - 1] - top[:, k]).min()))
     return margin
@@ -80,46 +80,82 @@ def row_margins(name: str, length: int, seed: int, rounded: bool):
                                      return_routing=True)
     k = cfg["num_experts_per_tok"]
     margins = torch.full((length,), float("inf"), dtype=torch.float64)
-    for _, _, keys in routing:
+    for _, _, keys, _ in routing:
         top = torch.sort(keys, dim=-1, descending=True).values
         margins = torch.minimum(margins, top[:, k - 1] - top[:, k])
     return margins
 
 
 class RoutingRecorder:
-    """An engine observer that keeps every routed layer's picks by (request, position)."""
+    """An engine observer that keeps every routed layer's picks and router logits by (request, position)."""
 
     def __init__(self, n_layers):
         self.n_layers = n_layers
-        self.picks = {}   # request -> {position: [ids per layer]}
+        self.picks = {}    # request -> {position: [ids per layer]}
+        self.logits = {}   # request -> {position: [router logits per layer]}
 
     def __call__(self, step, kind, **tensors):
         if kind != "routing":
             return
         ids = tensors["ids"].cpu()
+        z = tensors["logits"].cpu()
         for e in step.entries:
             rows = self.picks.setdefault(e.request, {})
+            zrows = self.logits.setdefault(e.request, {})
             for r in range(e.n):
                 rows.setdefault(e.past + r, [None] * self.n_layers)[step.run_index] = ids[e.row0 + r].long()
+                zrows.setdefault(e.past + r, [None] * self.n_layers)[step.run_index] = z[e.row0 + r].clone()
 
     def of(self, request, length):
         """Per layer [length, k] picks of a request."""
         rows = self.picks[request]
         return [torch.stack([rows[p][layer] for p in range(length)]) for layer in range(self.n_layers)]
 
+    def logits_of(self, request, length):
+        """Per layer [length, experts] float32 router logits of a request, as the engine computed them."""
+        rows = self.logits[request]
+        return [torch.stack([rows[p][layer] for p in range(length)]) for layer in range(self.n_layers)]
 
-def plain_logits_with_picks(name, tokens, picks, rounded=True, slack=4e-3):
-    """The plain implementation's logits under the engine's expert picks, after checking that every pick is a
-    legitimate one: its key is within `slack` of the k-th best key of the plain implementation's own router."""
+
+# A pick must be one of the k best keys of the engine's OWN router logits.  Keys are float32 values of about 1; the
+# kernel's expf and the host's differ in the last place, so a key may lie below the k-th best by a few units of 6e-8.
+PICK_SLACK = 4e-7
+# The engine's router logits against the plain implementation's (run with the engine's picks in the layers before),
+# relative to the largest logit (at least 1).  float32: sums of float32 products in another order; the largest
+# difference met over all configurations of these tests is 2.5e-6.  bfloat16: the router reads unrounded rows in both;
+# what differs lies upstream: the engine rounds the softmax weights to bfloat16 as the value product's operand, which
+# the plain implementation does not, and single roundings fall the other way; the largest difference met is 6.0e-3
+# (the test session prints what it met).
+ROUTER_TOL = {False: 1e-5, True: 1e-2}
+MEASURED = {"pick_gap": 0.0, "router_f32": 0.0, "router_bf16": 0.0}
+
+
+def plain_logits_with_picks(name, tokens, picks, rounded=True, engine_logits=None):
+    """The plain implementation's logits under the engine's expert picks, after checking every row's picks: no expert
+    twice, and each pick's key (sigmoid of the engine's own router logit in float32, plus the bias) among the k best
+    of that row within PICK_SLACK; the engine's router logits lie within ROUTER_TOL of the plain ones."""
     cfg, w = plain(name)
     logits, routing = plain_model.forward(cfg, w, tokens, torch.float64, torch.bfloat16 if rounded else None,
                                           return_routing=True, picks=picks)
     k = cfg["num_experts_per_tok"]
-    for layer, (ids, _, keys) in enumerate(routing):
-        kth = torch.sort(keys, dim=-1, descending=True).values[:, k - 1]
-        chosen = torch.gather(keys, 1, ids)
-        assert (chosen >= kth[:, None] - slack).all(), f"layer {layer}: the engine picked an expert whose key is not among the best {k}"
+    for layer, (ids, _, keys, z) in enumerate(routing):
         assert all(len(set(row.tolist())) == k for row in ids), f"layer {layer}: an expert was picked twice"
+        if engine_logits is None:
+            own = keys
+            slack = 1e-5
+        else:
+            ze = engine_logits[layer].float()
+            bias = w[f"model.layers.{layer}.mlp.gate.e_score_correction_bias"].float()
+            own = (1.0 / (1.0 + torch.exp(-ze)) + bias).double()
+            slack = PICK_SLACK
+            scale = max(1.0, float(z.abs().max()))
+            gap = float((ze.double() - z).abs().max()) / scale
+            MEASURED["router_bf16" if rounded else "router_f32"] = max(MEASURED["router_bf16" if rounded else "router_f32"], gap)
+            assert gap <= ROUTER_TOL[rounded], f"layer {layer}: the engine's router logits differ from the plain ones by {gap:.3e} of the largest"
+        kth = torch.sort(own, dim=-1, descending=True).values[:, k - 1]
+        chosen = torch.gather(own, 1, ids)
+        MEASURED["pick_gap"] = max(MEASURED["pick_gap"], float((kth[:, None] - chosen).max()))
+        assert (chosen >= kth[:, None] - slack).all(), f"layer {layer}: the engine picked an expert whose key is not among the best {k}"
     return logits
 
 

@@ -204,18 +204,23 @@ def moe_layer(h, w, prefix, cfg, round_to=None, picks=None):
     else:
         ids, weights = forced_route(z, bias, picks, cfg["norm_topk_prob"], cfg["routed_scaling_factor"])
     hin = _rounded(h, round_to)
-    gate_up = w[prefix + "experts.gate_up_proj"].to(dt)
-    down = w[prefix + "experts.down_proj"].to(dt)
+    gate_up = w[prefix + "experts.gate_up_proj"]      # indexed by expert before widening: only the picked experts are touched
+    down = w[prefix + "experts.down_proj"]
+    # each picked expert's output for the rows that picked it (an expert's weights are widened once) ...
+    y = torch.zeros(ids.shape[0], ids.shape[1], h.shape[1], dtype=dt)
+    for e in sorted(set(ids.flatten().tolist()) - {-1}):
+        rows, slots = torch.nonzero(ids == e, as_tuple=True)
+        y[rows, slots] = swiglu_expert(hin[rows], gate_up[e].to(dt), down[e].to(dt), round_to)
+    # ... and each row's weighted sum in slot order
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         acc = torch.zeros(h.shape[1], dtype=dt)
         for j in range(ids.shape[1]):
-            e = int(ids[t, j])
-            if e >= 0:
-                acc = acc + weights[t, j] * swiglu_expert(hin[t], gate_up[e], down[e], round_to)
+            if int(ids[t, j]) >= 0:
+                acc = acc + weights[t, j] * y[t, j]
         out[t] = acc
     keys = 1.0 / (1.0 + torch.exp(-z)) + bias
-    return out, ids, weights, keys
+    return out, ids, weights, keys, z
 
 
 def rotary_dim_of(cfg):
@@ -234,12 +239,12 @@ def forward(cfg, w, tokens, dtype=torch.float64, round_to=None, return_routing=F
     Embedding (src/model/arch/blocks.hpp:95-97), per layer norm -> mixer joined -> norm -> experts joined
     (src/model/arch/minimax_m3.hpp:247-287, pre-norm, two residual adds), final norm and head (blocks.hpp:267-272).
     `picks` (per layer [T, k] expert ids) replaces the router's own picks; `return_routing` also returns per layer
-    (ids, weights, keys) with keys = sigmoid(z) + bias.
+    (ids, weights, keys, z) with the router logits z and keys = sigmoid(z) + bias.
     """
     tokens = list(tokens)
     T = len(tokens)
     positions = list(range(T)) if positions is None else list(positions)
-    x = w["model.embed_tokens.weight"].to(dtype)[tokens]
+    x = w["model.embed_tokens.weight"][tokens].to(dtype)
     eps = cfg["rms_norm_eps"]
     routing = []
     for layer in range(cfg["num_hidden_layers"]):
@@ -247,8 +252,8 @@ def forward(cfg, w, tokens, dtype=torch.float64, round_to=None, return_routing=F
         h = rms_norm(x, w[p + "input_layernorm.weight"].to(dtype), eps)
         x = x + attention_layer(h, positions, w, p + "self_attn.", cfg, round_to)
         h = rms_norm(x, w[p + "post_attention_layernorm.weight"].to(dtype), eps)
-        y, ids, weights, keys = moe_layer(h, w, p + "mlp.", cfg, round_to, None if picks is None else picks[layer])
-        routing.append((ids, weights, keys))
+        y, ids, weights, keys, z = moe_layer(h, w, p + "mlp.", cfg, round_to, None if picks is None else picks[layer])
+        routing.append((ids, weights, keys, z))
         x = x + y
     h = _rounded(rms_norm(x, w["model.norm.weight"].to(dtype), eps), round_to)
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings") else w["lm_head.weight"]

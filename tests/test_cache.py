@@ -93,7 +93,8 @@ def test_window_gives_pages_back_as_it_passes_them():
 def test_random_orders_never_lose_or_share_a_page(seed):
     rng = random.Random(seed)
     groups = [GroupSpec("kv", 4, 40), GroupSpec("win", 8, 12, window=20)]
-    m = CacheManager(groups, max_requests=5)
+    shadows = seed % 2 == 1
+    m = CacheManager(groups, max_requests=5, shadow_slots=shadows)
     live, next_id = {}, 0
     for _ in range(600):
         action = rng.random()
@@ -101,6 +102,16 @@ def test_random_orders_never_lose_or_share_a_page(seed):
             m.open(next_id)
             live[next_id] = 0
             next_id += 1
+        elif action < 0.35 and live:
+            r = rng.choice(list(live))
+            to = rng.randint(0, live[r])
+            try:
+                m.truncate(r, to)
+            except CacheLogicError as e:
+                assert "keeps the last 20 keys only" in str(e) and m.length(r) == live[r]
+            else:
+                live[r] = to
+                assert m.length(r) == to and m.pages_held(r, 0) == -(-to // 4)
         elif action < 0.85 and live:
             r = rng.choice(list(live))
             n = rng.choice([1, 1, 1, 2, 3, 7, 16])
@@ -127,9 +138,89 @@ def test_random_orders_never_lose_or_share_a_page(seed):
             assert all(0 <= p < g.n_pages for p in held)
         assert m.slots.in_use == len(live)
         assert len({m.slot(r) for r in live}) == len(live)
+        assert all(m.step_slot(r) == m.slot(r) for r in live)      # no step is in progress: nobody holds a second slot
     for r in list(live):
         m.close(r)
     assert all(m.pages_in_use(g) == 0 for g in range(2)) and m.slots.in_use == 0
     m.open("after")
     m.prepare("after", 40 * 4 if False else 12 * 8)        # a request as long as the smaller pool: every page came back
     m.commit("after")
+
+
+def test_truncate_returns_the_pages_beyond_the_new_length():
+    """/root/reference/src/model/kv_cache.hpp:126-134: the history is rolled back to `length` and the blocks beyond it
+    go back; reset is truncate(0)."""
+    m = CacheManager([GroupSpec("kv", 4, 10)], max_requests=2)
+    m.open("a")
+    m.prepare("a", 18)
+    m.commit("a")
+    held = list(m.table("a", 0))
+    assert m.pages_in_use() == 5
+    m.truncate("a", 18)                                   # to its own length: nothing changes
+    assert m.table("a", 0) == held
+    m.truncate("a", 9)                                    # position 8 lies in the third page: it stays, two go back
+    assert m.length("a") == 9 and m.table("a", 0) == held[:3] and m.pages_in_use() == 3
+    m.prepare("a", 4)                                     # the request goes on from there, first with the freed pages
+    m.commit("a")
+    assert m.length("a") == 13 and m.table("a", 0)[:3] == held[:3] and set(m.table("a", 0)) <= set(held)
+    with pytest.raises(CacheLogicError, match="holds 13 tokens and cannot be taken back to 14"):
+        m.truncate("a", 14)
+    with pytest.raises(CacheLogicError, match="cannot be taken back to -1"):
+        m.truncate("a", -1)
+    m.prepare("a", 1)
+    with pytest.raises(CacheLogicError, match="step in progress"):
+        m.truncate("a", 2)
+    m.abort("a")
+    m.truncate("a", 0)
+    assert m.length("a") == 0 and m.table("a", 0) == [] and m.pages_in_use() == 0
+    with pytest.raises(CacheLogicError, match="not open"):
+        m.truncate("b", 0)
+
+
+def test_truncate_inside_a_window_that_gave_pages_back_is_refused():
+    m = CacheManager([GroupSpec("all", 4, 64), GroupSpec("win", 4, 64, window=6)], max_requests=1)
+    m.open("r")
+    m.prepare("r", 30)
+    m.commit("r")                       # the window group holds the pages of positions 24.. only
+    before = (m.length("r"), list(m.table("r", 0)), list(m.table("r", 1)))
+    assert m.table("r", 1)[:6] == [-1] * 6
+    with pytest.raises(CacheLogicError, match="win keeps the last 6 keys only and has given back the page of position 16"):
+        m.truncate("r", 22)             # a row at 22 reads keys 17..21
+    assert (m.length("r"), m.table("r", 0), m.table("r", 1)) == before       # the refusal changed nothing, in either group
+    m.truncate("r", 29)                 # a row at 29 reads 24..28: still held
+    assert m.length("r") == 29 and m.pages_held("r", 0) == 8
+    m.truncate("r", 0)                  # to nothing is always possible
+    assert m.pages_in_use(0) == 0 and m.pages_in_use(1) == 0
+
+
+def test_shadow_slots_keep_the_committed_state_apart_from_a_running_step():
+    """With shadow slots a step writes a second slot; commit makes it the request's, abort drops it (the reference keeps
+    the live slot as a mark while a pass writes another: /root/reference/src/model/kv_cache.hpp:216-266)."""
+    m = CacheManager([GroupSpec("kv", 4, 8)], max_requests=2, shadow_slots=True)
+    assert m.slots.capacity == 4
+    a = m.open("a")
+    m.open("b")
+    with pytest.raises(OutOfPages, match="every request slot is taken"):
+        m.open("c")                                       # two requests at most, however many slots there are
+    assert m.step_slot("a") == a
+    m.prepare("a", 3)
+    shadow = m.step_slot("a")
+    assert shadow != a and m.slot("a") == a and m.slots.in_use == 3
+    m.abort("a")
+    assert m.slot("a") == a and m.step_slot("a") == a and m.slots.in_use == 2
+    m.prepare("a", 3)
+    shadow = m.step_slot("a")
+    m.commit("a")
+    assert m.slot("a") == shadow and m.slots.in_use == 2  # the old slot went back
+    m.prepare("a", 1)
+    m.prepare("b", 1)
+    assert len({m.step_slot("a"), m.step_slot("b"), m.slot("a"), m.slot("b")}) == 4
+    m.close("a")                                          # ending a request during its step gives both slots back
+    m.abort("b")
+    m.close("b")
+    assert m.slots.in_use == 0 and m.pages_in_use() == 0
+    with pytest.raises(OutOfPages):
+        full = CacheManager([GroupSpec("kv", 4, 1)], max_requests=1, shadow_slots=True)
+        full.open("x")
+        full.prepare("x", 9)
+    assert full.slots.in_use == 1 and full.step_slot("x") == full.slot("x")   # the failed prepare took no second slot

@@ -56,3 +56,22 @@ def test_sampling_ranges_are_checked_before_anything_is_loaded(tmp_path, capsys)
     assert rc in (1, 2) and "top_p" in err
     rc, _, err = run(["generate", str(tmp_path), "1,2", "--stop", "x"], capsys)
     assert rc == 2 and "token ids" in err
+
+
+def test_config_and_random_name_a_model_without_a_folder(tmp_path, capsys):
+    """`--config JSON --random SEED` stands in the model folder's place; the two go together and leave the prompt as
+    the only positional (the run itself needs the GPU and is tested there)."""
+    rc, _, err = run(["generate", "--config", "c.json", "1,2"], capsys)
+    assert rc == 2 and "--config and --random go together" in err
+    rc, _, err = run(["generate", "--random", "3", "m", "1,2"], capsys)
+    assert rc == 2 and "--config and --random go together" in err
+    rc, _, err = run(["generate"], capsys)
+    assert rc == 2 and "needs a model folder, or --config JSON --random SEED" in err
+    rc, _, err = run(["generate", "--config", str(tmp_path / "none.json"), "--random", "0", "1,2"], capsys)
+    assert rc == 2 and "none.json" in err
+    rc, _, err = run(["generate", "--config", "c.json", "--random", "0", "1,2", "extra"], capsys)
+    assert rc == 2 and "unexpected argument 'extra'" in err
+    bad = tmp_path / "c.json"
+    bad.write_text(json.dumps({"architectures": ["MiniMaxM3ForCausalLM"], "head_dim": 16}))
+    rc, _, err = run(["generate", "--config", str(bad), "--random", "0", "1,2"], capsys)
+    assert rc == 1 and "missing key" in err

@@ -72,11 +72,11 @@ def test_a_drawn_configuration(seed, wide, length, dtype):
     whole = engine_tests.run_whole(engine, "w", tokens)
     assert torch.isfinite(whole).all()
     # Among hundreds of rows drawn without care some router keys lie closer than float32 resolves (1e-7 apart), so in
-    # both dtypes the plain implementation takes the engine's picks, after checking each: in float32 a pick's key may
-    # lie below the plain router's k-th best by rounding only.
+    # both dtypes the plain implementation takes the engine's picks, after checking each against the engine's own router
+    # logits, and those logits against the plain ones.
     rounded = dtype == "bfloat16"
     want = helpers.plain_logits_with_picks(name, tokens, engine.observer.of("w", length), rounded=rounded,
-                                           slack=4e-3 if rounded else 1e-5)
+                                           engine_logits=engine.observer.logits_of("w", length))
     tol = engine_tests.BF16_TOL if rounded else engine_tests.F32_TOL
     err, scale = float((whole.double() - want).abs().max()), float(want.abs().max())
     assert err <= tol * scale, f"{helpers.TINY[name][0]} {dtype}: max error {err:.3e} against scale {scale:.3e}"

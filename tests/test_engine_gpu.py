@@ -23,7 +23,8 @@ F32_TOL = 2e-5
 # bfloat16: both round at the same places; what is left are float32 sums of bfloat16 products whose last-bit
 # differences flip a bfloat16 rounding (2^-8 relative) of single activations here and there.  Such a flip can also
 # turn a router's near-tie (the tiny models' closest keys lie 1e-5 apart), so in bfloat16 the plain implementation is
-# given the engine's picks, after checking that each pick's key is within rounding of the best k.
+# given the engine's picks, after checking in every row that they are the k best keys of the engine's own router logits
+# and that those logits are the plain ones within their noise (helpers.plain_logits_with_picks).
 BF16_TOL = 2e-2
 
 LENGTHS = {"A": (5, 17, 32, 75), "B": (1, 9, 23, 40, 67), "A16": (5, 17, 32, 75)}
@@ -67,7 +68,8 @@ def run_cut(engine, rid, tokens, cuts):
 
 def check_against_plain(name, dtype, length, seed, got, engine=None, rid=None):
     if dtype == "bfloat16":
-        want = plain_logits_with_picks(name, tokens_for(name, length, seed), engine.observer.of(rid, length))
+        want = plain_logits_with_picks(name, tokens_for(name, length, seed), engine.observer.of(rid, length),
+                                       engine_logits=engine.observer.logits_of(rid, length))
     else:
         want = plain_logits(name, length, seed, False)
     tol = F32_TOL if dtype == "float32" else BF16_TOL
@@ -115,11 +117,71 @@ def test_first_tokens(setup):
         tokens = tokens_for(name, 67 if name == "B" else 75, 0)[:length]
         got = run_whole(engine, "f", tokens)
         if dtype == "bfloat16":
-            want = plain_logits_with_picks(name, tokens, engine.observer.of("f", length))
+            want = plain_logits_with_picks(name, tokens, engine.observer.of("f", length), engine_logits=engine.observer.logits_of("f", length))
         else:
             want = plain_logits(name, 67 if name == "B" else 75, 0, False)[:length]
         tol = F32_TOL if dtype == "float32" else BF16_TOL
         assert float((got.double() - want).abs().max()) <= tol * float(want.abs().max())
+
+
+def test_truncate_takes_a_request_back_to_a_prefix(setup):
+    """A request is taken back to 41 of its tokens (inside a page) and goes on with other tokens: the logits are those
+    of a fresh run of the new sequence, bit for bit, and the pages beyond the prefix went back to the pool."""
+    from llmx_amd.engine import StepEntry
+    name, dtype, engine = setup
+    page = TINY[name][2]
+    length = 67 if name == "B" else 75
+    tokens, other = tokens_for(name, length, 0), tokens_for(name, length, 9)
+    joined = tokens[:41] + other[41:]
+    whole, whole_joined = run_whole(engine, "w", tokens), run_whole(engine, "w", joined)
+    every = lambda t: list(range(len(t)))
+    engine.add_request("t")
+    assert torch.equal(engine.step([StepEntry("t", tokens, every(tokens))]).cpu(), whole)
+    assert engine.cache.pages_in_use() == -(-length // page)
+    engine.truncate("t", 41)
+    assert engine.length("t") == 41 and engine.cache.pages_in_use() == -(-41 // page)
+    assert torch.equal(engine.step([StepEntry("t", other[41:], every(other[41:]))]).cpu(), whole_joined[41:])
+    engine.truncate("t", 0)
+    assert engine.cache.pages_in_use() == 0
+    assert torch.equal(engine.step([StepEntry("t", tokens[:30], every(tokens[:30]))]).cpu(), whole[:30])
+    from llmx_amd.cache import CacheLogicError
+    with pytest.raises(CacheLogicError, match="cannot be taken back to 31"):
+        engine.truncate("t", 31)
+    engine.end_request("t")
+    assert engine.cache.pages_in_use() == 0
+
+
+def test_the_router_reads_unrounded_rows_in_bfloat16():
+    """The router's logits come from the float32 normed rows, not from their bfloat16 roundings
+    (/root/reference/src/backends/backend.hpp:943-947: the router's product is F32 whatever the step's type).  Eight
+    one-token requests in one step: with a single key the softmax weight is exactly 1, so everything before the router is
+    the plain implementation's arithmetic up to the order of float32 sums, and the engine's logits can be told apart from
+    the logits a router reading rounded rows would give."""
+    import plain_model as pm
+    from helpers import INIT_B, TINY_B, plain
+    from llmx_amd.engine import StepEntry
+    helpers.TINY["B1"] = (dict(TINY_B, num_hidden_layers=1), INIT_B, 8)
+    engine = make_engine("B1", "bfloat16")
+    engine.observer = RoutingRecorder(1)
+    tokens = tokens_for("B1", 8, 3)
+    for i in range(8):
+        engine.add_request(i)
+    engine.step([StepEntry(i, [t], []) for i, t in enumerate(tokens)])
+    z_engine = torch.stack([engine.observer.logits_of(i, 1)[0][0] for i in range(8)]).double()
+    cfg, w = plain("B1")
+    bf, eps, p = torch.bfloat16, cfg["rms_norm_eps"], "model.layers.0."
+    z_wide, z_rounded = [], []
+    for t in tokens:
+        x = w["model.embed_tokens.weight"].double()[[t]]
+        x = x + pm.attention_layer(pm.rms_norm(x, w[p + "input_layernorm.weight"].double(), eps), [0], w, p + "self_attn.", cfg, bf)
+        h = pm.rms_norm(x, w[p + "post_attention_layernorm.weight"].double(), eps)
+        z_wide.append(h @ w[p + "mlp.gate.weight"].double().T)
+        z_rounded.append(pm._rounded(h, bf) @ w[p + "mlp.gate.weight"].double().T)
+    z_wide, z_rounded = torch.cat(z_wide), torch.cat(z_rounded)
+    apart = float((z_rounded - z_wide).abs().max())
+    assert apart > 1e-4 * float(z_wide.abs().max())                     # the two readings can be told apart here
+    assert float((z_engine - z_wide).abs().max()) < 0.02 * apart        # and the engine's is the unrounded one
+    assert float((z_engine - z_rounded).abs().max()) > 0.5 * apart
 
 
 MIXED_LENGTHS = [40, 23, 67, 9, 31, 52]
@@ -228,8 +290,6 @@ def test_decode_steps_replayed_as_graphs_equal_eager_steps(name, dtype):
             if i == 30:
                 eng.step([StepEntry("x", extra[33:], [36])])
                 eng.end_request("x")
-            if i == 40 and "b" in live and eng is engines[0]:
-                pass
             outs.append(eng.step([StepEntry(rid, [nxt[rid]], [0]) for rid in live]).clone())
         assert torch.equal(outs[0], outs[1]), f"step {i}: the replayed step differs from the eager one"
         picks = outs[0].argmax(dim=1).tolist()
@@ -240,6 +300,39 @@ def test_decode_steps_replayed_as_graphs_equal_eager_steps(name, dtype):
             live = ["a", "c"]
             nxt.pop("b")
     assert engines[0].graph_replays >= 40 and engines[1].graph_replays == 0
+
+
+@pytest.mark.parametrize("name,dtype,prompt_len", [("A", "bfloat16", 250), ("A16", "bfloat16", 885), ("B", "float32", 505)])
+def test_graph_replays_across_the_edges_their_key_exists_for(name, dtype, prompt_len):
+    """Decoding crosses the sizes a recorded step is keyed by: the block table's width (64 pages: 256 tokens on pages of
+    4, 512 on pages of 8), the attention plan's segment count (896 tokens, where the split contexts' partial results get
+    more slots), and scratch storage that moves because another request's larger portion ran between two replays (the
+    recorded graphs are dropped and recorded again).  Every step equals an engine that records nothing."""
+    from llmx_amd.engine import Engine, StepEntry
+    page = TINY[name][2]
+    engines = [Engine.load(model_folder(name), dtype=dtype, kv_tokens=2048, page_tokens=page, max_requests=4, graphs=g) for g in (True, False)]
+    prompt, extra = tokens_for(name, prompt_len, 21), tokens_for(name, 400, 22)
+    nxt = None
+    for eng in engines:
+        eng.add_request("a")
+        for s in range(0, prompt_len, 200):        # portions of 200: the larger portion below makes scratch storage grow
+            part = prompt[s:s + 200]
+            out = eng.step([StepEntry("a", part, [len(part) - 1])])
+        nxt = int(out.argmax(dim=1))
+    replays_before_growth = None
+    for i in range(40):
+        outs = []
+        for eng in engines:
+            if i == 20:
+                eng.add_request("x")
+                eng.step([StepEntry("x", extra, [])])
+                eng.end_request("x")
+            outs.append(eng.step([StepEntry("a", [nxt], [0])]).clone())
+        if i == 19:
+            replays_before_growth = engines[0].graph_replays
+        assert torch.equal(outs[0], outs[1]), f"step {i} (context {prompt_len + i + 1}): the replayed step differs from the eager one"
+        nxt = int(outs[0].argmax(dim=1))
+    assert replays_before_growth >= 10 and engines[0].graph_replays >= replays_before_growth + 10 and engines[1].graph_replays == 0
 
 
 def test_refusals_leave_nothing_behind(setup):

@@ -177,6 +177,29 @@ def test_command_line(tmp_path):
     assert bad.returncode == 2 and "at least 2" in bad.stderr
 
 
+def test_command_line_runs_a_configuration_with_random_weights(tmp_path):
+    """`llmx generate --config JSON --random SEED`: weights come from the seed on the device, no folder is read or
+    written; the tokens are those of an engine made from the same configuration and seed in this process."""
+    import json
+    from helpers import TINY_B
+    from llmx_amd import Engine, MiniMaxM3Config, RandomInit, SamplingParams, generate
+    cfg = MiniMaxM3Config(**TINY_B)
+    path = tmp_path / "config.json"
+    path.write_text(json.dumps(cfg.to_json()))
+    prompt = tokens_for("B", 9, 3)
+    engine = Engine.from_random(cfg, RandomInit(seed=5, std=0.05), dtype="float32", kv_tokens=64, page_tokens=8, max_requests=1)
+    want = generate(engine, [prompt], SamplingParams(max_tokens=6, temp=0.0))[0]
+    cmd = [os.path.join(ROOT, "bin", "llmx"), "generate", "--config", str(path), "--random", "5", "--std", "0.05", ",".join(map(str, prompt)),
+           "-n", "6", "--temp", "0", "--dtype", "f32", "--page-tokens", "8"]
+    run = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert run.stdout.strip().split("\n")[-1].split() == [str(t) for t in want]
+    lg = subprocess.run([os.path.join(ROOT, "bin", "llmx"), "logits", "--config", str(path), "--random", "5", "--std", "0.05",
+                         ",".join(map(str, prompt)), "--top", "1", "--dtype", "f32", "--page-tokens", "8"], capture_output=True, text=True, timeout=300)
+    assert lg.returncode == 0, lg.stderr[-2000:]
+    assert int(lg.stdout.strip().split("\n")[-1].split()[0]) == want[0]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_many_requests_through_a_small_pool_equal_their_runs_alone(dtype):
     """Thirty requests of drawn lengths, counts and settings, through pages for about three of them: requests wait for

@@ -848,7 +848,7 @@ def test_penalties():
 def test_fill_random_matches_host():
     from llmx_amd.parts.spec import TensorSpec
     from llmx_amd.weights import RandomInit, host_values
-    from llmx_amd.weights.device_init import fill_random
+    from llmx_amd.weights.random_init import fill_random
     init = RandomInit(seed=3, std=0.05, norm_std=0.1, bias_range=0.2)
     for spec in (TensorSpec("a.weight", (37, 53), "matrix"), TensorSpec("n.weight", (100,), "norm"), TensorSpec("b.bias", (64,), "bias")):
         want = host_values(spec, init)

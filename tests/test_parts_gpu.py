@@ -339,6 +339,8 @@ def define_toy_parts():
         def load(self, tensors):
             self.weight = tensors[self.name("mix.weight")]
 
+        fail_after_writing = False     # set by a test: the step dies once this layer has written its state
+
         def forward(self, step, h, out, accumulate, cache, h32=None):
             y = h32 @ self.weight.T
             result = torch.empty_like(y)
@@ -348,6 +350,8 @@ def define_toy_parts():
                     s = self.decay * s + (1.0 - self.decay) * y[r]
                     result[r] = s
                 cache.state[e.slot] = s
+            if self.fail_after_writing:
+                raise RuntimeError("the toy mixer was told to fail")
             if accumulate:
                 out += result
             else:
@@ -481,6 +485,48 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         engine.add_request("c")       # takes a slot that held state
         got = engine.step([StepEntry("c", seqs["b"], list(range(len(seqs["b"]))))]).cpu().double()
         assert (got - want["b"]).abs().max() < 2e-5 * want["b"].abs().max()
+    finally:
+        unregister_architecture("ToyHybridForCausalLM")
+        unregister("mixer", "toy_running_mean")
+
+
+def test_a_step_that_fails_leaves_the_state_as_it_found_it(tmp_path):
+    """A step in which the stateful toy mixer has already written its state raises; the next step gives the bits of an
+    engine that never failed: pages were returned and every request's state is what the last good step left."""
+    from llmx_amd import Engine, RandomInit
+    from llmx_amd.engine import StepEntry, StepError
+    from llmx_amd.models import register_architecture, unregister_architecture
+    from llmx_amd.parts import unregister
+    from llmx_amd.weights.folder import write_random_model
+    define_toy_parts()
+    register_architecture("ToyHybridForCausalLM", ToyConfig, toy_assemble, replace=True)
+    try:
+        folder = write_random_model(tmp_path / "toy", ToyConfig(), RandomInit(seed=4, std=0.2, norm_std=0.05, storage="float32"))
+        failing, steady = (Engine.load(folder, dtype="float32", kv_tokens=64, page_tokens=4, max_requests=2) for _ in range(2))
+        a, b = [3, 14, 15, 9, 2, 6, 5, 35, 8, 9, 7, 9], [2, 7, 18, 28, 18, 2, 8]
+        every = lambda t: list(range(len(t)))
+        for eng in (failing, steady):
+            eng.add_request("a")
+            eng.add_request("b")
+            eng.step([StepEntry("a", a[:5], []), StepEntry("b", b[:3], [])])
+        pages = failing.cache.pages_in_use()
+        slots = (failing.cache.slot("a"), failing.cache.slot("b"))
+        last_toy = failing.model.blocks[3].mixer
+        last_toy.fail_after_writing = True
+        with pytest.raises(RuntimeError, match="told to fail"):
+            failing.step([StepEntry("a", a[5:9], every(a[5:9])), StepEntry("b", b[3:4], [0])])
+        last_toy.fail_after_writing = False
+        assert failing.cache.pages_in_use() == pages and failing.length("a") == 5 and failing.length("b") == 3
+        assert (failing.cache.slot("a"), failing.cache.slot("b")) == slots and failing.cache.slots.in_use == 2
+        for cut in ([StepEntry("a", a[5:9], every(a[5:9])), StepEntry("b", b[3:4], [0])], [StepEntry("a", a[9:], every(a[9:])), StepEntry("b", b[4:], every(b[4:]))]):
+            assert torch.equal(failing.step(cut), steady.step(cut))
+        # a state cannot be unwound: taking a stateful request back to a prefix is refused, to nothing is allowed
+        with pytest.raises(StepError, match="keeps a state of fixed size"):
+            failing.truncate("a", 4)
+        failing.truncate("a", 0)
+        steady.end_request("a")
+        steady.add_request("a")
+        assert torch.equal(failing.step([StepEntry("a", a, every(a))]), steady.step([StepEntry("a", a, every(a))]))
     finally:
         unregister_architecture("ToyHybridForCausalLM")
         unregister("mixer", "toy_running_mean")

@@ -163,7 +163,7 @@ def test_experts():
     h = rand(7, E)
     cfg = dict(num_experts_per_tok=1, norm_topk_prob=True, routed_scaling_factor=1.7)
     w = one_layer_weights(1, E, Fe)
-    out, ids, weights, _ = pm.moe_layer(h, w, "", cfg)
+    out, ids, weights, _, _ = pm.moe_layer(h, w, "", cfg)
     gu, dn = w["experts.gate_up_proj"][0], w["experts.down_proj"][0]
     mlp = (F.silu(h @ gu[:Fe].T) * (h @ gu[Fe:].T)) @ dn.T                 # one expert, one pick: a plain SwiGLU MLP times the scale
     assert torch.allclose(out, 1.7 * mlp, rtol=1e-10)
@@ -181,7 +181,7 @@ def test_experts():
     assert torch.equal(pm.moe_layer(h, zero, "", cfg3)[0], torch.zeros(7, E, dtype=D64))   # no down projection: nothing is added
     # combine in slot order with the router's weights
     w6 = one_layer_weights(6, E, Fe)
-    out6, ids6, weights6, _ = pm.moe_layer(h, w6, "", cfg3)
+    out6, ids6, weights6, _, _ = pm.moe_layer(h, w6, "", cfg3)
     t = 2
     want = sum(weights6[t, j] * pm.swiglu_expert(h[t], w6["experts.gate_up_proj"][ids6[t, j]], w6["experts.down_proj"][ids6[t, j]]) for j in range(3))
     assert torch.allclose(out6[t], want)
@@ -225,3 +225,99 @@ def test_greedy_and_rounding():
     rounded = pm.forward(cfg, w, [5, 17, 3, 9], round_to=torch.bfloat16)
     full = pm.forward(cfg, w, [5, 17, 3, 9])
     assert 0 < (rounded - full).abs().max() < 2e-2 * full.abs().max()
+
+
+# -- points of the reading that no library routine fixes: each as an invariant a wrong reading breaks -----------------
+def _attention_cfg():
+    return dict(num_attention_heads=4, num_key_value_heads=2, head_dim=8, rotary_dim=4, rms_norm_eps=1e-6,
+                rope_parameters={"rope_theta": 1e4})
+
+
+def _attention_weights(scale=1.0):
+    E, Hq, Hkv, D = 24, 4, 2, 8
+    return {"q_proj.weight": rand(Hq * D, E) * scale, "k_proj.weight": rand(Hkv * D, E) * scale, "v_proj.weight": rand(Hkv * D, E) * scale,
+            "o_proj.weight": rand(E, Hq * D) * scale, "q_norm.weight": 1 + 0.1 * rand(Hq * D), "k_norm.weight": 1 + 0.1 * rand(Hkv * D)}
+
+
+def test_queries_and_keys_are_normed_and_values_are_not():
+    """The norm (with the rotation) is applied to the q and k rows only; v goes to the cache as projected
+    (/root/reference/src/model/arch/minimax_m3.hpp:258-259 norm q and k, :264 writes v_rows untouched).  A norm's output
+    does not change when its input is scaled, so scaling W_q or W_k changes nothing (up to eps), while the output is
+    linear in W_v: scaling W_v by c scales it by c, and W_v = 0 gives exactly 0.  Norming v as well, or forgetting the
+    norm of q or k, breaks one of the three."""
+    cfg, w = _attention_cfg(), _attention_weights()
+    h = rand(6, 24)
+    out = pm.attention_layer(h, list(range(6)), w, "", cfg)
+    for name in ("q_proj.weight", "k_proj.weight"):
+        scaled = dict(w)
+        scaled[name] = w[name] * 7.0
+        assert torch.allclose(pm.attention_layer(h, list(range(6)), scaled, "", cfg), out, rtol=1e-5, atol=1e-9), name
+    scaled = dict(w)
+    scaled["v_proj.weight"] = w["v_proj.weight"] * 7.0
+    assert torch.allclose(pm.attention_layer(h, list(range(6)), scaled, "", cfg), 7.0 * out, rtol=1e-12)
+    zero = dict(w)
+    zero["v_proj.weight"] = torch.zeros_like(w["v_proj.weight"])
+    assert torch.equal(pm.attention_layer(h, list(range(6)), zero, "", cfg), torch.zeros(6, 24, dtype=D64))
+    # the norm comes before the rotation and spans the projection: a norm weight that differs inside a rotated pair is seen
+    skew = dict(w)
+    skew["q_norm.weight"] = w["q_norm.weight"].clone()
+    skew["q_norm.weight"][0] *= 3.0
+    assert not torch.allclose(pm.attention_layer(h, list(range(6)), skew, "", cfg), out)
+
+
+def _bf16_by_hand(v: float) -> float:
+    """Round to nearest, ties to even, on the bits (/root/reference/src/core/bf16.hpp:5-11), without torch's conversion."""
+    import struct
+    u = struct.unpack("<I", struct.pack("<f", v))[0]
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return struct.unpack("<f", struct.pack("<I", u))[0]
+
+
+def test_where_the_bfloat16_path_rounds():
+    """The bfloat16 path rounds the inputs of weight products and what the cache stores, nothing else: sums, norms, the
+    softmax, the router's logits and the residual stay wide (/root/reference/src/backends/backend.hpp:943-962: the
+    router's product is F32 whatever the step's dtype, the experts' three products read their inputs in the step's dtype
+    and sum in F32).  Each site is fixed by a vector whose rounding is worked out by hand on the bits."""
+    bf = torch.bfloat16
+    # the expert's activation is rounded once, before the down product; the sums are not rounded
+    h = torch.tensor([3.0], dtype=D64)                       # exact in bfloat16: the caller has rounded it
+    one = torch.ones(1, 1, dtype=D64)
+    a = (3.0 / (1.0 + math.exp(-3.0))) * 3.0                 # silu(3) * 3 = 8.5731...
+    y = pm.swiglu_expert(h, torch.cat([one, one]), one * 1.5, bf)
+    assert float(y) == _bf16_by_hand(a) * 1.5 and float(y) != a * 1.5
+    assert float(pm.swiglu_expert(h, torch.cat([one, one]), one * 1.5)) == pytest.approx(a * 1.5, rel=1e-15)
+    # the layer rounds the rows the experts read and leaves the rows the router reads: a change below half a unit of
+    # bfloat16's last place moves the router's logits and keys, and leaves every expert's output bit for bit
+    E, X, Fi = 16, 4, 8
+    cfg = dict(num_experts_per_tok=2, norm_topk_prob=False, routed_scaling_factor=1.0)
+    w = {"gate.weight": rand(X, E), "gate.e_score_correction_bias": torch.zeros(X, dtype=D64),
+         "experts.gate_up_proj": rand(X, 2 * Fi, E), "experts.down_proj": rand(X, E, Fi)}
+    h = pm._rounded(rand(5, E), bf)
+    nudged = h * (1.0 + 2.0 ** -11)                          # a quarter of a unit in the last place: rounds back to h
+    assert torch.equal(pm._rounded(nudged, bf), h)
+    base = pm.moe_layer(h, w, "", cfg, bf)
+    moved = pm.moe_layer(nudged, w, "", cfg, bf, picks=base[1])
+    assert not torch.equal(moved[4], base[4]) and torch.allclose(moved[4], base[4] * (1.0 + 2.0 ** -11), rtol=1e-12)   # the router saw it
+    same_weights = pm.moe_layer(nudged, {**w, "gate.weight": torch.zeros(X, E, dtype=D64)}, "", cfg, bf, picks=base[1])[0]
+    flat = pm.moe_layer(h, {**w, "gate.weight": torch.zeros(X, E, dtype=D64)}, "", cfg, bf, picks=base[1])[0]
+    assert torch.equal(same_weights, flat)                   # with equal weights the experts' sum is the same bits: they read rounded rows
+    # attention: the projections read rounded rows (a nudge below rounding changes nothing at all), and q, k, v and the
+    # attention output are rounded where they are stored, so the layer's result differs from the wide one
+    acfg, aw = _attention_cfg(), {k: pm._rounded(v, bf) for k, v in _attention_weights(0.3).items()}
+    h = pm._rounded(rand(4, 24), bf)
+    assert torch.equal(pm.attention_layer(h * (1.0 + 2.0 ** -11), [0, 1, 2, 3], aw, "", acfg, bf), pm.attention_layer(h, [0, 1, 2, 3], aw, "", acfg, bf))
+    assert not torch.equal(pm.attention_layer(h * (1.0 + 2.0 ** -11), [0, 1, 2, 3], aw, "", acfg), pm.attention_layer(h, [0, 1, 2, 3], aw, "", acfg))
+    # one key: the softmax weight is 1 and the layer's output is o_proj applied to the rounded v row, rounded again as
+    # the attention output: worked out by hand for one element
+    one_row = pm.attention_layer(h[:1], [0], aw, "", acfg, bf)
+    v_row = [_bf16_by_hand(float(x)) for x in (h[:1] @ aw["v_proj.weight"].T)[0]]
+    heads_v = torch.tensor([v_row[8 * (hq // 2) + d] for hq in range(4) for d in range(8)], dtype=D64)   # head hq reads KV head hq // 2
+    assert torch.allclose(one_row[0], heads_v @ aw["o_proj.weight"].T, rtol=1e-12)
+    # the whole model: the final norm's rows are rounded before the head, the residual never is
+    cfg_a, w_a = plain("A")
+    tokens = [5, 17, 3]
+    x = w_a["model.embed_tokens.weight"].double()[tokens]
+    w0 = {k: (torch.zeros_like(v) if k.endswith("o_proj.weight") or k.endswith("experts.down_proj") else v) for k, v in w_a.items()}
+    rows = pm.rms_norm(x, w_a["model.norm.weight"].double(), cfg_a["rms_norm_eps"])
+    want = torch.tensor([[_bf16_by_hand(float(v)) for v in r] for r in rows], dtype=D64) @ w_a["lm_head.weight"].double().T
+    assert torch.allclose(pm.forward(cfg_a, w0, tokens, round_to=bf), want, rtol=1e-12)

@@ -1,0 +1,81 @@
+"""Refusals that must come before anything is reserved or allocated: kernel size limits when a model is read or
+built, a step's own rules when it is submitted, and a kernel library built from other sources."""
+
+import pytest
+import torch
+
+from helpers import TINY_A
+from llmx_amd import ConfigError, MiniMaxM3Config
+from llmx_amd.cache import CacheManager, GroupSpec
+from llmx_amd.engine.batch import StepEntry, StepError, check_entries
+from llmx_amd.limits import MAX_EXPERTS, MAX_HEAD_DIM, MAX_STEP_ROWS, MAX_TOP_K
+from llmx_amd.parts.base import BuildContext, build_part
+from llmx_amd.parts.spec import PartSpec
+
+
+@pytest.mark.parametrize("change,text", [
+    (dict(head_dim=272, rotary_dim=8), f"head_dim .272 is above the attention kernels' limit of {MAX_HEAD_DIM}"),
+    (dict(num_local_experts=1025), f"num_local_experts .1025 is above the routing kernels' limit of {MAX_EXPERTS}"),
+    (dict(num_local_experts=512, num_experts_per_tok=257), f"num_experts_per_tok .*above the kernels' limit of {MAX_TOP_K}"),
+])
+def test_a_configuration_beyond_a_kernel_limit_is_refused_when_read(change, text):
+    with pytest.raises(ConfigError, match=text):
+        MiniMaxM3Config(**{**TINY_A, **change})
+
+
+def test_parts_refuse_sizes_their_kernels_do_not_take():
+    """The same limits hold for a part built by any architecture: they belong to the part, not to a configuration."""
+    ctx = BuildContext(torch.float32, torch.device("cpu"), 64)
+    with pytest.raises(ValueError, match=f"head_dim 320 is outside what the attention kernels take .1 to {MAX_HEAD_DIM}."):
+        build_part("mixer", PartSpec("attention", {"hidden": 64, "heads": 2, "kv_heads": 1, "head_dim": 320}), ctx)
+    with pytest.raises(ValueError, match=f"2048 experts with 8 picks a token; the routing kernels take at most {MAX_EXPERTS} experts and {MAX_TOP_K} picks"):
+        build_part("feed_forward", PartSpec("routed_experts", {"hidden": 64, "experts": 2048, "top_k": 8, "intermediate": 32}), ctx)
+    with pytest.raises(ValueError, match="300 picks a token"):
+        build_part("feed_forward", PartSpec("routed_experts", {"hidden": 64, "experts": 512, "top_k": 300, "intermediate": 32}), ctx)
+
+
+def test_step_refusals_by_text_and_nothing_reserved():
+    cache = CacheManager([GroupSpec("kv", 4, 8)], max_requests=2)
+    cache.open("a")
+    cache.open("b")
+    ok = StepEntry("a", [1, 2, 3], [2])
+    cases = [
+        ([], "an empty batch"),
+        ([ok, StepEntry("a", [4])], "request 'a' appears twice"),
+        ([StepEntry("zz", [1])], "request 'zz' is not open"),
+        ([StepEntry("a", [])], "brings no tokens"),
+        ([StepEntry("a", list(range(40)))], "context length exceeded: request 'a' would hold 40 tokens of 32"),
+        ([StepEntry("a", [1, 50])], "token id 50 is outside the embedding's rows"),
+        ([StepEntry("a", [1, -1])], "token id -1 is outside"),
+        ([StepEntry("a", [1, 2], [2])], "wants the logits of place 2 among 2 tokens"),
+    ]
+    for entries, text in cases:
+        with pytest.raises(StepError, match=text):
+            check_entries(entries, cache, 32, 50)
+    views = check_entries([ok, StepEntry("b", [7], [0])], cache, 32, 50)
+    assert [(v.row0, v.n, v.past) for v in views] == [(0, 3, 0), (3, 1, 0)]
+    assert cache.pages_in_use() == 0
+    # more rows than a step takes: refused as a step error, before any page is asked for
+    big = CacheManager([GroupSpec("kv", 64, 4096)], max_requests=2)
+    big.open("a")
+    big.open("b")
+    with pytest.raises(StepError, match=f"{MAX_STEP_ROWS + 1} token rows in one step; a step takes at most {MAX_STEP_ROWS}"):
+        check_entries([StepEntry("a", [0] * MAX_STEP_ROWS), StepEntry("b", [0])], big, 1 << 20, 50)
+    assert big.pages_in_use() == 0
+
+
+def test_a_library_built_from_other_sources_is_built_again(tmp_path, monkeypatch):
+    from llmx_amd.csrc import build
+    lib = tmp_path / build.LIB_NAME
+    lib.write_bytes(b"old")
+    stamp = tmp_path / (build.LIB_NAME + ".stamp")
+    built = []
+    monkeypatch.setattr(build, "lib_candidates", lambda: [lib])
+    monkeypatch.setattr(build, "build", lambda verbose=True: built.append(1) or lib)
+    stamp.write_text(build._stamp())
+    assert build.load_path(verbose=False) == lib and not built          # current: taken as it is
+    stamp.write_text("something else")
+    assert build.load_path(verbose=False) == lib and built == [1]       # stale: compiled again, not used with a warning
+    stamp.unlink()
+    build.load_path(verbose=False)
+    assert built == [1, 1]                                              # no stamp at all counts as stale

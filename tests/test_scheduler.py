@@ -158,3 +158,42 @@ def test_random_loads_finish_and_return_everything(seed):
     assert cache.pages_in_use() == 0 and cache.slots.in_use == 0 and s.reserved == [0]
     assert all(len({e.request for e in p}) == len(p) for p in plans)                     # a request at most once a step
     assert all(sum(len(e.tokens) for e in p) <= s.max_step_tokens for p in plans)
+
+
+def test_the_last_token_the_limit_allows_is_fed_without_logits():
+    """At max_tokens the last token goes into the cache in the next step (no logits wanted) and then the request ends;
+    an end token and a token completing a stop sequence are never fed (/root/reference/src/inference/generate.hpp:28-45)."""
+    groups = [GroupSpec("kv", 4, 100)]
+    cache = CacheManager(groups, max_requests=3)
+    s = Scheduler(groups, 3, 16, eos_token_id=EOS)
+    s.submit(Request("len", [1, 2, 3], greedy(2)))
+    s.submit(Request("eos", [1, 2, 3], greedy(5)))
+    s.submit(Request("stop", [1, 2, 3], SamplingParams(max_tokens=5, temp=0.0, stop=(5, 5))))
+    held = {}
+
+    def token_for(r, i):
+        return EOS if (r.id == "eos" and i == 1) else 5
+
+    plans = []
+    while not s.idle:
+        for r in s.admit():
+            cache.open(r.id)
+        plan = s.plan()
+        by_id = {r.id: r for r in s.running}
+        for e in plan:
+            cache.prepare(e.request, len(e.tokens))
+            cache.commit(e.request)
+        done = s.advance(plan, {e.request: token_for(by_id[e.request], len(by_id[e.request].generated)) for e in plan if e.wants_logits})
+        for r in done:
+            held[r.id] = cache.length(r.id)
+            cache.close(r.id)
+        plans.append([(e.request, list(e.tokens), e.wants_logits) for e in plan])
+    assert plans[2] == [("len", [5], False)]                 # step 0: prompts, step 1: second tokens, step 2: the fed last token
+    assert s.finished["len"].generated == [5, 5] and held["len"] == 3 + 2       # the cache held the whole reply
+    assert s.finished["eos"].generated == [5] and held["eos"] == 3 + 1          # the end token was neither kept nor fed
+    assert s.finished["stop"].generated == [5, 5] and held["stop"] == 3 + 1     # the completing token was kept, not fed
+    assert s.reserved == [0] and cache.pages_in_use() == 0
+    # without the feed the request ends with the step that drew its last token
+    s = Scheduler(groups, 1, 16, feed_last=False)
+    s.submit(Request("a", [1, 2, 3], greedy(2)))
+    assert len(run(s)) == 2
