@@ -717,7 +717,8 @@ __global__ void __launch_bounds__(512) gemm_wide_kernel(TileArgs g) {
     }
 }
 
-// form: which kernel takes the product.  The lean forms need whole 64-wide tiles of K and runs that end on them.
+// form: which kernel takes the product.  The lean forms need whole 64-wide tiles of K, runs that end on them, and
+// operands whose byte offsets fit 32 bits (llmx_gemm_tile_offsets_fit).
 enum : int { FORM_64 = 0, FORM_128 = 1, FORM_WIDE = 2, FORM_BOUNDED = 3 };
 
 template <int EPI, typename TC, bool GROUPED, bool SPLIT>
@@ -755,6 +756,16 @@ static int tile_launch_typed(const TileArgs& g, int form, dim3 grid, bool groupe
     return 0;
 }
 
+// The lean forms keep each thread's places in A and in a group's W as 32-bit byte offsets from a base the whole wave
+// shares.  Whether every such offset fits: the last row of a group's weights (2 N rows under SwiGLU) and the last row of
+// A that can be read.  Host arithmetic only; products that do not fit take the bounded form, which carries pointers.
+extern "C" int llmx_gemm_tile_offsets_fit(int M, int N, int K, int lda, int epi, int n_groups, int a_div, int up_offset) {
+    const size_t w_rows = (size_t)N + (epi == TL_SWIGLU ? (size_t)up_offset : 0);
+    const size_t a_rows = n_groups > 0 ? ((size_t)M + (a_div > 0 ? a_div : 1) - 1) / (a_div > 0 ? a_div : 1) : (size_t)M;
+    const size_t limit = (size_t)1 << 32;
+    return w_rows * (size_t)K * sizeof(bf16_t) < limit && a_rows * (size_t)lda * sizeof(bf16_t) < limit ? 1 : 0;
+}
+
 static int form_rows(int form) { return form == FORM_64 || form == FORM_BOUNDED ? 64 : 128; }
 static int form_feats(int form, int epi) { return (epi == TL_SWIGLU ? 64 : 128) * (form == FORM_WIDE ? 2 : 1); }
 
@@ -777,7 +788,7 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
     const bool grouped = n_groups > 0;
     if (ks != 1 && ks != 2 && ks != 4 && ks != 8) return -2;
     const int steps = (K + 31) / 32, per = (steps + ks - 1) / ks;
-    const bool lean = K % TL_BK == 0 && (ks == 1 || per % 2 == 0);
+    const bool lean = K % TL_BK == 0 && (ks == 1 || per % 2 == 0) && llmx_gemm_tile_offsets_fit(M, N, K, lda, epi, n_groups, a_div, up_offset);
     TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
                w_group_stride, up_offset, 0, ks, 64, nullptr, 0};
     auto launch = [&](int form, int tiles_y) -> int {

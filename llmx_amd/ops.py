@@ -70,6 +70,7 @@ def _declare(h) -> None:
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
         "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P],
         "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P],
+        "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],

@@ -79,3 +79,29 @@ def test_a_library_built_from_other_sources_is_built_again(tmp_path, monkeypatch
     stamp.unlink()
     build.load_path(verbose=False)
     assert built == [1, 1]                                              # no stamp at all counts as stale
+
+
+def test_tiled_products_whose_offsets_pass_32_bits_leave_the_lean_forms():
+    """The lean tiled kernels address A and a group's W by 32-bit byte offsets; the launcher must see when a product does
+    not fit and take the form that carries pointers (host arithmetic of the built library, no GPU needed)."""
+    import ctypes
+    from llmx_amd.csrc import build
+    from llmx_amd.ops import EPI_STORE, EPI_SWIGLU
+    h = ctypes.CDLL(str(build.load_path(verbose=False)))
+    fit = h.llmx_gemm_tile_offsets_fit
+    fit.argtypes = [ctypes.c_int] * 8
+    fit.restype = ctypes.c_int
+    # the served shapes fit: the head (200,064 x 3,072), an expert's gate and up rows, a prompt's 16,384 pairs
+    assert fit(2048, 200064, 3072, 3072, EPI_STORE, 0, 1, 0) == 1
+    assert fit(16384, 1536, 3072, 3072, EPI_SWIGLU, 256, 8, 1536) == 1
+    assert fit(16384, 3072, 1536, 1536, EPI_STORE, 256, 1, 0) == 1
+    # W of 4 GiB and more does not: N * K * 2 bytes at the edge
+    assert fit(64, 524288, 4096, 4096, EPI_STORE, 0, 1, 0) == 0          # exactly 2^32 bytes
+    assert fit(64, 524287, 4096, 4096, EPI_STORE, 0, 1, 0) == 1
+    assert fit(64, 262144, 4096, 4096, EPI_SWIGLU, 4, 1, 262144) == 0    # gate and up rows together
+    assert fit(64, 262143, 4096, 4096, EPI_SWIGLU, 4, 1, 262144) == 1
+    # A: rows * lda * 2 bytes; grouped products read row pair / a_div
+    assert fit(65536, 128, 32768, 32768, EPI_STORE, 0, 1, 0) == 0
+    assert fit(65535, 128, 32768, 32768, EPI_STORE, 0, 1, 0) == 1
+    assert fit(8 * 65536, 128, 32768, 32768, EPI_STORE, 16, 8, 0) == 0
+    assert fit(8 * 65535, 128, 32768, 32768, EPI_STORE, 16, 8, 0) == 1
