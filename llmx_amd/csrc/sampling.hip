@@ -485,3 +485,251 @@ extern "C" int llmx_sample_topk(const float* scores, const float* temp, const in
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n);
     return LLMX_CHECK_LAUNCH();
 }
+
+// ---------------------------------------------------------------------------
+// The same sampler for kept sets of any size: top-k above SAMPLE_MAX_KEEP, and top-p over the whole row (sampler.hpp:149-252
+// ranks as far as the nucleus reaches; :293-378 the draw).  Nothing is sorted.  A token's place in the ranking is the
+// reference's rank key (:76-82): the score's ordered bits above the complemented id, so keys are distinct and a larger
+// key is a better token.  "The first token, best first, at which the running weight reaches a goal" is found by
+// histograms over the keys' range: 2,048 buckets of equal width take the tokens' weights, a scan from the top finds the
+// bucket in which the goal is reached, and the search goes on inside that bucket's range until it holds at most 1,024
+// tokens, which are ranked in LDS and walked by one thread.  Weights are exp((score - best) / temp) as 64-bit fixed-point
+// numbers (w * 2^SCALE, SCALE chosen so that a row's sum fits): integer sums do not depend on the order in which they
+// are formed, so a draw does not depend on how the atomics land.  A weight below 2^-SCALE (2^-44 for rows of up to
+// 2^18 tokens) counts as 0; the reference sums doubles.
+#define RANKED_BUCKETS 2048
+#define RANKED_CAP 1024
+
+struct RankedShared {
+    unsigned long long hist_q[RANKED_BUCKETS];
+    int hist_c[RANKED_BUCKETS];
+    unsigned long long g_key[RANKED_CAP], g_q[RANKED_CAP];
+    int order[RANKED_CAP];
+    unsigned long long wave_q[SAMPLE_WAVES];
+    int wave_c[SAMPLE_WAVES];
+    unsigned long long found_key, found_before, lo, hi, goal;
+    int found_bucket, found_count, gathered, found_rank;
+};
+
+__device__ __forceinline__ unsigned long long rank_key(float score, int id) {
+    return ((unsigned long long)ordered_bits(score) << 32) | (unsigned long long)(0xFFFFFFFFu - (uint32_t)id);
+}
+
+// Sum of one value per thread over the block (integers: the order does not matter); every thread gets it.
+__device__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* scratch) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+    __syncthreads();
+    unsigned long long all = 0;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) all += scratch[w];
+    __syncthreads();
+    return all;
+}
+__device__ unsigned long long block_max_u64(unsigned long long v, unsigned long long* scratch) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = __shfl_xor(v, o, 64);
+        v = other > v ? other : v;
+    }
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+    __syncthreads();
+    unsigned long long all = 0;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) all = scratch[w] > all ? scratch[w] : all;
+    __syncthreads();
+    return all;
+}
+
+// The first token, largest key first, at which the running sum of weight(i) over the tokens with key(i) in [lo, hi]
+// reaches `goal` (>= 1).  key(i) returns 0 for a token that takes no part (no key is 0: the low half holds ~id).
+// Returns true and sets *at_key to its key and *before to the running sum before it; false when the sum stays below
+// the goal.  Every thread of the block calls it with the same arguments and gets the same answer.
+template <typename KeyFn, typename WeightFn>
+__device__ bool ranked_find(int n, KeyFn key, WeightFn weight, unsigned long long lo, unsigned long long hi, unsigned long long goal,
+                            RankedShared& sh, unsigned long long* at_key, unsigned long long* before) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    unsigned long long passed = 0;   // weight of the tokens above the present range
+    for (;;) {
+        int shift = 0;
+        while (((hi - lo) >> shift) >= RANKED_BUCKETS) ++shift;
+        for (int b = tid; b < RANKED_BUCKETS; b += SAMPLE_THREADS) {
+            sh.hist_q[b] = 0;
+            sh.hist_c[b] = 0;
+        }
+        if (tid == 0) {
+            sh.found_bucket = -1;
+            sh.gathered = 0;
+        }
+        __syncthreads();
+        for (int i = tid; i < n; i += SAMPLE_THREADS) {
+            const unsigned long long k = key(i);
+            if (k < lo || k > hi || k == 0) continue;
+            const int b = (int)((k - lo) >> shift);
+            const unsigned long long q = weight(i);
+            if (q) atomicAdd(&sh.hist_q[b], q);
+            atomicAdd(&sh.hist_c[b], 1);
+        }
+        __syncthreads();
+        // scan from the top bucket down: thread t holds buckets top - 2t and top - 2t - 1
+        const int b1 = RANKED_BUCKETS - 1 - 2 * tid, b0 = b1 - 1;
+        const unsigned long long q1 = sh.hist_q[b1], q0 = sh.hist_q[b0];
+        unsigned long long incl = q1 + q0;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const unsigned long long up = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += up;
+        }
+        if (lane == 63) sh.wave_q[wave] = incl;
+        __syncthreads();
+        unsigned long long excl = incl - (q1 + q0);
+        for (int w = 0; w < wave; ++w) excl += sh.wave_q[w];
+        const unsigned long long need = goal - passed;   // what is left to reach inside the range
+        if (excl < need && need <= excl + q1) {
+            sh.found_bucket = b1;
+            sh.found_before = excl;
+        } else if (excl + q1 < need && need <= excl + q1 + q0) {
+            sh.found_bucket = b0;
+            sh.found_before = excl + q1;
+        }
+        __syncthreads();
+        const int fb = sh.found_bucket;
+        if (fb < 0) return false;
+        passed += sh.found_before;
+        const int count = sh.hist_c[fb];
+        lo = lo + ((unsigned long long)fb << shift);
+        const unsigned long long bucket_hi = lo + ((1ull << shift) - 1ull);
+        hi = bucket_hi < hi ? bucket_hi : hi;
+        __syncthreads();
+        if (count > RANKED_CAP) continue;   // the range has shrunk by at least 1,024 times; go on inside it
+        // the bucket's tokens into LDS (in any order), ranked by key, walked by one thread
+        for (int i = tid; i < n; i += SAMPLE_THREADS) {
+            const unsigned long long k = key(i);
+            if (k < lo || k > hi || k == 0) continue;
+            const int at = atomicAdd(&sh.gathered, 1);
+            sh.g_key[at] = k;
+            sh.g_q[at] = weight(i);
+        }
+        __syncthreads();
+        for (int r = tid; r < count; r += SAMPLE_THREADS) {
+            const unsigned long long mine = sh.g_key[r];
+            int better = 0;
+            for (int j = 0; j < count; ++j) better += sh.g_key[j] > mine;
+            sh.order[better] = r;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            unsigned long long acc = passed;
+            sh.found_rank = -1;
+            for (int r = 0; r < count; ++r) {
+                const int at = sh.order[r];
+                if (acc + sh.g_q[at] >= goal) {
+                    sh.found_rank = r;
+                    sh.found_key = sh.g_key[at];
+                    sh.found_before = acc;
+                    break;
+                }
+                acc += sh.g_q[at];
+            }
+        }
+        __syncthreads();
+        if (sh.found_rank < 0) return false;   // cannot happen: the bucket's sum reaches the goal
+        *at_key = sh.found_key;
+        *before = sh.found_before;
+        __syncthreads();
+        return true;
+    }
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const float* __restrict__ scores, const float* __restrict__ temp,
+                                                                      const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                                                      const float* __restrict__ min_p, const float* __restrict__ unit,
+                                                                      const int* __restrict__ skip, int* __restrict__ out, int n) {
+    __shared__ RankedShared sh;
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float* s = scores + (size_t)r * n;
+    const int sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
+    const int m = sk < n ? n - 1 : n;
+    int keep = top_k[r];
+    if (keep <= 0 || keep > m) keep = m;
+    const float tmp = temp[r], p = top_p[r], cut = min_p ? min_p[r] : 0.0f;
+    if (!(tmp > 0.0f)) return;   // a greedy row is not this kernel's: its entry of `out` is not written
+    const unsigned long long all_lo = 1ull, all_hi = ~0ull;
+    auto key_of = [&](int i) -> unsigned long long { return i == sk ? 0ull : rank_key(s[i], i); };
+
+    // the best token: the largest key
+    unsigned long long top = 0;
+    for (int i = tid; i < n; i += SAMPLE_THREADS) {
+        const unsigned long long k = key_of(i);
+        top = k > top ? k : top;
+    }
+    top = block_max_u64(top, sh.wave_q);
+    const int best = (int)(0xFFFFFFFFu - (uint32_t)top);
+    const float best_score = s[best];
+    // fixed-point weights: a row's sum stays below 2^62
+    int scale_bits = 62;
+    while ((1ll << (62 - scale_bits)) < (long long)n) --scale_bits;
+    const double scale = (double)(1ull << scale_bits);
+    auto weight_of = [&](int i) -> unsigned long long { return (unsigned long long)((double)expf((s[i] - best_score) / tmp) * scale); };
+    auto cut_weight_of = [&](int i) -> unsigned long long {
+        const float w = expf((s[i] - best_score) / tmp);
+        return w < cut ? 0ull : (unsigned long long)((double)w * scale);
+    };
+
+    // the kept set: the `keep` largest keys, that is every key from the keep-th largest up
+    unsigned long long kept_from = all_lo, unused;
+    if (keep < m) {
+        auto one = [&](int) -> unsigned long long { return 1ull; };
+        if (!ranked_find(n, key_of, one, all_lo, all_hi, (unsigned long long)keep, sh, &kept_from, &unused)) kept_from = all_lo;
+    }
+    auto kept_key = [&](int i) -> unsigned long long {
+        const unsigned long long k = key_of(i);
+        return k >= kept_from ? k : 0ull;
+    };
+
+    int pick = best;
+    if (p >= 1.0f) {
+        // no nucleus: the draw walks the kept tokens in id order, weights below min_p counting 0 (sampler.hpp:341-352)
+        unsigned long long mine = 0;
+        for (int i = tid; i < n; i += SAMPLE_THREADS)
+            if (kept_key(i)) mine += cut_weight_of(i);
+        const unsigned long long total = block_sum_u64(mine, sh.wave_q);
+        const unsigned long long goal = (unsigned long long)floor((double)unit[r] * (double)total) + 1ull;
+        auto id_order = [&](int i) -> unsigned long long { return kept_key(i) ? (unsigned long long)(0xFFFFFFFFu - (uint32_t)i) + 1ull : 0ull; };
+        unsigned long long at = 0;
+        if (ranked_find(n, id_order, cut_weight_of, all_lo, 1ull << 32, goal, sh, &at, &unused)) pick = (int)(0xFFFFFFFFu - (uint32_t)(at - 1ull));
+    } else {
+        // the nucleus: the shortest ranked prefix of the kept set whose weight reaches top_p of the kept weight (:354-363)
+        unsigned long long mine = 0;
+        for (int i = tid; i < n; i += SAMPLE_THREADS)
+            if (kept_key(i)) mine += weight_of(i);
+        const unsigned long long total = block_sum_u64(mine, sh.wave_q);
+        unsigned long long goal = (unsigned long long)ceil((double)p * (double)total);
+        if (goal < 1ull) goal = 1ull;   // the nucleus holds at least the best token
+        unsigned long long nucleus_from = kept_from;
+        if (!ranked_find(n, kept_key, weight_of, all_lo, all_hi, goal, sh, &nucleus_from, &unused)) nucleus_from = kept_from;
+        // min_p cuts the nucleus' tail: weights fall along the ranking, so that is every weight below it (:364-372)
+        auto nucleus_key = [&](int i) -> unsigned long long {
+            const unsigned long long k = key_of(i);
+            if (k < nucleus_from) return 0ull;
+            return (cut > 0.0f && expf((s[i] - best_score) / tmp) < cut) ? 0ull : k;
+        };
+        mine = 0;
+        for (int i = tid; i < n; i += SAMPLE_THREADS)
+            if (nucleus_key(i)) mine += weight_of(i);
+        const unsigned long long nucleus_weight = block_sum_u64(mine, sh.wave_q);
+        const unsigned long long target = (unsigned long long)floor((double)unit[r] * (double)nucleus_weight) + 1ull;
+        unsigned long long at = 0;
+        if (ranked_find(n, nucleus_key, weight_of, all_lo, all_hi, target, sh, &at, &unused)) pick = (int)(0xFFFFFFFFu - (uint32_t)at);
+    }
+    if (tid == 0) out[r] = pick;
+}
+
+// Rows with any top_k (0 or above the row keeps every token) and any top_p; the sampler sends here the rows that
+// llmx_sample_topk (kept sets of at most 1,024, ranked exactly) and llmx_sample_all (everything kept, no nucleus) do not take.
+extern "C" int llmx_sample_ranked(const float* scores, const float* temp, const int* top_k, const float* top_p, const float* min_p,
+                                  const float* unit, const int* skip, int* out, int rows, int n, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (n <= 0 || n > (1 << 30)) return -2;
+    hipLaunchKernelGGL(sample_ranked_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n);
+    return LLMX_CHECK_LAUNCH();
+}

@@ -73,6 +73,7 @@ def _declare(h) -> None:
         "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
+        "llmx_sample_ranked": [P, P, P, P, P, P, P, P, I, I, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
     }
     for name, args in sigs.items():
@@ -533,6 +534,17 @@ def sample_topk(scores: torch.Tensor, temp: torch.Tensor, top_k: torch.Tensor, t
                                   _dev(min_p, "min_p", torch.float32, (rows,)), _dev(unit, "unit", torch.float32, (rows,)),
                                   _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()),
            "sample_topk")
+
+
+def sample_ranked(scores: torch.Tensor, temp: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,
+                  unit: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Tensor] = None) -> None:
+    """Top-k of any size (0 keeps all), top-p, min-p and the draw, without sorting; rows with temp <= 0 are left unwritten."""
+    rows, n = scores.shape
+    _check(lib().llmx_sample_ranked(_dev(scores, "scores", torch.float32), _dev(temp, "temp", torch.float32, (rows,)),
+                                    _dev(top_k, "top_k", torch.int32, (rows,)), _dev(top_p, "top_p", torch.float32, (rows,)),
+                                    _dev(min_p, "min_p", torch.float32, (rows,)), _dev(unit, "unit", torch.float32, (rows,)),
+                                    _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()),
+           "sample_ranked")
 
 
 def penalize(scores: torch.Tensor, rows: torch.Tensor, ids: torch.Tensor, counts: torch.Tensor, penalty: torch.Tensor,

@@ -1,8 +1,8 @@
 """Sampling: settings, per-request generators, and the device sampler."""
 
-from .params import MAX_DEVICE_TOP_K, SamplingParams, XorShift64
+from .params import MAX_EXACT_TOP_K, SamplingParams, XorShift64
 
-__all__ = ["MAX_DEVICE_TOP_K", "SamplingParams", "XorShift64", "Sampler"]
+__all__ = ["MAX_EXACT_TOP_K", "SamplingParams", "XorShift64", "Sampler"]
 
 
 def __getattr__(name):

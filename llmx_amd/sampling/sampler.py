@@ -14,7 +14,7 @@ import numpy as np
 import torch
 
 from .. import ops
-from .params import SamplingParams, XorShift64
+from .params import MAX_EXACT_TOP_K, SamplingParams, XorShift64
 
 
 class Sampler:
@@ -63,15 +63,25 @@ class Sampler:
         min_p = self._f32([p.min_p for p in params])
         # ids a draw can give: all, less a masked end token; a top_k that leaves them all is no top_k
         m = [self.vocab - (1 if (eos is not None and p.ignore_eos and 0 <= eos < self.vocab and self.vocab > 1) else 0) for p in params]
-        all_kept = [p.greedy or ((p.top_k <= 0 or p.top_k >= mr) and p.top_p >= 1.0) for p, mr in zip(params, m)]
-        if all(all_kept):
+        # which kernel takes a row: everything kept and no nucleus: the walk over the whole row; a top-k of at most
+        # MAX_EXACT_TOP_K: ranked whole in LDS; anything else (a larger top-k, a nucleus over the whole row): the search
+        # by histograms.  With mixed settings each kernel in use runs over all rows and a row takes the result of its own.
+        def kernel_of(p, mr):
+            if p.greedy or ((p.top_k <= 0 or p.top_k >= mr) and p.top_p >= 1.0):
+                return "all"
+            return "topk" if 0 < p.top_k <= MAX_EXACT_TOP_K else "ranked"
+        which = [kernel_of(p, mr) for p, mr in zip(params, m)]
+        results = {}
+        if "all" in which:
             ops.sample_all(logits, temp, unit, out, min_p, skip)
-            return out.tolist()
-        # mixed settings: both kernels run over all rows and each row takes the result of its own
-        top = torch.empty(W, dtype=torch.int32, device=self.device)
-        ops.sample_topk(logits, temp, self._i32([p.top_k for p in params]), self._f32([p.top_p for p in params]), min_p, unit, top, skip)
-        if any(all_kept):
-            ops.sample_all(logits, temp, unit, out, min_p, skip)
-            picks_all, picks_top = out.tolist(), top.tolist()
-            return [a if k else t for a, t, k in zip(picks_all, picks_top, all_kept)]
-        return top.tolist()
+            results["all"] = out
+        if "topk" in which or "ranked" in which:
+            top_k, top_p = self._i32([p.top_k for p in params]), self._f32([p.top_p for p in params])
+            for name, kernel in (("topk", ops.sample_topk), ("ranked", ops.sample_ranked)):
+                if name in which:
+                    results[name] = torch.zeros(W, dtype=torch.int32, device=self.device)
+                    kernel(logits, temp, top_k, top_p, min_p, unit, results[name], skip)
+        if len(results) == 1:
+            return next(iter(results.values())).tolist()
+        lists = {name: t.tolist() for name, t in results.items()}
+        return [lists[name][row] for row, name in enumerate(which)]

@@ -793,6 +793,70 @@ def test_samplers_match_reference_draw_for_draw(V):
             assert got == want, f"draw {draw}, row {r} ({s}): device {got}, reference {want}"
 
 
+@pytest.mark.parametrize("V,draws", [(320, 25), (5000, 25), (200064, 6)])
+def test_ranked_sampler_matches_reference_draw_for_draw(V, draws):
+    """Kept sets of any size: a nucleus over the whole row (top_k 0), top-k above 1,024, with and without min_p and a
+    masked id; rows of quantized logits, where many scores tie and the lower id must rank first; and small kept sets,
+    where the search by histograms must give what the kernel that ranks them whole gives."""
+    o = ops()
+    from llmx_amd.sampling import XorShift64
+    settings = [dict(temp=0.8, top_k=0, top_p=0.9, min_p=0.0), dict(temp=1.0, top_k=5000, top_p=1.0, min_p=0.0),
+                dict(temp=1.5, top_k=5000, top_p=0.7, min_p=0.02), dict(temp=1.0, top_k=0, top_p=0.5, min_p=0.1),
+                dict(temp=0.7, top_k=2000, top_p=1.0, min_p=0.05), dict(temp=1.2, top_k=0, top_p=0.999, min_p=0.0),
+                dict(temp=0.8, top_k=40, top_p=0.95, min_p=0.0), dict(temp=1.0, top_k=300, top_p=0.5, min_p=0.1)]
+    rows = len(settings)
+    logits = rnd(rows, V, scale=2.0, seed=V + 1)
+    logits[5] = torch.round(logits[5] * 2.0) / 2.0          # a row of ties: steps of 0.5
+    logits[2] = torch.round(logits[2] * 4.0) / 4.0
+    skip_ids = [-1, 7, -1, int(logits[3].argmax()), -1, -1, -1, -1]   # row 3 masks its best token
+    skip = torch.tensor(skip_ids, dtype=torch.int32, device=DEV)
+    f = lambda key: torch.tensor([s[key] for s in settings], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([s["top_k"] for s in settings], dtype=torch.int32, device=DEV)
+    rng = XorShift64(99)
+    host = logits.cpu()
+    for draw in range(draws):
+        units = [rng.unit() for _ in range(rows)]
+        if draw == 0:
+            units[0], units[1] = 0.0, 1.0 - 2.0 ** -24     # the ends of the range a unit takes
+        unit = torch.tensor(units, dtype=torch.float32, device=DEV)
+        out = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        o.sample_ranked(logits, f("temp"), top_k, f("top_p"), f("min_p"), unit, out, skip)
+        exact = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        o.sample_topk(logits, f("temp"), top_k, f("top_p"), f("min_p"), unit, exact, skip)
+        for r, s in enumerate(settings):
+            want = sampler_reference.sample(host[r].tolist(), s["temp"], s["top_k"], s["top_p"], s["min_p"], units[r],
+                                            skip=skip_ids[r] if skip_ids[r] >= 0 else None)
+            assert int(out[r]) == want, f"draw {draw}, row {r} ({s}): device {int(out[r])}, reference {want}"
+            if 0 < s["top_k"] <= 1024:
+                assert int(exact[r]) == want
+    # a greedy row is not written
+    out = torch.full((rows,), -5, dtype=torch.int32, device=DEV)
+    o.sample_ranked(logits, torch.zeros(rows, device=DEV), top_k, f("top_p"), f("min_p"), unit, out, skip)
+    assert out.tolist() == [-5] * rows
+
+
+def test_sampler_sends_each_row_to_the_kernel_that_takes_it():
+    """One call with greedy rows, rows that keep everything, small top-k sets and rows only the search by histograms
+    takes: every row's token is the reference's for that row's settings and generator."""
+    from llmx_amd.sampling import Sampler, SamplingParams, XorShift64
+    V = 3000
+    logits = rnd(6, V, scale=2.0, seed=77)
+    params = [SamplingParams(temp=0.0), SamplingParams(temp=0.9, top_k=0, top_p=1.0), SamplingParams(temp=1.1, top_k=30, top_p=0.9),
+              SamplingParams(temp=1.0, top_k=0, top_p=0.8), SamplingParams(temp=0.7, top_k=2500, top_p=1.0, min_p=0.01),
+              SamplingParams(temp=1.3, top_k=2000, top_p=0.6)]
+    sampler = Sampler(V, torch.device(DEV))
+    host = logits.cpu()
+    for kinds in ([0, 1, 2, 3, 4, 5], [3, 4, 5], [1, 3], [2, 5], [3]):
+        rngs = [XorShift64(50 + i) for i in kinds]
+        twins = [XorShift64(50 + i) for i in kinds]
+        got = sampler.sample(logits[kinds].contiguous(), [params[i] for i in kinds], [[] for _ in kinds], rngs, None)
+        for row, i in enumerate(kinds):
+            p = params[i]
+            unit = 0.0 if p.greedy else twins[row].unit()
+            want = sampler_reference.sample(host[i].tolist(), p.temp, p.top_k, p.top_p, p.min_p, unit)
+            assert got[row] == want, f"rows {kinds}, row {row} ({p})"
+
+
 def test_sampling_frequencies():
     """Empirical frequencies of 10,000 draws lie within 3 sigma of the softmax (method of sampler.cpp:41-53,128-150)."""
     o = ops()

@@ -32,11 +32,12 @@ def test_defaults_and_ranges():
         (64, 0.8, 40, 0.95, 0.0, 1.0, 0.0, 0.0, 0, False)
     d.validate()
     for bad in (dict(max_tokens=0), dict(temp=-0.1), dict(top_k=-1), dict(top_p=1.5), dict(min_p=-0.1), dict(penalty=0.5),
-                dict(presence_penalty=3.0), dict(frequency_penalty=-2.5), dict(seed=-1), dict(top_k=5000, top_p=1.0)):
+                dict(presence_penalty=3.0), dict(frequency_penalty=-2.5), dict(seed=-1)):
         with pytest.raises(ValueError, match="sampling: " + next(iter(bad))):
             SamplingParams(**bad).validate()
-    with pytest.raises(ValueError, match="sampling: top_p below 1 needs a top_k"):
-        SamplingParams(top_k=0, top_p=0.9).validate()
+    # a nucleus over the whole row and a top-k of any size are taken, as in the reference (sampler.hpp:149-252)
+    SamplingParams(top_k=0, top_p=0.9).validate()
+    SamplingParams(top_k=5000, top_p=1.0).validate()
     SamplingParams(temp=0.0, top_k=0, top_p=0.5).validate()     # greedy reads neither
     assert SamplingParams(temp=0.0).greedy and not SamplingParams().greedy and SamplingParams(penalty=1.2).penalized
 

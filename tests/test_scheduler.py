@@ -130,7 +130,7 @@ def test_requests_that_can_never_fit_are_refused_at_submit():
     with pytest.raises(SchedulerError, match="already submitted"):
         s.submit(Request("ok", [1], greedy(1)))
     with pytest.raises(ValueError, match="top_p"):
-        s.submit(Request("p", [1], SamplingParams(top_k=0, top_p=0.5)))
+        s.submit(Request("p", [1], SamplingParams(top_k=0, top_p=1.5)))
 
 
 def test_windowed_groups_reserve_a_window_not_the_whole_request():
