@@ -60,10 +60,12 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"{self.prefix}experts holds both fused and per-expert tensors")
         self.per_expert = has_single
         if has_single:
+            # each expert's tensors go from the host straight into their places in the fused tensors
+            down = self.name("experts.down_proj")
             for e in range(X):
-                specs += [TensorSpec(self.name(f"experts.{e}.gate_proj.weight"), (F, E)),
-                          TensorSpec(self.name(f"experts.{e}.up_proj.weight"), (F, E)),
-                          TensorSpec(self.name(f"experts.{e}.down_proj.weight"), (E, F))]
+                specs += [TensorSpec(self.name(f"experts.{e}.gate_proj.weight"), (F, E), into=(fused, (X, 2 * F, E), (e, slice(0, F)))),
+                          TensorSpec(self.name(f"experts.{e}.up_proj.weight"), (F, E), into=(fused, (X, 2 * F, E), (e, slice(F, 2 * F)))),
+                          TensorSpec(self.name(f"experts.{e}.down_proj.weight"), (E, F), into=(down, (X, E, F), (e,)))]
         else:
             specs += [TensorSpec(fused, (X, 2 * F, E)), TensorSpec(self.name("experts.down_proj"), (X, E, F))]
         return specs
@@ -72,14 +74,9 @@ class RoutedExperts(FeedForward):
         self.w_router = tensors[self.name("gate.weight")]
         if self.use_bias:
             self.bias = tensors[self.name("gate.e_score_correction_bias")]
-        if self.per_expert:
-            X = self.experts
-            self.w_gate_up = torch.stack([torch.cat([tensors[self.name(f"experts.{e}.gate_proj.weight")],
-                                                     tensors[self.name(f"experts.{e}.up_proj.weight")]], dim=0) for e in range(X)]).contiguous()
-            self.w_down = torch.stack([tensors[self.name(f"experts.{e}.down_proj.weight")] for e in range(X)]).contiguous()
-        else:
-            self.w_gate_up = tensors[self.name("experts.gate_up_proj")]
-            self.w_down = tensors[self.name("experts.down_proj")]
+        # per-expert files arrive fused too (see tensor_specs)
+        self.w_gate_up = tensors[self.name("experts.gate_up_proj")]
+        self.w_down = tensors[self.name("experts.down_proj")]
 
     def forward(self, step, h, out, accumulate, h32=None):
         T, X, k = step.rows, self.experts, self.top_k

@@ -17,10 +17,14 @@ class TensorSpec:
 
     role: "matrix" / "table" keep bfloat16 (or the stored 32 bits) in the bf16 path and are widened to float32 in the
           32-bit path; "norm" and "bias" vectors and "router" matrices are always float32; "int" tables are int32.
+    into: (target name, target shape, index): the tensor is one slice of a larger device tensor that the part reads
+          instead; the loader allocates the target once and copies each file tensor from the host straight into
+          target[index], so the slices are never on the device beside their fused copy.
     """
     name: str
     shape: Tuple[int, ...]
     role: str = "matrix"
+    into: Optional[Tuple[str, Tuple[int, ...], tuple]] = None
 
     ROLES = ("matrix", "table", "norm", "bias", "router", "int")
 

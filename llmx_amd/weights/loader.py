@@ -129,5 +129,14 @@ def load(specs: List[TensorSpec], files: ModelFiles, device: torch.device, exact
     out: Dict[str, torch.Tensor] = {}
     for s in specs:
         host = files.tensor(s.name)
-        out[s.name] = host.to(device=device, dtype=device_dtype(s, host.dtype, exact)).contiguous()
+        dtype = device_dtype(s, host.dtype, exact)
+        if s.into is None:
+            out[s.name] = host.to(device=device, dtype=dtype).contiguous()
+            continue
+        target, shape, index = s.into
+        if target not in out:
+            out[target] = torch.empty(shape, dtype=dtype, device=device)
+        elif out[target].dtype != dtype:
+            raise WeightsError(f"weights: {s.name} is stored as {host.dtype}, other parts of {target} in another type")
+        out[target][index].copy_(host.to(dtype))
     return out

@@ -335,6 +335,38 @@ def test_graph_replays_across_the_edges_their_key_exists_for(name, dtype, prompt
     assert replays_before_growth >= 10 and engines[0].graph_replays >= replays_before_growth + 10 and engines[1].graph_replays == 0
 
 
+def test_a_folder_with_per_expert_tensors_gives_the_fused_folder's_logits(tmp_path):
+    """experts.N.{gate,up,down}_proj.weight instead of the fused tensors: the loader fuses them on the way to the device."""
+    import json, shutil
+    from safetensors import safe_open
+    from llmx_amd.engine import Engine, StepEntry
+    from llmx_amd.weights import write_safetensors
+    src = model_folder("B")
+    split = {}
+    with safe_open(f"{src}/model.safetensors", framework="pt") as f:
+        for name in f.keys():
+            t = f.get_tensor(name)
+            if name.endswith("experts.gate_up_proj"):
+                half = t.shape[1] // 2
+                for e in range(t.shape[0]):
+                    split[name[:-len("gate_up_proj")] + f"{e}.gate_proj.weight"] = t[e, :half].clone()
+                    split[name[:-len("gate_up_proj")] + f"{e}.up_proj.weight"] = t[e, half:].clone()
+            elif name.endswith("experts.down_proj"):
+                for e in range(t.shape[0]):
+                    split[name[:-len("down_proj")] + f"{e}.down_proj.weight"] = t[e].clone()
+            else:
+                split[name] = t
+    shutil.copy(f"{src}/config.json", tmp_path / "config.json")
+    write_safetensors(tmp_path / "model.safetensors", split)
+    tokens = tokens_for("B", 23, 4)
+    outs = []
+    for folder in (src, str(tmp_path)):
+        eng = Engine.load(folder, dtype="bfloat16", kv_tokens=64, page_tokens=8, max_requests=1)
+        eng.add_request(0)
+        outs.append(eng.step([StepEntry(0, tokens, list(range(23)))]).clone())
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_refusals_leave_nothing_behind(setup):
     from llmx_amd.engine import StepEntry, StepError
     name, dtype, engine = setup

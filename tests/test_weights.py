@@ -126,7 +126,15 @@ def test_per_expert_tensor_names_are_an_alternative(tmp_path):
     model = BuiltModel(assemble(cfg), BuildContext(torch.float32, torch.device("cpu"), 8))
     specs = model.tensor_specs(set(split))
     check(specs, {n: (t.dtype, tuple(t.shape)) for n, t in split.items()})
-    model.load({n: t.float() for n, t in split.items()})
+    # through the loader: every expert's tensors are copied from the host into their places in the fused tensors, so
+    # what reaches the device is the fused pair alone (never the slices beside their fused copy)
+    write_safetensors(tmp_path / "model.safetensors", split)
+    files = ModelFiles(tmp_path)
+    loaded = load(specs, files, torch.device("cpu"), exact=True)
+    files.close()
+    assert not any(".experts." in n and n.endswith("_proj.weight") for n in loaded)
+    assert sum(t.numel() for t in loaded.values()) == sum(t.numel() for t in tensors.values())
+    model.load(loaded)
     ffn = model.blocks[0].ffn
     assert torch.equal(ffn.w_gate_up, tensors["model.layers.0.mlp.experts.gate_up_proj"].float())
     assert torch.equal(ffn.w_down, tensors["model.layers.0.mlp.experts.down_proj"].float())
