@@ -328,6 +328,183 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
     }
 }
 
+// Decoding rows of head_dim 128 when a step has few items: a workgroup of 4 waves works on one item, so that a
+// segment's 64 KB of keys and values are asked for at once by four waves instead of chunk after chunk by one.  Wave w
+// forms the scores of chunk w (keys 32w .. 32w+31 of the segment) and the value product of dims 32w .. 32w+31 over all
+// four chunks.  What the waves exchange through LDS: the chunks' maxima (a maximum does not depend on its order), every
+// lane's 32 softmax weights, which each wave adds in the order segment_softmax adds them, and the weights as the value
+// product's operands.  Per column the operations and their order are those of the kernel above: the same bits.
+// The items write their segments' (m, l, o) for the merge (a step of few items always shares its contexts out).
+__global__ void __launch_bounds__(256) paged_attention_split4_kernel(AttnMfmaArgs a) {
+    constexpr int DT = 8, QS = 4, D = 128;
+    __shared__ float top_s[2][4][64];
+    __shared__ __attribute__((aligned(16))) float p_s[2][4][64][8];
+    __shared__ __attribute__((aligned(16))) uint32_t pf_s[2][4][64][4];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int* it = a.items + (size_t)blockIdx.x * AM_ITEM_INTS;
+    const int row0 = __builtin_amdgcn_readfirstlane(it[0]), n_rows = __builtin_amdgcn_readfirstlane(it[1]);
+    const int head0 = __builtin_amdgcn_readfirstlane(it[2]), n_heads_item = __builtin_amdgcn_readfirstlane(it[3]);
+    const int split = __builtin_amdgcn_readfirstlane(it[4]), n_splits = __builtin_amdgcn_readfirstlane(it[5]);
+    const int slot = __builtin_amdgcn_readfirstlane(it[6]), slots = __builtin_amdgcn_readfirstlane(it[7]);
+    const int bt = a.page_tokens, Hkv = a.n_kv_heads;
+    const int c = lane & 15, g = lane >> 4;
+    const int n_cols = n_rows * n_heads_item;
+    const bool col_ok = c < n_cols;
+    const int t = row0 + (col_ok ? c / n_heads_item : 0);
+    const int h = head0 + (col_ok ? c % n_heads_item : 0);
+    const int kvh = head0 / (a.n_heads / Hkv);
+    const int p_col = a.pos[t];
+    const int p_first = __builtin_amdgcn_readfirstlane(a.pos[row0]), p_last = __builtin_amdgcn_readfirstlane(a.pos[row0 + n_rows - 1]);
+    const int* table = a.tables + (size_t)__builtin_amdgcn_readfirstlane(a.row_entry[row0]) * a.max_blocks;
+    const int lo_col = (a.window > 0 && p_col - a.window + 1 > 0) ? p_col - a.window + 1 : 0;
+    const int lo_first = (a.window > 0 && p_first - a.window + 1 > 0) ? p_first - a.window + 1 : 0;
+    const int seg_first = lo_first / AM_SEG;
+    const int n_seg = p_last / AM_SEG - seg_first + 1;
+    const int segs_per = (n_seg + n_splits - 1) / n_splits;
+    const int my_seg0 = seg_first + split * segs_per;
+    const int my_seg1 = min(seg_first + n_seg, my_seg0 + segs_per);
+    const int key_begin = my_seg0 * AM_SEG;
+    const int key_end = min(p_last + 1, my_seg1 * AM_SEG);
+    if (key_begin >= key_end) return;   // the whole workgroup
+
+    bf16x8_t qf[QS];
+#pragma unroll
+    for (int s = 0; s < QS; ++s) {
+        u32x4_t v = {0u, 0u, 0u, 0u};
+        if (col_ok) v = *reinterpret_cast<const u32x4_t*>(a.q + ((size_t)t * a.n_heads + h) * D + 32 * s + 8 * g);
+        qf[s] = __builtin_bit_cast(bf16x8_t, v);
+    }
+    // a segment's loads of this wave: the keys of chunk `wave` (two tiles of 16) and, of every chunk, the values of
+    // the wave's 32 dims
+    struct Loaded {
+        bf16x8_t kf[2][QS];
+        bf16x8_t vf[4][2];
+        int tile_in;   // bit tl: tile tl of the segment holds keys of the item
+    };
+    auto fetch = [&](int seg0, Loaded& x) {
+        x.tile_in = 0;
+        int pages[8], subs[8];
+#pragma unroll
+        for (int tl = 0; tl < 8; ++tl) {
+            const int key0 = seg0 + 16 * tl;
+            const bool in = key0 < key_end;
+            pages[tl] = in ? table[key0 / bt] : -1;
+            subs[tl] = key0 % bt;
+            if (in) x.tile_in |= 1 << tl;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            // tile 2 wave + u; selected without indexing the arrays by a run-time value
+            int page = -1, sub = 0;
+#pragma unroll
+            for (int tl = 0; tl < 8; ++tl)
+                if (tl == 2 * wave + u) {
+                    page = pages[tl];
+                    sub = subs[tl];
+                }
+            const bf16_t* src = a.k_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * bt + sub + c) * D + 8 * g;
+#pragma unroll
+            for (int s = 0; s < QS; ++s) {
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                if (page >= 0) v = *reinterpret_cast<const u32x4_t*>(src + 32 * s);
+                x.kf[u][s] = __builtin_bit_cast(bf16x8_t, v);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int page0 = pages[2 * v], page1 = pages[2 * v + 1];
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int dim = 32 * wave + 16 * q + c;
+                const bf16_t* src0 = a.v_cache + (((size_t)(page0 < 0 ? 0 : page0) * Hkv + kvh) * D + dim) * bt + subs[2 * v] + 4 * g;
+                const bf16_t* src1 = a.v_cache + (((size_t)(page1 < 0 ? 0 : page1) * Hkv + kvh) * D + dim) * bt + subs[2 * v + 1] + 4 * g;
+                u32x2_t v0 = {0u, 0u}, v1 = {0u, 0u};
+                if (page0 >= 0) v0 = *reinterpret_cast<const u32x2_t*>(src0);
+                if (page1 >= 0) v1 = *reinterpret_cast<const u32x2_t*>(src1);
+                const u32x4_t both = {v0[0], v0[1], v1[0], v1[1]};
+                x.vf[v][q] = __builtin_bit_cast(bf16x8_t, both);
+            }
+        }
+    };
+
+    Loaded cur, next;
+    fetch(key_begin, cur);
+    int par = 0;
+    for (int seg0 = key_begin; seg0 < key_end; seg0 += AM_SEG, par ^= 1) {
+        const bool more = seg0 + AM_SEG < key_end;
+        if (more) fetch(seg0 + AM_SEG, next);     // the next segment travels while this one is worked on
+        f32x4_t s0, s1;
+        chunk_scores<DT>(cur.kf, qf, s0, s1);
+        // the keys that count for the lane's column: bits 8 v + 4 u + i of the segment's mask, tiles without keys taken out
+        uint32_t ok = segment_mask(seg0, g, col_ok, lo_col, p_col, key_end);
+#pragma unroll
+        for (int tl = 0; tl < 8; ++tl)
+            if (!((cur.tile_in >> tl) & 1)) ok &= ~(0xfu << (4 * tl));
+        const uint32_t mine = (ok >> (8 * wave)) & 0xffu;
+        float top = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if ((mine >> i) & 1u) top = fmaxf(top, s0[i]);
+            if ((mine >> (4 + i)) & 1u) top = fmaxf(top, s1[i]);
+        }
+        top = rows_max4(top);
+        top_s[par][wave][lane] = top;
+        __syncthreads();
+        top = fmaxf(fmaxf(top_s[par][0][lane], top_s[par][1][lane]), fmaxf(top_s[par][2][lane], top_s[par][3][lane]));
+        const float m = top * a.scale;
+        const float k = a.scale * 1.44269504088896340736f;
+        const float shift = -(top * k);
+        float pv[8];
+        bf16x8_t pf_mine;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const bool counts = ((mine >> j) & 1u) && top != -INFINITY;
+            const float sc = j < 4 ? s0[j & 3] : s1[j & 3];
+            pv[j] = counts ? __builtin_amdgcn_exp2f(fmaf(sc, k, shift)) : 0.0f;
+            pf_mine[j] = (__bf16)pv[j];
+        }
+        *reinterpret_cast<f32x4_t*>(&p_s[par][wave][lane][0]) = f32x4_t{pv[0], pv[1], pv[2], pv[3]};
+        *reinterpret_cast<f32x4_t*>(&p_s[par][wave][lane][4]) = f32x4_t{pv[4], pv[5], pv[6], pv[7]};
+        *reinterpret_cast<u32x4_t*>(&pf_s[par][wave][lane][0]) = __builtin_bit_cast(u32x4_t, pf_mine);
+        __syncthreads();
+        // the lane's 32 weights added in the order segment_softmax adds them (chunk after chunk), then over the column's 4 lanes
+        float sum = 0.0f;
+        bf16x8_t pf[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const f32x4_t lo4 = *reinterpret_cast<const f32x4_t*>(&p_s[par][v][lane][0]);
+            const f32x4_t hi4 = *reinterpret_cast<const f32x4_t*>(&p_s[par][v][lane][4]);
+            sum += lo4[0];
+            sum += lo4[1];
+            sum += lo4[2];
+            sum += lo4[3];
+            sum += hi4[0];
+            sum += hi4[1];
+            sum += hi4[2];
+            sum += hi4[3];
+            pf[v] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&pf_s[par][v][lane][0]));
+        }
+        const float l = rows_sum4(sum);
+        f32x4_t o[2] = {f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int q = 0; q < 2; ++q) o[q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.vf[v][q], pf[v], o[q], 0, 0, 0);
+        if (col_ok) {
+            const size_t at = (size_t)slot * 16 + (size_t)c * slots + (seg0 / AM_SEG - seg_first);
+            float* dst = a.part_o + at * D + 32 * wave + 4 * g;   // the wave's dims: tiles 2 wave and 2 wave + 1 of 16
+            *reinterpret_cast<f32x4_t*>(dst) = o[0];
+            *reinterpret_cast<f32x4_t*>(dst + 16) = o[1];
+            if (wave == 0 && g == 0) {
+                a.part_ml[at * 2] = m;
+                a.part_ml[at * 2 + 1] = l;
+            }
+        }
+        if (more) cur = next;
+    }
+}
+
 // Prompt tiles that share their keys: a workgroup's 4 waves hold 4 items (tiles of up to 16 rows of one head each) of one
 // request and one KV head, for instance 4 of the query heads that read it.  A segment's 128 keys and values are brought
 // from the pages into LDS once by all 256 threads and every wave takes its fragments from there, so each byte of the
@@ -869,12 +1046,13 @@ extern "C" int llmx_attention_partial_pad() { return MERGE_PAD; }
 // `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 8: one workgroup each 8, or
 // each 4 for head sizes other than 128),
 // then the n_direct items that fold their segments themselves (slot < 0), then the n_partial items that write them
-// (slot >= 0).
+// (slot >= 0).  wide_items: a decoding item is worked on by a workgroup of 4 waves instead of one wave (head_dim 128 only;
+// the form for steps of few items; the same bits).
 extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
                                          const int* tables, const int* items, int n_shared, int n_direct, int n_partial, const int* merges,
                                          int n_merges,
                                          void* out, float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
-                                         int page_tokens, int max_blocks, int window, hipStream_t stream) {
+                                         int page_tokens, int max_blocks, int window, int wide_items, hipStream_t stream) {
     if (n_shared + n_direct + n_partial <= 0) return 0;
     if (n_shared % 8) return -2;
     if (head_dim % 16 || head_dim > AM_MAX_D || page_tokens % 16 || n_heads % n_kv_heads) return -2;
@@ -894,7 +1072,10 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
             hipLaunchKernelGGL(paged_attention_tiles128_kernel, dim3(n_shared / 8), dim3(512), 0, stream, sh);                          \
         else if (n_shared > 0) hipLaunchKernelGGL((paged_attention_tiles_kernel<DT>), dim3(n_shared / 4), block, 0, stream, sh);        \
         if (n_direct > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, false>), dim3((n_direct + 3) / 4), block, 0, stream, a);  \
-        if (n_partial > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, true>), dim3((n_partial + 3) / 4), block, 0, stream, b); \
+        if (n_partial > 0 && DT == 8 && wide_items)                                                                          \
+            hipLaunchKernelGGL(paged_attention_split4_kernel, dim3(n_partial), block, 0, stream, b);                                    \
+        else if (n_partial > 0)                                                                                              \
+            hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, true>), dim3((n_partial + 3) / 4), block, 0, stream, b);                \
         break;
         AM_CASE(1) AM_CASE(2) AM_CASE(3) AM_CASE(4) AM_CASE(5) AM_CASE(6) AM_CASE(7) AM_CASE(8)
         AM_CASE(9) AM_CASE(10) AM_CASE(11) AM_CASE(12) AM_CASE(13) AM_CASE(14) AM_CASE(15) AM_CASE(16)

@@ -62,7 +62,7 @@ def _declare(h) -> None:
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
         "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
-        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, P],
+        "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
@@ -263,6 +263,8 @@ class AttentionPlan:
         self.n_items = len(items)
         self.n_merges = len(merges)
         self.n_slots = n_slots
+        # few decoding items: each is worked on by a workgroup of 4 waves (the kernel takes this form for head_dim 128)
+        self.wide_items = 0 < self.n_items - self.n_shared <= ATTENTION_WIDE_ITEMS
         self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 8), device=device) if items else None
         self.merges = torch.tensor(np.asarray(merges, dtype=np.int32).reshape(-1, 8), device=device) if merges else None
 
@@ -270,6 +272,7 @@ class AttentionPlan:
 _PLAN_CACHE: dict = {}
 ATTENTION_TARGET_WAVES = 2048   # work items wanted before long contexts stop being split further
 ATTENTION_SEGMENT = 128         # keys in a segment: the unit contexts are split in (the kernel's AM_SEG)
+ATTENTION_WIDE_ITEMS = 1024     # up to this many decoding items a step, an item gets a workgroup of 4 waves instead of one wave
 
 
 def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, window: int = 0) -> AttentionPlan:
@@ -359,7 +362,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                                plan.n_items - plan.n_shared - plan.n_direct,
                                                _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
                                                _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale), n_heads, n_kv_heads,
-                                               head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention_mfma")
+                                               head_dim, page_tokens, tables.shape[1], int(window), 1 if plan.wide_items else 0, _stream()),
+               "paged_attention_mfma")
         return
     _check(lib().llmx_paged_attention_generic(*common, _dev(out, "out"), _code(q.dtype), float(scale), rows, n_heads, n_kv_heads,
                                               head_dim, page_tokens, tables.shape[1], int(window), _stream()), "paged_attention")

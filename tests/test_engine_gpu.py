@@ -335,7 +335,7 @@ def test_graph_replays_across_the_edges_their_key_exists_for(name, dtype, prompt
     assert replays_before_growth >= 10 and engines[0].graph_replays >= replays_before_growth + 10 and engines[1].graph_replays == 0
 
 
-def test_a_folder_with_per_expert_tensors_gives_the_fused_folder's_logits(tmp_path):
+def test_a_folder_with_per_expert_tensors_gives_the_logits_of_the_fused_folder(tmp_path):
     """experts.N.{gate,up,down}_proj.weight instead of the fused tensors: the loader fuses them on the way to the device."""
     import json, shutil
     from safetensors import safe_open

@@ -528,6 +528,58 @@ def test_attention_row_is_the_same_bits_alone_or_in_a_tile(L, Hq, Hkv, D, window
             assert torch.equal(alone[0], tile[r]), f"row {r} (context {ctx}, target {target}) differs from its bits in the tile"
 
 
+@pytest.mark.parametrize("contexts,Hq,Hkv,window", [((4096,), 48, 8, 0), ((1, 130, 517, 2000, 64, 129), 12, 2, 0), ((900, 3000), 8, 8, 700),
+                                                     ((5000, 77), 20, 1, 0)])
+def test_decoding_items_worked_on_by_four_waves_give_the_bits_of_one_wave(contexts, Hq, Hkv, window):
+    """Head size 128: in a step of few items a workgroup of four waves shares an item's segments (a wave a chunk of 32
+    keys for the scores, a wave 32 dims for the values); the partial results and the merged rows must be those of the
+    form with one wave an item, for contexts that end anywhere in a segment, a single key, a window and several rows."""
+    o = ops()
+    D, page = 128, 16
+    n = len(contexts)
+    blocks = [-(-c // page) for c in contexts]
+    order = list(range(sum(blocks)))
+    random.Random(n).shuffle(order)
+    table = torch.full((n, max(blocks)), -1, dtype=torch.int32)
+    at = 0
+    for i, b in enumerate(blocks):
+        table[i, :b] = torch.tensor(order[at:at + b])
+        at += b
+    table = table.to(DEV)
+    k_cache = rnd(sum(blocks), Hkv, page, D, dtype=torch.bfloat16, scale=0.5)
+    v_cache = rnd(sum(blocks), Hkv, D, page, dtype=torch.bfloat16, seed=2)
+    q = rnd(n, Hq * D, dtype=torch.bfloat16, seed=3)
+    pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device=DEV)
+    ent = torch.arange(n, dtype=torch.int32, device=DEV)
+    outs = []
+    saved = o.ATTENTION_WIDE_ITEMS
+    for wide in (saved, 0):
+        o.ATTENTION_WIDE_ITEMS = wide
+        o._PLAN_CACHE.clear()
+        try:
+            plan = o.attention_plan([1] * n, list(contexts), Hq, Hkv, DEV, window)
+        finally:
+            o.ATTENTION_WIDE_ITEMS = saved
+        assert plan.wide_items == (wide > 0) and plan.n_merges > 0
+        out = torch.zeros(n, Hq * D, dtype=torch.bfloat16, device=DEV)
+        o.paged_attention(q, k_cache, v_cache, pos, ent, table, out, 1.0 / math.sqrt(D), Hq, window, plan=plan)
+        outs.append(out)
+    o._PLAN_CACHE.clear()
+    assert torch.equal(outs[0], outs[1])
+    # and the plain softmax for one head of every row
+    inv = torch.tensor(order, device=DEV)
+    for i, c in enumerate(contexts):
+        pages = table[i, :blocks[i]].long()
+        keys = k_cache[pages].permute(1, 0, 2, 3).reshape(Hkv, -1, D)[:, :c].double()
+        values = v_cache[pages].permute(1, 0, 3, 2).reshape(Hkv, -1, D)[:, :c].double()
+        lo = max(0, c - window) if window else 0
+        h = (i * 5) % Hq
+        kv = h // (Hq // Hkv)
+        w = torch.softmax((keys[kv, lo:] @ q[i, h * D:(h + 1) * D].double()) / math.sqrt(D), dim=0)
+        want = w @ values[kv, lo:]
+        assert (outs[0][i, h * D:(h + 1) * D].double() - want).abs().max() <= 1.2e-2 * want.abs().max() + 2e-4
+
+
 @pytest.mark.parametrize("L,Hq,Hkv,D", [(70000, 2, 1, 32), (66000, 4, 2, 160)])
 def test_attention_very_long_context(L, Hq, Hkv, D):
     """A decoded row over more than 512 segments of keys (the merge works through them in several rounds): the same bits
