@@ -25,24 +25,29 @@ struct QkvArgs {
     int n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode;
     int page_tokens, max_blocks, write_kv;
     int q_slices, k_slices;  // blocks that share a row's q (k) projection: each norms with the whole sum and writes its slice
+    int pairing;             // which dims of a head rotate together: ROPE_HALVES (i, i + R/2) or ROPE_INTERLEAVED (2i, 2i + 1)
 };
+
+enum : int { ROPE_HALVES = 0, ROPE_INTERLEAVED = 1 };
 
 // Two blocks per row: one norms and rotates q, the other norms and rotates k and writes k and v to the row's page.
 // Norm over the whole projection: the sum of squares of the row's q (or k) values, strided per thread, butterfly per
-// wave, waves in order.  Then y = x * (r * w) and the NeoX rotation of pairs (i, i + R/2) of each head:
+// wave, waves in order.  Then y = x * (r * w) and the rotation of each head's pairs (a, b), pair j by the angle of
+// frequency j: the NeoX halves (j, j + R/2) or the interleaved pairs (2j, 2j + 1):
 // a' = fma(-b, sin, a*cos), b' = fma(a, sin, b*cos); dims [R, D) pass through.
 __device__ __forceinline__ float normed_rotated(const float* __restrict__ row, const float* __restrict__ weight, const float* __restrict__ cs,
-                                                int i, int D, int rotary_dim, bool normed, float r) {
+                                                int i, int D, int rotary_dim, bool normed, float r, int pairing) {
     const int d = i % D, half = rotary_dim / 2;
     float x = row[i];
     if (normed) x = x * (r * weight[i]);
     if (d < rotary_dim) {
-        const int j = d < half ? d : d - half;
-        const int other = d < half ? i + half : i - half;
+        const bool first = pairing == ROPE_HALVES ? d < half : (d & 1) == 0;    // the pair's a
+        const int j = pairing == ROPE_HALVES ? (d < half ? d : d - half) : d >> 1;
+        const int other = pairing == ROPE_HALVES ? (first ? i + half : i - half) : (first ? i + 1 : i - 1);
         float y = row[other];
         if (normed) y = y * (r * weight[other]);
         const float c = cs[j], s = cs[half + j];
-        x = d < half ? fmaf(-y, s, x * c) : fmaf(y, s, x * c);
+        x = first ? fmaf(-y, s, x * c) : fmaf(y, s, x * c);
     }
     return x;
 }
@@ -67,7 +72,7 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
         const int per = (qw + a.q_slices - 1) / a.q_slices;
         const int begin = blockIdx.y * per, end = min(qw, begin + per);
         TQ* q_out = (TQ*)a.q_out + (size_t)t * qw;
-        for (int i = begin + threadIdx.x; i < end; i += 256) st(q_out + i, normed_rotated(row, a.q_weight, cs, i, D, a.rotary_dim, normed, r));
+        for (int i = begin + threadIdx.x; i < end; i += 256) st(q_out + i, normed_rotated(row, a.q_weight, cs, i, D, a.rotary_dim, normed, r, a.pairing));
         return;
     }
     if (!a.write_kv) return;
@@ -87,7 +92,7 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_kernel(QkvArgs a) {
     for (int i = begin + threadIdx.x; i < end; i += 256) {
         const int h = i / D, d = i % D;
         const size_t head_at = (size_t)page * a.n_kv_heads + h;
-        st(kc + (head_at * a.page_tokens + slot) * D + d, normed_rotated(krow, a.k_weight, cs, i, D, a.rotary_dim, normed, r));
+        st(kc + (head_at * a.page_tokens + slot) * D + d, normed_rotated(krow, a.k_weight, cs, i, D, a.rotary_dim, normed, r, a.pairing));
         st(vc + (head_at * D + d) * a.page_tokens + slot, krow[kw + i]);
     }
 }
@@ -120,7 +125,7 @@ struct HeadDim {
 
 template <int KEPT>
 __device__ __forceinline__ void norm_rotate_kept(const float* __restrict__ src, const float* __restrict__ weight, int width,
-                                                 const float* __restrict__ cs, int D, int rotary_dim, int norm_mode, float eps,
+                                                 const float* __restrict__ cs, int D, int rotary_dim, int norm_mode, float eps, int pairing,
                                                  float* __restrict__ row_lds, float* __restrict__ scratch, KeptRow<KEPT>& out) {
     const int tid = threadIdx.x, half = rotary_dim / 2;
     const bool normed = norm_mode != QKNORM_NONE;
@@ -152,11 +157,11 @@ __device__ __forceinline__ void norm_rotate_kept(const float* __restrict__ src, 
     for (int j = 0; j < KEPT; ++j) {
         const int i = tid + 256 * j;
         if (i < width && at.d < rotary_dim) {
-            const bool low = at.d < half;
-            const int pair = low ? at.d : at.d - half;
-            const float y = row_lds[low ? i + half : i - half];
+            const bool first = pairing == ROPE_HALVES ? at.d < half : (at.d & 1) == 0;
+            const int pair = pairing == ROPE_HALVES ? (first ? at.d : at.d - half) : at.d >> 1;
+            const float y = row_lds[pairing == ROPE_HALVES ? (first ? i + half : i - half) : (first ? i + 1 : i - 1)];
             const float c = cs_lds[pair], sn = cs_lds[half + pair];
-            out.x[j] = low ? fmaf(-y, sn, out.x[j] * c) : fmaf(y, sn, out.x[j] * c);
+            out.x[j] = first ? fmaf(-y, sn, out.x[j] * c) : fmaf(y, sn, out.x[j] * c);
         }
         at.next();
     }
@@ -174,7 +179,7 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_rows_kernel(QkvArgs a
     const float* cs = a.cos_sin + (size_t)p * a.rotary_dim;
     if (blockIdx.y == 0) {
         KeptRow<KQ> q;
-        norm_rotate_kept<KQ>(row, a.q_weight, qw, cs, D, a.rotary_dim, a.norm_mode, a.eps, row_lds, scratch, q);
+        norm_rotate_kept<KQ>(row, a.q_weight, qw, cs, D, a.rotary_dim, a.norm_mode, a.eps, a.pairing, row_lds, scratch, q);
         TQ* q_out = (TQ*)a.q_out + (size_t)t * qw;
 #pragma unroll
         for (int j = 0; j < KQ; ++j)
@@ -188,7 +193,7 @@ __global__ void __launch_bounds__(256) qknorm_rope_kvwrite_rows_kernel(QkvArgs a
 #pragma unroll
     for (int j = 0; j < KK; ++j) vals[j] = tid + 256 * j < kw ? row[qw + kw + tid + 256 * j] : 0.0f;
     KeptRow<KK> k;
-    norm_rotate_kept<KK>(row + qw, a.k_weight, kw, cs, D, a.rotary_dim, a.norm_mode, a.eps, row_lds, scratch, k);
+    norm_rotate_kept<KK>(row + qw, a.k_weight, kw, cs, D, a.rotary_dim, a.norm_mode, a.eps, a.pairing, row_lds, scratch, k);
     TKV* kc = (TKV*)a.k_cache;
     TKV* vc = (TKV*)a.v_cache;
     HeadDim at(tid, D);
@@ -217,9 +222,10 @@ static void launch_qkv_rows(const QkvArgs& a, int rows, int qw, int kw, hipStrea
 extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight, const float* k_weight, const float* cos_sin, const int* pos,
                                         const int* row_entry, const int* tables, void* q_out, void* k_cache, void* v_cache, int dtype,
                                         float eps, int rows, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int norm_mode,
-                                        int page_tokens, int max_blocks, int write_kv, hipStream_t stream) {
+                                        int page_tokens, int max_blocks, int write_kv, int pairing, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (norm_mode != QKNORM_NONE && norm_mode != QKNORM_PROJECTION) return -2;
+    if (pairing != ROPE_HALVES && pairing != ROPE_INTERLEAVED) return -2;
     // few rows: many blocks a row, so the chip is used; many rows: two blocks a row, so the sum is not formed over and over
     const int qw = n_heads * head_dim, kw = n_kv_heads * head_dim;
     int q_slices = 1, k_slices = 1;
@@ -230,7 +236,7 @@ extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight,
         if (k_slices > 4) k_slices = 4;
     }
     QkvArgs a{qkv, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
-              n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, q_slices, k_slices};
+              n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, q_slices, k_slices, pairing};
     if (rows > 256 && qw <= 32 * 256 && kw <= 32 * 256 && head_dim <= 256) {   // rows kept in registers
         if (dtype == LLMX_F32) launch_qkv_rows<float, float>(a, rows, qw, kw, stream);
         else launch_qkv_rows<bf16_t, bf16_t>(a, rows, qw, kw, stream);

@@ -20,6 +20,7 @@ from .limits import MAX_EXPERTS, MAX_HEAD_DIM, MAX_TOP_K
 F32, BF16 = 0, 1
 EPI_STORE, EPI_ADD, EPI_SWIGLU = 0, 1, 2
 QKNORM_NONE, QKNORM_PROJECTION, QKNORM_HEAD = 0, 1, 2
+ROPE_HALVES, ROPE_INTERLEAVED = 0, 1        # a head's rotated pairs: (i, i + R/2) or (2i, 2i + 1)
 SCORE_SIGMOID, SCORE_SOFTMAX = 0, 1
 
 
@@ -60,7 +61,7 @@ def _declare(h) -> None:
         "llmx_read_probe": [P, L, P, P],
         "llmx_attention_partial_pad": [],
         "llmx_gemm_generic": [P, I, P, I, P, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P],
-        "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, P],
+        "llmx_qknorm_rope_kvwrite": [P, P, P, P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_generic": [P, P, P, P, P, P, P, I, F, I, I, I, I, I, I, I, P],
         "llmx_paged_attention_mfma": [P, P, P, P, P, P, P, I, I, I, P, I, P, P, P, F, I, I, I, I, I, I, I, P],
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P],
@@ -229,7 +230,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
 def qknorm_rope_kvwrite(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], cos_sin: torch.Tensor,
                         pos: torch.Tensor, row_entry: torch.Tensor, tables: torch.Tensor, q_out: torch.Tensor,
                         k_cache: torch.Tensor, v_cache: torch.Tensor, eps: float, n_heads: int, n_kv_heads: int, head_dim: int,
-                        rotary_dim: int, norm_mode: int, write_kv: bool = True) -> None:
+                        rotary_dim: int, norm_mode: int, write_kv: bool = True, pairing: int = ROPE_HALVES) -> None:
     rows = qkv.shape[0]
     qw, kw = n_heads * head_dim, n_kv_heads * head_dim
     n_pages, hk, page_tokens, d = k_cache.shape
@@ -248,7 +249,7 @@ def qknorm_rope_kvwrite(qkv: torch.Tensor, q_weight: Optional[torch.Tensor], k_w
         _dev(cos_sin, "cos_sin", torch.float32), _dev(pos, "pos", torch.int32, (rows,)), _dev(row_entry, "row_entry", torch.int32, (rows,)),
         _dev(tables, "tables", torch.int32), _dev(q_out, "q_out", shape=(rows, qw)), _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"),
         _code(q_out.dtype), float(eps), rows, n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, tables.shape[1],
-        1 if write_kv else 0, _stream()), "qknorm_rope_kvwrite")
+        1 if write_kv else 0, int(pairing), _stream()), "qknorm_rope_kvwrite")
 
 
 class AttentionPlan:

@@ -22,7 +22,8 @@ _NORM_MODES = {"none": ops.QKNORM_NONE, "projection": ops.QKNORM_PROJECTION}
 
 
 class Attention(Mixer):
-    """params: hidden, heads, kv_heads, head_dim, qk_norm ("projection" | "none"), eps, window (None | int), position (PartSpec)."""
+    """params: hidden, heads, kv_heads, head_dim, qk_norm ("projection" | "none"), eps, window (None | int), position (PartSpec),
+    scale (None: head_dim^-1/2; else the factor the scores are multiplied by)."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx: BuildContext):
@@ -42,7 +43,14 @@ class Attention(Mixer):
             raise ValueError(f"qk_norm {p.get('qk_norm')!r} is not one of {sorted(_NORM_MODES)}")
         self.norm_mode = _NORM_MODES[p.get("qk_norm", "none")]
         self.position = build_part("position", p.get("position") or PartSpec("none"), ctx)
-        self.scale = float(np.float32(1.0) / np.sqrt(np.float32(self.head_dim)))
+        pairing = getattr(self.position, "pairing", "halves")
+        if pairing not in ("halves", "interleaved"):
+            raise ValueError(f"attention: rotary pairing {pairing!r} is not one the kernels rotate (halves, interleaved)")
+        self.pairing = ops.ROPE_INTERLEAVED if pairing == "interleaved" else ops.ROPE_HALVES
+        # softmax(q.k * scale): head_dim^-1/2 unless the architecture gives its own
+        self.scale = float(p["scale"]) if p.get("scale") is not None else float(np.float32(1.0) / np.sqrt(np.float32(self.head_dim)))
+        if not self.scale > 0.0:
+            raise ValueError(f"attention: the softmax scale must be positive, not {self.scale}")
         self.q_width = self.heads * self.head_dim
         self.kv_width = self.kv_heads * self.head_dim
         self.wqkv = self.wo = self.q_norm = self.k_norm = None
@@ -82,7 +90,8 @@ class Attention(Mixer):
         cos_sin, rotary = self.position.rotation()
         tables = step.tables(cache.group)
         ops.qknorm_rope_kvwrite(qkv, self.q_norm, self.k_norm, cos_sin, step.positions, step.row_entry, tables, q, cache.k, cache.v,
-                                self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode, write_kv=cache.writes)
+                                self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode, write_kv=cache.writes,
+                                pairing=self.pairing)
         o = step.buf("attention.out", (T, self.q_width), act)
         plan = None
         if ops.attention_mfma_ok(act, self.head_dim, cache.k.shape[2]):

@@ -73,7 +73,11 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """Owns what a mixer needs to place a row at its position; for rotary forms a table of cos and sin."""
+    """Owns what a mixer needs to place a row at its position; for rotary forms a table of cos and sin, and which dims
+    of a head rotate together."""
+
+    #: "halves": dims i and i + R/2 are a pair; "interleaved": dims 2i and 2i + 1
+    pairing = "halves"
 
     def rotation(self):
         """(cos_sin [positions, rotary_dim] float32 on the device, rotary_dim), cos of the pairs then sin; rotary_dim 0 rotates nothing."""

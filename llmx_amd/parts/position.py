@@ -12,6 +12,8 @@ import torch
 
 from .base import PositionEncoding, register
 
+PAIRINGS = ("halves", "interleaved")
+
 
 def neox_table(positions: int, rotary_dim: int, theta: float) -> np.ndarray:
     """[positions, rotary_dim] float32: cos of the rotary_dim/2 pairs, then sin.
@@ -33,11 +35,15 @@ def neox_table(positions: int, rotary_dim: int, theta: float) -> np.ndarray:
 
 
 class PartialRotary(PositionEncoding):
-    """params: rotary_dim (even, at most head_dim; 0 rotates nothing), theta, head_dim."""
+    """params: rotary_dim (even, at most head_dim; 0 rotates nothing), theta, head_dim, pairing ("halves", the default:
+    dims i and i + rotary_dim/2 rotate together; "interleaved": dims 2i and 2i + 1)."""
     graph_safe = True
 
     def __init__(self, params, prefix, ctx):
         super().__init__(params, prefix, ctx)
+        self.pairing = str(params.get("pairing", "halves"))
+        if self.pairing not in PAIRINGS:
+            raise ValueError(f"rotary pairing {self.pairing!r} is not one of {sorted(PAIRINGS)}")
         self.rotary_dim = int(params["rotary_dim"])
         self.theta = float(params["theta"])
         head_dim = int(params["head_dim"])

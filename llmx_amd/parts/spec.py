@@ -39,12 +39,19 @@ class PartSpec:
 
 @dataclass
 class BlockSpec:
-    """One layer: how its parts are arranged ("prenorm": x += mixer(norm(x)); x += ffn(norm(x)))."""
+    """One layer: its parts and the name of their arrangement ("prenorm": x += mixer(norm(x)); x += ffn(norm(x))).
+
+    The four named parts are what most arrangements have; an arrangement that needs more (norms after the mixer and
+    the feed-forward, a second feed-forward, a gate) finds them in `extra` by the names it gives them, each with the
+    family ("norm", "mixer", "feed_forward", ...) it is built from.  The arrangement class builds what it uses and
+    lists it in `parts()`; the engine asks a block's `mixer` for what its cache number holds.
+    """
     mixer_norm: PartSpec
     mixer: PartSpec
     ffn_norm: PartSpec
     ffn: PartSpec
     arrangement: str = "prenorm"
+    extra: Dict[str, Tuple[str, PartSpec]] = field(default_factory=dict)   # name -> (family, part)
 
 
 @dataclass(frozen=True)

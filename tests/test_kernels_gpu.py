@@ -333,10 +333,22 @@ def test_routed_products(T, X, k, E, F, dtype):
 
 
 # ---------------------------------------------------------------------------
+def interleaved_rope(x, cos, sin, R):
+    """Pairs (2j, 2j + 1) of the first R dims of each head rotated by angle j; x [T, H, D], cos and sin [T, R/2]."""
+    out = x.clone()
+    a, b = x[..., 0:R:2], x[..., 1:R:2]
+    c, s = cos.to(x.dtype)[:, None, :], sin.to(x.dtype)[:, None, :]
+    out[..., 0:R:2] = a * c - b * s
+    out[..., 1:R:2] = b * c + a * s
+    return out
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("Hq,Hkv,D,R,norm", [(48, 8, 128, 64, True), (6, 2, 80, 80, True), (20, 20, 160, 34, True), (5, 1, 48, 0, True),
-                                              (30, 30, 256, 256, False), (12, 3, 16, 8, True)])
-def test_qknorm_rope_kvwrite_of_many_rows_keeps_the_bits_of_few_rows(Hq, Hkv, D, R, norm, dtype):
+@pytest.mark.parametrize("Hq,Hkv,D,R,norm,pairing", [(48, 8, 128, 64, True, "halves"), (6, 2, 80, 80, True, "halves"), (20, 20, 160, 34, True, "halves"),
+                                                      (5, 1, 48, 0, True, "halves"), (30, 30, 256, 256, False, "halves"), (12, 3, 16, 8, True, "halves"),
+                                                      (48, 8, 128, 64, True, "interleaved"), (6, 2, 80, 80, False, "interleaved"),
+                                                      (12, 3, 16, 6, True, "interleaved")])
+def test_qknorm_rope_kvwrite_of_many_rows_keeps_the_bits_of_few_rows(Hq, Hkv, D, R, norm, pairing, dtype):
     """More than 256 rows in one launch take the form that keeps a row in registers; it must give every row the bits of
     the launches of few rows (q, the key pages and the transposed value pages), and agree with the plain formulas
     (norm over the whole projection, NeoX halves over the first R dims).  The shapes reach all four register budgets
@@ -362,7 +374,7 @@ def test_qknorm_rope_kvwrite_of_many_rows_keeps_the_bits_of_few_rows(Hq, Hkv, D,
         vc = torch.zeros(2 * blocks, Hkv, D, page, dtype=dtype, device=DEV)
         for a, b in chunks:
             o.qknorm_rope_kvwrite(qkv[a:b], wq if norm else None, wk if norm else None, cos_sin, pos[a:b], ent[a:b], tables, q[a:b], kc, vc,
-                                  eps, Hq, Hkv, D, R, mode)
+                                  eps, Hq, Hkv, D, R, mode, pairing=o.ROPE_INTERLEAVED if pairing == "interleaved" else o.ROPE_HALVES)
         return q, kc, vc
 
     many = run([(0, rows)])
@@ -376,8 +388,9 @@ def test_qknorm_rope_kvwrite_of_many_rows_keeps_the_bits_of_few_rows(Hq, Hkv, D,
         qp, kp = plain_model.rms_norm(qp, wq.double().cpu(), eps), plain_model.rms_norm(kp, wk.double().cpu(), eps)
     cs_rows = cos_sin.double().cpu()[pos.long().cpu()]
     half = R // 2
-    qp = plain_model.apply_partial_rope(qp.reshape(rows, Hq, D), cs_rows[:, :half], cs_rows[:, half:], R)
-    kp = plain_model.apply_partial_rope(kp.reshape(rows, Hkv, D), cs_rows[:, :half], cs_rows[:, half:], R)
+    rotate = interleaved_rope if pairing == "interleaved" else plain_model.apply_partial_rope
+    qp = rotate(qp.reshape(rows, Hq, D), cs_rows[:, :half], cs_rows[:, half:], R)
+    kp = rotate(kp.reshape(rows, Hkv, D), cs_rows[:, :half], cs_rows[:, half:], R)
     tol = 3e-6 if dtype == torch.float32 else 2.0 ** -8
     assert (many[0].double().cpu().reshape(rows, Hq, D) - qp).abs().max() <= tol * qp.abs().max()
     tab = tables.cpu()

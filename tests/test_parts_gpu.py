@@ -532,6 +532,130 @@ def test_a_step_that_fails_leaves_the_state_as_it_found_it(tmp_path):
         unregister("mixer", "toy_running_mean")
 
 
+def test_an_arrangement_defined_here_with_norms_after_its_parts(tmp_path):
+    """Another arrangement of a layer, registered from outside: norms after the mixer and after the feed-forward as well
+    as before them (x += post(mixer(pre(x))); x += post(ffn(pre(x)))), the two further norms being extra parts of the
+    block, and a softmax scale of the architecture's own.  Built, loaded from a folder and stepped in portions; compared
+    with the formulas written out."""
+    from dataclasses import dataclass as dc
+    from llmx_amd import Engine, RandomInit
+    from llmx_amd.engine import StepEntry
+    from llmx_amd.models import register_architecture, unregister_architecture
+    from llmx_amd.parts import BlockSpec, ModelSpec, PartSpec, RunEntry, build_part, register, unregister
+    from llmx_amd.weights.folder import write_random_model
+    from safetensors import safe_open
+
+    class SandwichBlock:
+        graph_safe = False      # it adds with a library call
+
+        def __init__(self, spec, c):
+            self.mixer_norm, self.mixer = build_part("norm", spec.mixer_norm, c), build_part("mixer", spec.mixer, c)
+            self.ffn_norm, self.ffn = build_part("norm", spec.ffn_norm, c), build_part("feed_forward", spec.ffn, c)
+            self.after = {name: build_part(family, part, c) for name, (family, part) in spec.extra.items()}
+
+        def parts(self):
+            return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, *self.after.values()]
+
+        def forward(self, step, x, cache):
+            T, E = x.shape
+            h = step.buf("sandwich.h", (T, E), step.act_dtype)
+            y = step.buf("sandwich.y", (T, E), torch.float32)
+            y32 = step.buf("sandwich.y32", (T, E), torch.float32)
+            for norm, part, post, is_mixer in ((self.mixer_norm, self.mixer, self.after["post_mixer_norm"], True),
+                                               (self.ffn_norm, self.ffn, self.after["post_ffn_norm"], False)):
+                norm.forward(step, x, h)
+                if is_mixer:
+                    part.forward(step, h, y, False, cache)
+                else:
+                    part.forward(step, h, y, False)
+                post.forward(step, y, None, y32)
+                x += y32
+
+    @dc(frozen=True)
+    class SandwichConfig:
+        vocab_size: int = 40
+        hidden_size: int = 32
+        layers: int = 2
+        architecture = "ToySandwichForCausalLM"
+
+        @classmethod
+        def from_json(cls, values):
+            return cls(**{k: v for k, v in values.items() if k != "architectures"})
+
+        def to_json(self):
+            return {"architectures": [self.architecture], "vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "layers": self.layers}
+
+    SCALE = 0.2
+
+    def assemble(c):
+        E = c.hidden_size
+        norm = lambda prefix: PartSpec("rmsnorm", {"width": E, "eps": 1e-5}, prefix)
+        blocks = []
+        for i in range(c.layers):
+            p = f"layers.{i}."
+            mixer = PartSpec("attention", {"hidden": E, "heads": 4, "kv_heads": 2, "head_dim": 8, "qk_norm": "none", "scale": SCALE,
+                                           "position": PartSpec("rotary_neox_partial", {"rotary_dim": 8, "theta": 100.0, "head_dim": 8,
+                                                                                        "pairing": "interleaved"})}, p + "attn.")
+            blocks.append(BlockSpec(norm(p + "n1."), mixer, norm(p + "n2."), PartSpec("dense_glu", {"hidden": E, "intermediate": 24}, p + "mlp."),
+                                    arrangement="toy_sandwich",
+                                    extra={"post_mixer_norm": ("norm", norm(p + "n1_post.")), "post_ffn_norm": ("norm", norm(p + "n2_post."))}))
+        return ModelSpec(architecture=c.architecture, vocab_size=c.vocab_size, hidden_size=E, max_positions=64,
+                         embedding=PartSpec("token_embedding", {"vocab": c.vocab_size, "hidden": E}, "embed."), blocks=blocks,
+                         run_order=[RunEntry(i, i) for i in range(c.layers)], final_norm=norm("norm."),
+                         head=PartSpec("linear", {"vocab": c.vocab_size, "hidden": E, "tied": True}, "head."))
+
+    def interleaved_rope(x, positions, theta):
+        """pairs (2j, 2j + 1) of each head rotated by position * theta^(-2j / D)"""
+        D = x.shape[-1]
+        j = torch.arange(D // 2, dtype=torch.float64)
+        angle = torch.tensor(positions, dtype=torch.float64)[:, None] * (1.0 / theta ** (2.0 * j / D))[None, :]
+        c, s = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+        a, b = x[..., 0::2], x[..., 1::2]
+        out = torch.empty_like(x)
+        out[..., 0::2] = a * c - b * s
+        out[..., 1::2] = b * c + a * s
+        return out
+
+    def plain(w, c, tokens):
+        T = len(tokens)
+        x = w["embed.weight"].double()[tokens]
+        for i in range(c.layers):
+            p = f"layers.{i}."
+            h = pm.rms_norm(x, w[p + "n1.weight"].double(), 1e-5)
+            q = interleaved_rope((h @ w[p + "attn.q_proj.weight"].double().T).view(T, 4, 8), list(range(T)), 100.0)
+            k = interleaved_rope((h @ w[p + "attn.k_proj.weight"].double().T).view(T, 2, 8), list(range(T)), 100.0)
+            v = (h @ w[p + "attn.v_proj.weight"].double().T).view(T, 2, 8)
+            q = q * (SCALE * math.sqrt(8.0))         # causal_attention divides by sqrt(D): scores become q.k * SCALE
+            y = pm.causal_attention(q, k, v).reshape(T, 32) @ w[p + "attn.o_proj.weight"].double().T
+            x = x + pm.rms_norm(y, w[p + "n1_post.weight"].double(), 1e-5)
+            h = pm.rms_norm(x, w[p + "n2.weight"].double(), 1e-5)
+            gate_up = torch.cat([w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"]]).double()
+            y = pm.swiglu_expert(h, gate_up, w[p + "mlp.down_proj.weight"].double())
+            x = x + pm.rms_norm(y, w[p + "n2_post.weight"].double(), 1e-5)
+        return pm.rms_norm(x, w["norm.weight"].double(), 1e-5) @ w["embed.weight"].double().T
+
+    register("block", "toy_sandwich", SandwichBlock, replace=True)
+    register_architecture("ToySandwichForCausalLM", SandwichConfig, assemble, replace=True)
+    try:
+        c = SandwichConfig()
+        folder = write_random_model(tmp_path / "sandwich", c, RandomInit(seed=9, std=0.3, norm_std=0.1, storage="float32"))
+        with safe_open(str(folder / "model.safetensors"), framework="pt") as f:
+            weights = {n: f.get_tensor(n) for n in f.keys()}
+        assert "layers.1.n2_post.weight" in weights           # the extra parts' tensors are the model's
+        tokens = [3, 14, 15, 9, 2, 6, 5, 35, 8, 9, 7, 9, 3, 2, 38, 4, 6, 2, 6]
+        want = plain(weights, c, tokens)
+        engine = Engine.load(folder, dtype="float32", kv_tokens=64, page_tokens=4, max_requests=2)
+        engine.add_request("w")
+        whole = engine.step([StepEntry("w", tokens, list(range(len(tokens))))]).clone()
+        assert (whole.cpu().double() - want).abs().max() < 3e-5 * want.abs().max()
+        engine.add_request("p")
+        rows = [engine.step([StepEntry("p", tokens[a:b], list(range(b - a)))]).clone() for a, b in ((0, 7), (7, 9), (9, 18), (18, 19))]
+        assert torch.equal(torch.cat(rows), whole)
+    finally:
+        unregister_architecture("ToySandwichForCausalLM")
+        unregister("block", "toy_sandwich")
+
+
 def test_run_order_names_a_layer_twice_and_shares_a_cache():
     """The run order is data: layer 1's weights run twice (with a cache each), and the last entry reads layer 0's cache."""
     from helpers import TINY_A, INIT_A, plain

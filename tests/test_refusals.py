@@ -105,3 +105,15 @@ def test_tiled_products_whose_offsets_pass_32_bits_leave_the_lean_forms():
     assert fit(65535, 128, 32768, 32768, EPI_STORE, 0, 1, 0) == 1
     assert fit(8 * 65536, 128, 32768, 32768, EPI_STORE, 16, 8, 0) == 0
     assert fit(8 * 65535, 128, 32768, 32768, EPI_STORE, 16, 8, 0) == 1
+
+
+def test_attention_options_outside_what_is_built_are_refused_by_name():
+    ctx = BuildContext(torch.float32, torch.device("cpu"), 64)
+    base = {"hidden": 64, "heads": 2, "kv_heads": 1, "head_dim": 16}
+    with pytest.raises(ValueError, match="rotary pairing 'thirds' is not one of"):
+        build_part("mixer", PartSpec("attention", {**base, "position": PartSpec("rotary_neox_partial", {"rotary_dim": 8, "theta": 1e4, "head_dim": 16,
+                                                                                                      "pairing": "thirds"})}), ctx)
+    with pytest.raises(ValueError, match="softmax scale must be positive"):
+        build_part("mixer", PartSpec("attention", {**base, "scale": 0.0}), ctx)
+    a = build_part("mixer", PartSpec("attention", {**base, "scale": 0.3}), ctx)
+    assert a.scale == pytest.approx(0.3) and build_part("mixer", PartSpec("attention", base), ctx).scale == pytest.approx(0.25)
