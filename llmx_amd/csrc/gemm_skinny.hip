@@ -68,7 +68,27 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
     const bf16_t* wp = W + (size_t)w_row * K + kg * 8;
     const bf16_t* up = (EPI == SK_SWIGLU) ? wp + (size_t)g.up_offset * K : wp;
 
+    // A wave's share of K is fetched in rounds of SK_UNROLL steps.  With one tile of rows the rounds take turns in two
+    // sets of registers: the next round is asked for before the present one is multiplied, so the wave waits for memory
+    // once, not once a round; and a round's weights are asked for before anything else the workgroup reads (the rows'
+    // list, the old values an adding epilogue joins), since their addresses depend on nothing but the strip.
+    constexpr bool PIPELINED = MT == 1 && EPI != SK_SWIGLU;   // the SwiGLU form streams two strips: a second set of registers costs it a wave a SIMD (measured slower)
+    struct Round {
+        bf16x8_t wf[SK_UNROLL], uf[SK_UNROLL], af[SK_UNROLL][MT];
+    };
+    auto fetch_weights = [&](int s, Round& f) {
+#pragma unroll
+        for (int u = 0; u < SK_UNROLL; ++u) {
+            const int k = (s + u) * 32 + kg * 8;
+            const bool in = (s + u) < s_end && k < K;
+            f.wf[u] = load_frag(wp + (size_t)(s + u) * 32, in);
+            if (EPI == SK_SWIGLU) f.uf[u] = load_frag(up + (size_t)(s + u) * 32, in);
+        }
+    };
+
     for (int m0 = row_begin; m0 < row_end; m0 += 16 * MT) {
+        Round r0, r1;
+        if (PIPELINED) fetch_weights(s_begin, r0);
         if (tid < MT * 16) {
             const int m = m0 + tid;
             int ra = -1, rc = -1;
@@ -98,30 +118,60 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
         for (int t = 0; t < MT; ++t)
 #pragma unroll
             for (int a = 0; a < NACC; ++a) acc[t][a] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-
-        for (int s = s_begin; s < s_end; s += SK_UNROLL) {
-            bf16x8_t wf[SK_UNROLL], uf[SK_UNROLL], af[SK_UNROLL][MT];
+        // what an adding epilogue joins: asked for now, used after the loop
+        float c_old[MT][4];
+        if (EPI == SK_ADD && wave == 0) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const int rc = rows_c[t * 16 + r];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool in = rc >= 0 && n0 + 4 * kg + i < g.N;
+                    c_old[t][i] = in ? ld((const TC*)g.C + (size_t)rc * g.ldc + n0 + 4 * kg + i) : 0.0f;
+                }
+            }
+        }
+        auto fetch_rows = [&](int s, Round& f) {
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u) {
                 const int k = (s + u) * 32 + kg * 8;
                 const bool in = (s + u) < s_end && k < K;
-                wf[u] = load_frag(wp + (size_t)(s + u) * 32, in);
-                if (EPI == SK_SWIGLU) uf[u] = load_frag(up + (size_t)(s + u) * 32, in);
-            }
 #pragma unroll
-            for (int u = 0; u < SK_UNROLL; ++u) {
-                const int k = (s + u) * 32 + kg * 8;
-                const bool in = (s + u) < s_end && k < K;
-#pragma unroll
-                for (int t = 0; t < MT; ++t) af[u][t] = load_frag(ap[t] + (size_t)(s + u) * 32, in && a_in[t]);
+                for (int t = 0; t < MT; ++t) f.af[u][t] = load_frag(ap[t] + (size_t)(s + u) * 32, in && a_in[t]);
             }
+        };
+        auto multiply = [&](const Round& f) {
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u) {
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
-                    acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], af[u][t], acc[t][0], 0, 0, 0);
-                    if (EPI == SK_SWIGLU) acc[t][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uf[u], af[u][t], acc[t][1], 0, 0, 0);
+                    acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.wf[u], f.af[u][t], acc[t][0], 0, 0, 0);
+                    if (EPI == SK_SWIGLU) acc[t][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.uf[u], f.af[u][t], acc[t][1], 0, 0, 0);
                 }
+            }
+        };
+        if (PIPELINED) {
+            fetch_rows(s_begin, r0);
+            for (int s = s_begin; s < s_end; s += 2 * SK_UNROLL) {
+                const bool second = s + SK_UNROLL < s_end;     // the same for the whole wave
+                if (second) {
+                    fetch_weights(s + SK_UNROLL, r1);
+                    fetch_rows(s + SK_UNROLL, r1);
+                }
+                multiply(r0);
+                if (second) {
+                    if (s + 2 * SK_UNROLL < s_end) {
+                        fetch_weights(s + 2 * SK_UNROLL, r0);
+                        fetch_rows(s + 2 * SK_UNROLL, r0);
+                    }
+                    multiply(r1);
+                }
+            }
+        } else {
+            for (int s = s_begin; s < s_end; s += SK_UNROLL) {
+                fetch_weights(s, r0);
+                fetch_rows(s, r0);
+                multiply(r0);
             }
         }
         // partial sums of the waves, added in wave order
@@ -157,7 +207,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
                     if (n0 + 4 * kg + i >= g.N) continue;
                     float x = v[0][i];
                     if (EPI == SK_SWIGLU) x = (x / (1.0f + expf(-x))) * v[1][i];
-                    if (EPI == SK_ADD) x = ld(c + i) + x;
+                    if (EPI == SK_ADD) x = c_old[t][i] + x;
                     st(c + i, x);
                 }
             }
@@ -166,12 +216,15 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
     }
 }
 
+// steps of K in a round of loads: with one tile of rows two rounds are in flight (see the kernel)
+#define SKINNY_ROUND(MT, EPI) 4
+
 template <int KS, int MT, int EPI, typename TC>
 static void launch_grouped(const SkinnyArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
     if (grouped)
-        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true, (MT == 1 && EPI != SK_SWIGLU) ? 8 : 4>), grid, dim3(64 * KS), 0, stream, g);
+        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true, SKINNY_ROUND(MT, EPI)>), grid, dim3(64 * KS), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false, (MT == 1 && EPI != SK_SWIGLU) ? 8 : 4>), grid, dim3(64 * KS), 0, stream, g);
+        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false, SKINNY_ROUND(MT, EPI)>), grid, dim3(64 * KS), 0, stream, g);
 }
 
 template <int KS, int MT>
