@@ -159,4 +159,79 @@ __device__ __forceinline__ float strided_squares(const float* __restrict__ row, 
     return s;
 }
 
+// RMSNorm of a few rows inside another kernel, with the bits the norm kernels give: y = x * (r * w),
+// r = 1 / sqrt(mean(x^2) + eps).  The norm kernels use 1,024 threads: thread v adds the squares of elements v, v + 1024,
+// ... in this order with fmaf, each wave of 64 threads adds its threads' sums with wave_sum, and the 16 waves' sums are
+// added in wave order.  Here a workgroup of NW waves does the same: wave w stands for the waves w, w + NW, ... of that
+// block.  store(row, i, y) receives every element.  Rows of at most 4,096 values with at least 4 waves are kept in
+// registers, all asked for (with the weights) before anything is added, so the workgroup waits for memory once a row.
+// scratch32: 32 floats of LDS.  The caller puts a barrier between the stores and their first read.
+template <int NW, typename Store>
+__device__ __forceinline__ void rms_rows_as_1024(const float* __restrict__ X, size_t ldx, int rows, int n, const float* __restrict__ w,
+                                                 float eps, float* scratch32, Store store) {
+    static_assert(NW == 1 || NW == 2 || NW == 4 || NW == 8 || NW == 16, "waves of the workgroup");
+    constexpr int VW = 16 / NW;       // waves of the 1,024-thread block that one wave stands for
+    constexpr int KEPT = 4;
+    const int wave = threadIdx.x / LLMX_WAVE, lane = threadIdx.x & (LLMX_WAVE - 1);
+    if (VW * KEPT <= 16 && n <= 1024 * KEPT) {
+        float nw[VW][KEPT];
+#pragma unroll
+        for (int j = 0; j < VW; ++j)
+#pragma unroll
+            for (int e = 0; e < KEPT; ++e) {
+                const int i = (wave + j * NW) * LLMX_WAVE + lane + e * 1024;
+                nw[j][e] = i < n ? w[i] : 0.0f;
+            }
+        for (int row = 0; row < rows; ++row) {
+            const float* x = X + (size_t)row * ldx;
+            float* scratch = scratch32 + 16 * (row & 1);   // rows take turns in two sets, so one barrier a row is enough
+            float v[VW][KEPT];
+#pragma unroll
+            for (int j = 0; j < VW; ++j)
+#pragma unroll
+                for (int e = 0; e < KEPT; ++e) {
+                    const int i = (wave + j * NW) * LLMX_WAVE + lane + e * 1024;
+                    v[j][e] = i < n ? x[i] : 0.0f;
+                }
+#pragma unroll
+            for (int j = 0; j < VW; ++j) {
+                float sq = 0.0f;     // an element past the end adds fmaf(0, 0, s) = s
+#pragma unroll
+                for (int e = 0; e < KEPT; ++e) sq = fmaf(v[j][e], v[j][e], sq);
+                sq = wave_sum(sq);
+                if (lane == 0) scratch[wave + j * NW] = sq;
+            }
+            __syncthreads();
+            float s = scratch[0];
+#pragma unroll
+            for (int u = 1; u < 16; ++u) s += scratch[u];
+            const float scale = 1.0f / sqrtf(s / (float)n + eps);
+#pragma unroll
+            for (int j = 0; j < VW; ++j)
+#pragma unroll
+                for (int e = 0; e < KEPT; ++e) {
+                    const int i = (wave + j * NW) * LLMX_WAVE + lane + e * 1024;
+                    if (i < n) store(row, i, v[j][e] * (scale * nw[j][e]));
+                }
+        }
+        return;
+    }
+    for (int row = 0; row < rows; ++row) {
+        const float* x = X + (size_t)row * ldx;
+        float* scratch = scratch32 + 16 * (row & 1);
+        for (int vw = wave; vw < 16; vw += NW) {
+            float sq = 0.0f;
+            for (int i = vw * LLMX_WAVE + lane; i < n; i += 1024) sq = fmaf(x[i], x[i], sq);
+            sq = wave_sum(sq);
+            if (lane == 0) scratch[vw] = sq;
+        }
+        __syncthreads();
+        float s = scratch[0];
+#pragma unroll
+        for (int u = 1; u < 16; ++u) s += scratch[u];
+        const float scale = 1.0f / sqrtf(s / (float)n + eps);
+        for (int i = threadIdx.x; i < n; i += LLMX_WAVE * NW) store(row, i, x[i] * (scale * w[i]));
+    }
+}
+
 #define LLMX_CHECK_LAUNCH() (int)hipGetLastError()

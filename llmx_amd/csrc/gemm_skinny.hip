@@ -10,6 +10,10 @@
 // Grouped form: blockIdx.y walks the experts that have rows; A's rows are gathered through the expert-sorted pair list
 // and C's rows scattered to the pairs.  The SwiGLU form streams a gate strip and the matching up strip together and
 // stores silu(gate) * up.
+//
+// Normed rows: for steps of very few rows the product can take the float32 residual rows and an RMSNorm's weights
+// instead of A; every workgroup forms the normed, rounded rows itself (in LDS) while its first weights travel, and no
+// norm kernel is launched.  The rows' values are the norm kernel's, bit for bit.
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -32,6 +36,11 @@ struct SkinnyArgs {
     int a_div;
     long w_group_stride;
     int up_offset;
+    // normed rows (NORMED): A is not read; row m of A is bf16(X[m] * (r_m * norm_w)), r_m the RMSNorm scale of X[m]
+    const float* X;
+    const float* norm_w;
+    float norm_eps;
+    int x_rows;
 };
 
 __device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p, bool in) {
@@ -40,12 +49,14 @@ __device__ __forceinline__ bf16x8_t load_frag(const bf16_t* p, bool in) {
     return __builtin_bit_cast(bf16x8_t, v);
 }
 
-template <int KS, int MT, int EPI, typename TC, bool GROUPED, int SK_UNROLL>
+template <int KS, int MT, int EPI, typename TC, bool GROUPED, int SK_UNROLL, bool NORMED>
 __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
     constexpr int NACC = (EPI == SK_SWIGLU) ? 2 : 1;
     __shared__ float red[KS > 1 ? KS : 1][MT * NACC][256];
     __shared__ int rows_a[MT * 16];
     __shared__ int rows_c[MT * 16];
+    __shared__ float norm_scratch[32];
+    extern __shared__ __attribute__((aligned(16))) bf16_t normed_rows[];   // NORMED: [x_rows][K]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 15, kg = lane >> 4;
@@ -86,9 +97,16 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
         }
     };
 
+    bool rows_normed = false;
     for (int m0 = row_begin; m0 < row_end; m0 += 16 * MT) {
         Round r0, r1;
         if (PIPELINED) fetch_weights(s_begin, r0);
+        if (NORMED && !rows_normed) {
+            // the step's rows, normed and rounded as the norm kernel stores them, while the first weights travel
+            rms_rows_as_1024<KS>(g.X, (size_t)K, g.x_rows, K, g.norm_w, g.norm_eps, norm_scratch,
+                                 [&](int row, int i, float y) { normed_rows[(size_t)row * K + i] = f32_to_bf16(y); });
+            rows_normed = true;   // the barrier below stands between these stores and the first read
+        }
         if (tid < MT * 16) {
             const int m = m0 + tid;
             int ra = -1, rc = -1;
@@ -111,7 +129,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
         for (int t = 0; t < MT; ++t) {
             const int ra = rows_a[t * 16 + r];
             a_in[t] = ra >= 0;
-            ap[t] = g.A + (size_t)(ra >= 0 ? ra : 0) * g.lda + kg * 8;
+            ap[t] = (NORMED ? normed_rows : g.A) + (size_t)(ra >= 0 ? ra : 0) * (NORMED ? K : g.lda) + kg * 8;
         }
         f32x4_t acc[MT][NACC];
 #pragma unroll
@@ -221,10 +239,21 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
 
 template <int KS, int MT, int EPI, typename TC>
 static void launch_grouped(const SkinnyArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
+    if (g.X) {
+        // normed rows: one tile of rows, the rows kept in LDS
+        if constexpr (MT == 1 && EPI != SK_ADD) {
+            const size_t lds = (size_t)g.x_rows * g.K * sizeof(bf16_t);
+            if (grouped)
+                hipLaunchKernelGGL((gemm_skinny_kernel<KS, 1, EPI, TC, true, SKINNY_ROUND(MT, EPI), true>), grid, dim3(64 * KS), lds, stream, g);
+            else
+                hipLaunchKernelGGL((gemm_skinny_kernel<KS, 1, EPI, TC, false, SKINNY_ROUND(MT, EPI), true>), grid, dim3(64 * KS), lds, stream, g);
+        }
+        return;
+    }
     if (grouped)
-        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true, SKINNY_ROUND(MT, EPI)>), grid, dim3(64 * KS), 0, stream, g);
+        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true, SKINNY_ROUND(MT, EPI), false>), grid, dim3(64 * KS), 0, stream, g);
     else
-        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false, SKINNY_ROUND(MT, EPI)>), grid, dim3(64 * KS), 0, stream, g);
+        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false, SKINNY_ROUND(MT, EPI), false>), grid, dim3(64 * KS), 0, stream, g);
 }
 
 template <int KS, int MT>
@@ -258,16 +287,27 @@ static int launch_mt(const SkinnyArgs& g, int mt, int epi, int c_dtype, dim3 gri
 // A and W bfloat16, K a multiple of 8, rows of A and W 16-byte aligned.  n_groups == 0: dense, M rows.
 // n_groups > 0: grouped; `max_active` bounds the groups that have rows (grid.y), `n_active` holds their number.
 // ks: waves that share a strip's K (1, 2, 4 or 8); chosen by the caller from N and K only.
+// Normed rows (X != null): A is ignored; X holds x_rows float32 rows of K values (x_rows = M, or for a grouped product
+// the rows that the pairs' A rows p / a_div name), norm_w the norm's K weights.  At most SKINNY_NORMED_MAX_ROWS rows
+// of at most SKINNY_NORMED_MAX_BYTES together, no adding epilogue; -2 otherwise.
+#define SKINNY_NORMED_MAX_ROWS 4
+#define SKINNY_NORMED_MAX_BYTES 32768
+extern "C" int llmx_gemm_skinny_normed_ok(int x_rows, int K) {
+    return x_rows >= 1 && x_rows <= SKINNY_NORMED_MAX_ROWS && K % 8 == 0 && (size_t)x_rows * K * sizeof(bf16_t) <= SKINNY_NORMED_MAX_BYTES ? 1 : 0;
+}
+
 extern "C" int llmx_gemm_skinny(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                                 int n_groups, int max_active, const int* active, const int* n_active, const int* group_offsets,
-                                const int* list, int a_div, long w_group_stride, int up_offset, hipStream_t stream) {
+                                const int* list, int a_div, long w_group_stride, int up_offset, const float* X, const float* norm_w,
+                                float norm_eps, int x_rows, hipStream_t stream) {
     if (N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
     if (!grouped && M <= 0) return 0;
     if (grouped && max_active <= 0) return 0;
+    if (X && (!norm_w || epi == SK_ADD || !llmx_gemm_skinny_normed_ok(x_rows, K) || (!grouped && x_rows != M))) return -2;
     SkinnyArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, active, n_active, group_offsets, list, a_div > 0 ? a_div : 1,
-                 w_group_stride, up_offset};
+                 w_group_stride, up_offset, X, norm_w, norm_eps, x_rows};
     dim3 grid((N + 15) / 16, grouped ? max_active : 1, 1);
     int mt = 1;
     if (!grouped && epi != SK_SWIGLU) mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);

@@ -13,11 +13,17 @@ struct SkinnyF32Args {
     float* C;
     int M, N, K, lda, ldc, add;
     long slice_stride;   // gridDim.z > 1: slice z of K's steps goes to C + z * slice_stride (the reader adds the slices in order)
+    // normed rows (NORMED): A holds the residual rows x; row m of the product's A is x[m] * (r_m * norm_w), unrounded,
+    // r_m the RMSNorm scale of x[m]: the norm kernel's float32 output, formed here by every workgroup (in LDS)
+    const float* norm_w;
+    float norm_eps;
 };
 
-template <int KS, int MT>
+template <int KS, int MT, bool NORMED>
 __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args g) {
     __shared__ float red[KS > 1 ? KS : 1][MT][256];
+    __shared__ float norm_scratch[32];
+    extern __shared__ __attribute__((aligned(16))) float normed_rows[];   // NORMED: [M][K]
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int r = lane & 15, kg = lane >> 4;
     const int n0 = blockIdx.x * 16;
@@ -30,6 +36,11 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
     float* C = g.C + (size_t)blockIdx.z * g.slice_stride;
     const float* wp = g.W + (size_t)min(n0 + r, g.N - 1) * K + kg * 4;
 
+    if (NORMED) {
+        rms_rows_as_1024<KS>(g.A, (size_t)g.lda, g.M, K, g.norm_w, g.norm_eps, norm_scratch,
+                             [&](int row, int i, float y) { normed_rows[(size_t)row * K + i] = y; });
+        __syncthreads();
+    }
     // blockIdx.y walks the rows in chunks of 16*MT, so many rows spread over the chip (each chunk reads the strip again, from L2)
     for (int m0 = blockIdx.y * 16 * MT; m0 < g.M; m0 += gridDim.y * 16 * MT) {
         const float* ap[MT];
@@ -38,7 +49,7 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_f32_kernel(SkinnyF32Args 
         for (int t = 0; t < MT; ++t) {
             const int m = m0 + t * 16 + r;
             a_in[t] = m < g.M;
-            ap[t] = g.A + (size_t)(a_in[t] ? m : 0) * g.lda + kg * 4;
+            ap[t] = (NORMED ? normed_rows : g.A) + (size_t)(a_in[t] ? m : 0) * (NORMED ? K : g.lda) + kg * 4;
         }
         f32x4_t acc[MT];
 #pragma unroll
@@ -321,11 +332,19 @@ __global__ void __launch_bounds__(512) gemm_rows_f32_lds_kernel(SkinnyF32Args g,
 
 // K a multiple of 4, rows 16-byte aligned.  ks: 1, 2, 4, 8 or 16 waves share a strip's K.  slices > 1: K's steps are
 // cut into `slices` runs first, run z written to C + z * slice_stride (no add then); the caller adds the runs in order.
+// norm_w != null: A holds residual rows and the product reads them through an RMSNorm with these weights (at most
+// SKF_NORMED_MAX_BYTES of rows, kept in LDS by every workgroup; -2 beyond).
+#define SKF_NORMED_MAX_BYTES 32768
+extern "C" int llmx_gemm_skinny_f32_normed_ok(int M, int K) {
+    return M >= 1 && M <= 16 && K % 4 == 0 && (size_t)M * K * sizeof(float) <= SKF_NORMED_MAX_BYTES ? 1 : 0;
+}
+
 extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, int M, int N, int K, int lda, int ldc, int add, int ks,
-                                    int slices, long slice_stride, hipStream_t stream) {
+                                    int slices, long slice_stride, const float* norm_w, float norm_eps, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % 4 || slices < 1 || slices > 64 || (slices > 1 && add)) return -2;
-    SkinnyF32Args g{A, W, C, M, N, K, lda, ldc, add, slice_stride};
+    if (norm_w && !llmx_gemm_skinny_f32_normed_ok(M, K)) return -2;
+    SkinnyF32Args g{A, W, C, M, N, K, lda, ldc, add, slice_stride, norm_w, norm_eps};
     int chunks = (M + 63) / 64;
     if (chunks > 1024) chunks = 1024;
     const dim3 grid((N + 15) / 16, M <= 64 ? 1 : chunks, slices);
@@ -346,8 +365,15 @@ extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, in
         }
         return LLMX_CHECK_LAUNCH();
     }
-#define SKF_LAUNCH(KS, MT) hipLaunchKernelGGL((gemm_skinny_f32_kernel<KS, MT>), grid, dim3(64 * KS), 0, stream, g)
-#define SKF_MT(KS) do { if (M <= 16) SKF_LAUNCH(KS, 1); else if (M <= 32) SKF_LAUNCH(KS, 2); else SKF_LAUNCH(KS, 4); } while (0)
+#define SKF_LAUNCH(KS, MT) hipLaunchKernelGGL((gemm_skinny_f32_kernel<KS, MT, false>), grid, dim3(64 * KS), 0, stream, g)
+#define SKF_MT(KS)                                                                                                            \
+    do {                                                                                                                      \
+        if (norm_w)                                                                                                           \
+            hipLaunchKernelGGL((gemm_skinny_f32_kernel<KS, 1, true>), grid, dim3(64 * KS), (size_t)M * K * sizeof(float), stream, g); \
+        else if (M <= 16) SKF_LAUNCH(KS, 1);                                                                                  \
+        else if (M <= 32) SKF_LAUNCH(KS, 2);                                                                                  \
+        else SKF_LAUNCH(KS, 4);                                                                                               \
+    } while (0)
     switch (ks) {
         case 1: SKF_MT(1); break;
         case 2: SKF_MT(2); break;

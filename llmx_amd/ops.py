@@ -67,9 +67,11 @@ def _declare(h) -> None:
         "llmx_route_topk": [P, P, I, L, P, P, P, I, I, I, I, I, F, P],
         "llmx_moe_align": [P, I, I, P, P, P, P, P, P, P, P],
         "llmx_route_topk_align": [P, P, I, L, P, P, P, I, I, I, I, F, P, P, P, P, P, P],
-        "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P],
+        "llmx_gemm_skinny": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, I, L, I, P, P, F, I, P],
+        "llmx_gemm_skinny_normed_ok": [I, I],
+        "llmx_gemm_skinny_f32_normed_ok": [I, I],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
-        "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P],
+        "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P, F, P],
         "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P],
         "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
@@ -166,18 +168,53 @@ def _skinny_ok(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int)
             and (epilogue != EPI_ADD or c.dtype == torch.float32))
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False) -> None:
-    """c[M,N] (+)= a[M,K] @ w[N,K]^T, accumulated in float32; EPI_SWIGLU: c = silu(a @ w[:N]^T) * (a @ w[N:]^T)."""
+class NormedRows:
+    """The float32 rows x seen through an RMSNorm (weight, eps), not yet computed: a product that reads its rows this way
+    forms norm(x) itself while its weights travel (steps of very few rows only), and no norm kernel runs."""
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor, eps: float):
+        self.x, self.weight, self.eps = x, weight, float(eps)
+        self.shape = x.shape
+
+    def args(self):
+        return _dev(self.x, "x", torch.float32), _dev(self.weight, "norm weight", torch.float32, (self.x.shape[1],)), self.eps, self.x.shape[0]
+
+
+_NO_NORM = (0, 0, 0.0, 0)
+
+
+def gemm_takes_normed_rows(rows: int, w: torch.Tensor, c_dtype: torch.dtype, epilogue: int = EPI_STORE, grouped: bool = False) -> bool:
+    """Whether gemm / grouped_gemm would form `rows` normed rows itself for this product (the weight-streaming kernel runs
+    and the rows fit its LDS)."""
+    K = w.shape[-1]
+    return (w.dtype == torch.bfloat16 and epilogue != EPI_ADD and K % 8 == 0 and bool(lib().llmx_gemm_skinny_normed_ok(rows, K))
+            and (grouped and rows <= SKINNY_MAX_GROUPED_ROWS or not grouped))
+
+
+def gemm_f32_takes_normed_rows(rows: int, w: torch.Tensor) -> bool:
+    return bool(lib().llmx_gemm_skinny_f32_normed_ok(rows, w.shape[1]))
+
+
+def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False) -> None:
+    """c[M,N] (+)= a[M,K] @ w[N,K]^T, accumulated in float32; EPI_SWIGLU: c = silu(a @ w[:N]^T) * (a @ w[N:]^T).
+    `a` may be NormedRows where gemm_takes_normed_rows says so: the product reads bfloat16(norm(x))."""
     M, K = a.shape
     N = w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]   # swiglu: w holds gate rows, then up rows
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
+    if isinstance(a, NormedRows):
+        if not gemm_takes_normed_rows(M, w, c.dtype, epilogue):
+            raise KernelError("gemm: normed rows are not taken for this product")
+        _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
+                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *a.args(), _stream()),
+               "gemm_skinny (normed rows)")
+        return
     # beyond 16 rows a product wide enough to fill the chip with tiles streams its weights faster through the tiled kernel
     # (the LM head); both kernels give a row the same bits
     skinny = M <= 16 or (M <= SKINNY_MAX_ROWS and -(-N // 128) < TILE_FILL)
     if not force_generic and skinny and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()),
+                                      _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, _stream()),
                "gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
@@ -206,12 +243,21 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         raise KernelError("grouped_gemm: more pairs than rows")
     if token_rows is None:
         token_rows = n_pairs
+    if isinstance(a, NormedRows):
+        if active is None or n_active is None or not gemm_takes_normed_rows(a.shape[0], w, c.dtype, epilogue, grouped=True):
+            raise KernelError("grouped_gemm: normed rows are not taken for this product")
+        _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
+                                      _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
+                                      _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
+                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *a.args(), _stream()),
+               "grouped_gemm_skinny (normed rows)")
+        return
     if (not force_generic and active is not None and n_active is not None and _skinny_ok(a, w, c, epilogue)
             and token_rows <= SKINNY_MAX_GROUPED_ROWS):
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
                                       _dev(n_active, "n_active", torch.int32, (1,)), _dev(offsets, "offsets", torch.int32, (G + 1,)),
-                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, _stream()),
+                                      _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, _stream()),
                "grouped_gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
@@ -492,7 +538,7 @@ def gemm_f32_slices(N: int, K: int) -> int:
     return s
 
 
-def gemm_f32(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, add: bool = False, parts: Optional[torch.Tensor] = None) -> None:
+def gemm_f32(a, w: torch.Tensor, c: torch.Tensor, add: bool = False, parts: Optional[torch.Tensor] = None) -> None:
     """c[M,N] (+)= a[M,K] @ w[N,K]^T, everything float32, on the float32 matrix instruction (the router's product).
     A row's bits depend on the shape of w only.  K a multiple of 4; otherwise the universal kernel runs.
     `parts` [gemm_f32_slices(N, K), M, N] with more than one slice: K's runs are written there instead of c, spread over
@@ -501,6 +547,9 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, add: bool = Fals
     N = w.shape[0]
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm_f32 shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
+    normed = isinstance(a, NormedRows)    # the product reads norm(x), unrounded, formed by its own workgroups
+    if normed and not gemm_f32_takes_normed_rows(M, w):
+        raise KernelError("gemm_f32: normed rows are not taken for this product")
     if K % 4:
         if parts is not None:
             raise KernelError("gemm_f32: partial sums need K to be a multiple of 4")
@@ -517,8 +566,10 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, add: bool = Fals
     while ks < 16 and n_strips * slices * ks < 1024 and steps // (ks * 2) >= (8 if slices == 1 else 3):   # from w's shape only
         ks *= 2
     target = parts if parts is not None else c
-    _check(lib().llmx_gemm_skinny_f32(_dev(a, "a", torch.float32), _dev(w, "w", torch.float32), _dev(target, "c", torch.float32), M, N, K, K, N,
-                                      1 if add else 0, ks, slices, M * N, _stream()), "gemm_f32")
+    _check(lib().llmx_gemm_skinny_f32(_dev(a.x if normed else a, "a", torch.float32), _dev(w, "w", torch.float32), _dev(target, "c", torch.float32),
+                                      M, N, K, K, N, 1 if add else 0, ks, slices, M * N,
+                                      _dev(a.weight, "norm weight", torch.float32, (K,)) if normed else 0, a.eps if normed else 0.0, _stream()),
+           "gemm_f32")
 
 
 def sample_all(scores: torch.Tensor, temp: torch.Tensor, unit: torch.Tensor, out: torch.Tensor, min_p: Optional[torch.Tensor] = None,

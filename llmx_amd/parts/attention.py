@@ -81,6 +81,9 @@ class Attention(Mixer):
             self.q_norm = tensors[self.name("q_norm.weight")]
             self.k_norm = tensors[self.name("k_norm.weight")]
 
+    def takes_deferred_norm(self, step):
+        return ops.gemm_takes_normed_rows(step.rows, self.wqkv, torch.float32)
+
     def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
         T = step.rows
         act = step.act_dtype

@@ -71,6 +71,11 @@ class Norm(Part):
         """out (activation type) and/or out32 (float32) = norm of the float32 rows x (of rows x[pick] when given)."""
         raise NotImplementedError
 
+    def deferred(self, x: torch.Tensor):
+        """The norm of x as a description that a product can carry out itself (ops.NormedRows), or None when this norm
+        has no such form.  A block offers it to the part that follows; the part says whether it takes it."""
+        return None
+
 
 class PositionEncoding(Part):
     """Owns what a mixer needs to place a row at its position; for rotary forms a table of cos and sin, and which dims
@@ -98,6 +103,10 @@ class Mixer(Part):
     #: True when forward wants the normed rows also as float32 (`h32`)
     wants_f32_input = False
 
+    def takes_deferred_norm(self, step) -> bool:
+        """Whether, for this step, forward accepts a Norm.deferred() description as h and h32 in place of tensors."""
+        return False
+
     def cache_need(self) -> Union[KVNeed, StateNeed, None]:
         return None
 
@@ -109,6 +118,10 @@ class Mixer(Part):
 
 class FeedForward(Part):
     wants_f32_input = False
+
+    def takes_deferred_norm(self, step) -> bool:
+        """As Mixer.takes_deferred_norm."""
+        return False
 
     def forward(self, step, h: torch.Tensor, out: torch.Tensor, accumulate: bool, h32: Optional[torch.Tensor] = None) -> None:
         raise NotImplementedError

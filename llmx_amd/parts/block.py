@@ -24,14 +24,24 @@ class PreNormBlock:
     def parts(self):
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
 
-    def forward(self, step, x: torch.Tensor, cache: LayerCache) -> None:
+    @staticmethod
+    def normed(step, norm, part, x):
+        """(h, h32) for `part`: the norm's description where the norm has one and the part carries it out in its own
+        products for this step (a step of very few rows, where a norm kernel of its own costs more than its work);
+        otherwise the norm runs here."""
+        later = norm.deferred(x)
+        if later is not None and part.takes_deferred_norm(step):
+            return later, later
         T, E = x.shape
         h = step.buf("block.h", (T, E), step.act_dtype)
-        h32 = step.buf("block.h32", (T, E), torch.float32) if self.mixer.wants_f32_input else None
-        self.mixer_norm.forward(step, x, h, h32)
+        h32 = step.buf("block.h32", (T, E), torch.float32) if part.wants_f32_input else None
+        norm.forward(step, x, h, h32)
+        return h, h32
+
+    def forward(self, step, x: torch.Tensor, cache: LayerCache) -> None:
+        h, h32 = self.normed(step, self.mixer_norm, self.mixer, x)
         self.mixer.forward(step, h, x, True, cache, h32)
-        h32 = step.buf("block.h32", (T, E), torch.float32) if self.ffn.wants_f32_input else None
-        self.ffn_norm.forward(step, x, h, h32)
+        h, h32 = self.normed(step, self.ffn_norm, self.ffn, x)
         self.ffn.forward(step, h, x, True, h32)
 
 

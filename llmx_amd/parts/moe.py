@@ -78,6 +78,10 @@ class RoutedExperts(FeedForward):
         self.w_gate_up = tensors[self.name("experts.gate_up_proj")]
         self.w_down = tensors[self.name("experts.down_proj")]
 
+    def takes_deferred_norm(self, step):
+        return (ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU, grouped=True)
+                and ops.gemm_f32_takes_normed_rows(step.rows, self.w_router))
+
     def forward(self, step, h, out, accumulate, h32=None):
         T, X, k = step.rows, self.experts, self.top_k
         z = step.buf("experts.router_logits", (T, X), torch.float32)
@@ -123,6 +127,9 @@ class DenseGLU(FeedForward):
     def load(self, tensors):
         self.w_gate_up = torch.cat([tensors[self.name("gate_proj.weight")], tensors[self.name("up_proj.weight")]], dim=0).contiguous()
         self.w_down = tensors[self.name("down_proj.weight")]
+
+    def takes_deferred_norm(self, step):
+        return ops.gemm_takes_normed_rows(step.rows, self.w_gate_up, step.act_dtype, ops.EPI_SWIGLU)
 
     def forward(self, step, h, out, accumulate, h32=None):
         act = step.buf("glu.act", (step.rows, self.intermediate), step.act_dtype)

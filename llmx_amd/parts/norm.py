@@ -34,5 +34,8 @@ class RMSNorm(Norm):
     def forward(self, step, x, out, out32=None, pick=None):
         ops.rmsnorm(x, self.weight, self.eps, out, out32, pick)
 
+    def deferred(self, x):
+        return ops.NormedRows(x, self.weight, self.eps)
+
 
 register("norm", "rmsnorm", RMSNorm)

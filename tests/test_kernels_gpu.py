@@ -263,6 +263,57 @@ def test_gemm_swiglu(M, F, K, dtype):
         assert torch.equal(c1[0], c[M - 1]), "a row's bits depend on how many rows the product has"
 
 
+@pytest.mark.parametrize("rows,N,K,eps", [(1, 8192, 3072, 1e-6), (2, 48, 104, 1e-5), (4, 1536, 4096, 1e-6), (3, 640, 4104, 1e-2), (1, 100000, 64, 1e-6),
+                                          (1, 24, 8200, 1e-6)])
+def test_products_that_norm_their_rows_give_the_bits_of_norm_then_product(rows, N, K, eps):
+    """A product handed NormedRows forms the RMSNorm itself: the same bits as the norm kernel followed by the product,
+    for the plain product, the SwiGLU form, the routed form and the float32 product, with rows kept in registers
+    (K <= 4096 with four waves or more) and read twice (beyond)."""
+    o = ops()
+    x = rnd(rows, K, scale=3.0)
+    nw = 1.0 + rnd(K, seed=5, scale=0.3)
+    lazy = o.NormedRows(x, nw, eps)
+    h = torch.empty(rows, K, dtype=torch.bfloat16, device=DEV)
+    h32 = torch.empty(rows, K, dtype=torch.float32, device=DEV)
+    o.rmsnorm(x, nw, eps, h, h32)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=1, scale=0.2)
+    assert o.gemm_takes_normed_rows(rows, w, torch.float32) and not o.gemm_takes_normed_rows(5, w, torch.float32)
+    assert not o.gemm_takes_normed_rows(rows, w, torch.float32, o.EPI_ADD)
+    want, got = torch.empty(rows, N, dtype=torch.float32, device=DEV), torch.full((rows, N), 7.0, dtype=torch.float32, device=DEV)
+    o.gemm(h, w, want)
+    o.gemm(lazy, w, got)
+    assert torch.equal(got, want)
+    if N % 2 == 0:
+        want, got = torch.empty(rows, N // 2, dtype=torch.bfloat16, device=DEV), torch.zeros(rows, N // 2, dtype=torch.bfloat16, device=DEV)
+        o.gemm(h, w, want, o.EPI_SWIGLU)
+        o.gemm(lazy, w, got, o.EPI_SWIGLU)
+        assert torch.equal(got, want)
+    with pytest.raises(o.KernelError):
+        o.gemm(lazy, w, got, o.EPI_ADD)
+    # float32 (the router's product), also as partial sums
+    if N <= 1536 and o.gemm_f32_takes_normed_rows(rows, w):
+        w32 = rnd(N, K, seed=2, scale=0.2)
+        want, got = torch.empty(rows, N, dtype=torch.float32, device=DEV), torch.zeros(rows, N, dtype=torch.float32, device=DEV)
+        slices = o.gemm_f32_slices(N, K)
+        pw = torch.empty(slices, rows, N, dtype=torch.float32, device=DEV) if slices > 1 else None
+        pg = torch.zeros(slices, rows, N, dtype=torch.float32, device=DEV) if slices > 1 else None
+        o.gemm_f32(h32, w32, want, parts=pw)
+        o.gemm_f32(lazy, w32, got, parts=pg)
+        assert torch.equal(pg, pw) if slices > 1 else torch.equal(got, want)
+    # routed: k pairs a row over X experts
+    X, k, F = 6, 3, min(N, 96) // 2
+    ids = routed_setup(rows, X, k, rows + K).to(DEV)
+    wg = rnd(X, 2 * F, K, dtype=torch.bfloat16, seed=3, scale=0.2)
+    counts, offsets = torch.empty(X, dtype=torch.int32, device=DEV), torch.empty(X + 1, dtype=torch.int32, device=DEV)
+    pairs, active = torch.empty(rows * k, dtype=torch.int32, device=DEV), torch.empty(X, dtype=torch.int32, device=DEV)
+    n_active = torch.empty(1, dtype=torch.int32, device=DEV)
+    o.moe_align(ids, X, counts, offsets, pairs, active, n_active)
+    want, got = torch.zeros(rows * k, F, dtype=torch.bfloat16, device=DEV), torch.zeros(rows * k, F, dtype=torch.bfloat16, device=DEV)
+    o.grouped_gemm(h, wg, want, offsets, pairs, k, o.EPI_SWIGLU, active, n_active, token_rows=rows)
+    o.grouped_gemm(lazy, wg, got, offsets, pairs, k, o.EPI_SWIGLU, active, n_active, token_rows=rows)
+    assert torch.equal(got, want) and float(want.float().abs().max()) > 0
+
+
 def routed_setup(T, X, k, seed):
     rng = random.Random(seed)
     ids = torch.tensor([rng.sample(range(X), k) for _ in range(T)], dtype=torch.int32)
