@@ -37,6 +37,14 @@ class GroupSpec:
             return whole
         return min(whole, self.pages_for(self.window + step_tokens) + 1)
 
+    def pool_pages(self, total_tokens: int, requests: int, step_tokens: Optional[int]) -> int:
+        """Pages of a pool made for `total_tokens` tokens: all of them for a group that keeps every key; for a window,
+        when the most tokens a step brings of one request is known, what `requests` requests can hold at once."""
+        whole = self.pages_for(total_tokens)
+        if self.window is None or step_tokens is None:
+            return whole
+        return min(whole, requests * self.peak_pages(total_tokens, step_tokens))
+
 
 @dataclass
 class _Request:

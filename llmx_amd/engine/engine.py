@@ -55,10 +55,13 @@ class _StepGraph:
 class Engine:
     def __init__(self, config, spec: ModelSpec, dtype: Union[str, torch.dtype] = "bfloat16", *, kv_tokens: int,
                  page_tokens: int = 16, max_requests: int = 8, device: Union[str, torch.device] = "cuda:0", weights=None,
-                 graphs: bool = True):
+                 graphs: bool = True, step_tokens: Optional[int] = None):
         """`weights(engine)` returns the device tensors by name; it runs before the cache is allocated, so weights that
         do not fit the model are refused before anything large exists.  `graphs`: steps of single decoded tokens are
-        replayed as HIP graphs once their shape has been seen twice (see `_run`)."""
+        replayed as HIP graphs once their shape has been seen twice (see `_run`).  `step_tokens`: the most tokens a
+        step brings of one request, when the caller keeps to one (a scheduler's budget): a cache group that keeps only
+        a window of keys then gets a pool for `max_requests` windows instead of `kv_tokens` tokens; a step that brings
+        more finds the pool short and is refused like any step that runs out of pages."""
         if not torch.cuda.is_available():
             raise RuntimeError("llmx_amd runs on a GPU only: no GPU is visible and there is no CPU path")
         ops.lib()  # fail now, loudly, when the kernel library is missing
@@ -71,6 +74,9 @@ class Engine:
         self.page_tokens = int(page_tokens)
         self.kv_tokens = -(-int(kv_tokens) // self.page_tokens) * self.page_tokens
         self.max_requests = int(max_requests)
+        if step_tokens is not None and step_tokens < 1:
+            raise ValueError("step_tokens must be at least 1")
+        self.step_tokens = step_tokens
         self.max_positions = min(spec.max_positions, self.kv_tokens)
         torch.cuda.set_device(self.device)
         ctx = BuildContext(self.act_dtype, self.device, self.max_positions)
@@ -147,11 +153,12 @@ class Engine:
                 self._index_in_group.append(-1)
         self.group_needs = keys
         groups = [GroupSpec(f"kv{g}", self.page_tokens, n_pages, need.window) for g, need in enumerate(keys)]
+        groups = [replace(g, n_pages=g.pool_pages(self.kv_tokens, self.max_requests, self.step_tokens)) for g in groups]
         # a model with per-request state steps into a second slot, so that a step that fails leaves the state as it was
         self._stateful = any(isinstance(need, StateNeed) for need in needs)
         self.cache = CacheManager(groups, self.max_requests, shadow_slots=self._stateful)
         # [cache in group, K|V, page, kv head, token in page * head dim]; keys are [token][dim], values [dim][token]
-        self._kv = [torch.zeros((counts[g], 2, n_pages, need.kv_heads, self.page_tokens * need.head_dim), dtype=self.act_dtype,
+        self._kv = [torch.zeros((counts[g], 2, groups[g].n_pages, need.kv_heads, self.page_tokens * need.head_dim), dtype=self.act_dtype,
                                 device=self.device) for g, need in enumerate(keys)]
         self._state: List[Optional[torch.Tensor]] = []
         for need in needs:
@@ -166,8 +173,8 @@ class Engine:
                 store = self._kv[g][self._index_in_group[e.cache]]
                 need = keys[g]
                 self._layer_caches.append(LayerCache(
-                    group=g, k=store[0].view(n_pages, need.kv_heads, self.page_tokens, need.head_dim),
-                    v=store[1].view(n_pages, need.kv_heads, need.head_dim, self.page_tokens), writes=e.writes))
+                    group=g, k=store[0].view(groups[g].n_pages, need.kv_heads, self.page_tokens, need.head_dim),
+                    v=store[1].view(groups[g].n_pages, need.kv_heads, need.head_dim, self.page_tokens), writes=e.writes))
             else:
                 self._layer_caches.append(LayerCache(state=self._state[e.cache], writes=e.writes))
 

@@ -87,6 +87,26 @@ def test_window_gives_pages_back_as_it_passes_them():
     assert m.pages_in_use(0) == 0 and m.pages_in_use(1) == 0
     g = GroupSpec("win", 4, 64, window=6)
     assert g.peak_pages(1000, 8) == g.pages_for(14) + 1 and GroupSpec("all", 4, 64).peak_pages(1000, 8) == 250
+    # a pool made for windows: what the requests hold at once when a step brings at most 8 tokens; without that bound,
+    # or without a window, or when the whole context is shorter than that, a page for every token
+    assert g.pool_pages(1000, 3, 8) == 3 * (g.pages_for(14) + 1) and g.pool_pages(1000, 3, None) == 250
+    assert GroupSpec("all", 4, 64).pool_pages(1000, 3, 8) == 250 and g.pool_pages(12, 3, 8) == 3
+
+
+def test_a_pool_made_for_windows_is_enough_for_steps_within_the_bound():
+    """Three requests decode and take portions of at most 8 tokens through a windowed pool of pool_pages(...) pages:
+    no step runs out of pages, in any interleaving tried."""
+    g = GroupSpec("win", 4, 0, window=6)
+    pages = g.pool_pages(10_000, 3, 8)
+    rng = random.Random(5)
+    m = CacheManager([GroupSpec("win", 4, pages, window=6)], max_requests=3)
+    for r in "abc":
+        m.open(r)
+    for _ in range(600):
+        r = rng.choice("abc")
+        m.prepare(r, rng.choice([1, 1, 2, 5, 8]))
+        m.commit(r)
+        assert m.pages_in_use(0) <= pages
 
 
 @pytest.mark.parametrize("seed", range(8))

@@ -757,3 +757,19 @@ def test_window_attention_gives_pages_back(dtype, page):
         engine.end_request("w")
     engine.end_request("p")
     assert engine.cache.pages_in_use(0) == 0 and engine.cache.pages_in_use(1) == 0
+    # told the most tokens a step brings of a request, the engine makes the window's pool for windows, not for contexts;
+    # portions within the bound give the same logits through it
+    small = Engine(cfg, spec, dtype, kv_tokens=160, page_tokens=page, max_requests=2, step_tokens=12,
+                   weights=lambda e: load_weights(e.model.tensor_specs(set(files.names())), files, e.device, exact))
+    pools = [g.n_pages for g in small.cache.groups]
+    assert pools[0] == 160 // page and pools[1] == 2 * (-(-(W + 12) // page) + 1) < pools[0]
+    assert small._kv[1].shape[2] == pools[1]
+    small.add_request("q")
+    small.add_request("other")
+    cut = []
+    for a in range(0, 70, 12):
+        cut.append(small.step([StepEntry("q", tokens[a:a + 12], list(range(len(tokens[a:a + 12])))),
+                               StepEntry("other", tokens[69 - a:69 - a + 1], [])])[:len(tokens[a:a + 12])].clone())
+    assert (torch.cat(cut).cpu().double() - want).abs().max() <= tol * want.abs().max()
+    if exact:
+        assert torch.equal(torch.cat(cut), torch.cat(rows))
