@@ -52,6 +52,10 @@ def _add_sampling(p):
 def _add_exec(p):
     p.add_argument("--dtype", choices=["f32", "bf16", "float32", "bfloat16"], default="bf16", action=_Once,
                    help="bf16: the serving path; f32: everything in true 32-bit")
+    p.add_argument("--device", default="cuda:0", action=_Once, help="the GPU to run on (default %(default)s)")
+    p.add_argument("--cache-type-k", "-ctk", choices=["f32", "bf16", "f16"], default=None, action=_Once,
+                   help="type of the cached keys: the type of --dtype (the attention kernels read q, k and v in one type)")
+    p.add_argument("--cache-type-v", "-ctv", choices=["f32", "bf16", "f16"], default=None, action=_Once, help="type of the cached values: as --cache-type-k")
     p.add_argument("--ubatch", type=int, default=512, action=_Once, help="tokens a step takes at most (default %(default)s)")
     p.add_argument("--kv-tokens", type=int, default=0, action=_Once, help="the cache's token budget; 0 sizes it to the run")
     p.add_argument("--page-tokens", type=int, default=16, action=_Once, help="tokens a cache page holds (default %(default)s)")
@@ -65,6 +69,12 @@ def _add_exec(p):
 def _model_and_prompt(a, command: str):
     """The positionals are MODEL [PROMPT], or [PROMPT] alone when --config names the model."""
     words = list(a.words)
+    short = {"float32": "f32", "bfloat16": "bf16"}.get(a.dtype, a.dtype)
+    for flag, value in (("--cache-type-k", a.cache_type_k), ("--cache-type-v", a.cache_type_v)):
+        if value is not None and value != short:
+            raise SystemExit2(f"{flag} {value}: the cache is kept in the type of the activations (--dtype {short}); another cache type is not built")
+    if not re.fullmatch(r"cuda(:\d+)?", a.device):
+        raise SystemExit2(f"--device {a.device}: this engine runs on a GPU only (cuda or cuda:N)")
     if (a.config is None) != (a.random is None):
         raise SystemExit2(f"{command}: --config and --random go together")
     if a.config is None:
@@ -91,6 +101,7 @@ def _config_of(a):
 def _engine(a, cfg, **options):
     """The engine of the model folder, or of the configuration with weights generated on the device."""
     from .engine import Engine
+    options["device"] = a.device
     if a.model is not None:
         return Engine.load(a.model, dtype=a.dtype, **options)
     from .weights import RandomInit
@@ -243,7 +254,10 @@ def cmd_replay(a) -> int:
 
 
 def cmd_bench(rest) -> int:
-    """bench.py at the repository's root, with its own flags."""
+    """With --model (or --config and --random): the reference's model bench, cmd_bench_model.  Otherwise bench.py at
+    the repository's root, with its own flags: the decode and prefill record at the real layer sizes."""
+    if any(w == "--model" or w.startswith("--model=") or w == "--config" or w.startswith("--config=") for w in rest):
+        return cmd_bench_model(list(rest))
     import runpy
     script = Path(__file__).resolve().parent.parent / "bench.py"
     old = sys.argv
@@ -254,6 +268,94 @@ def cmd_bench(rest) -> int:
         return int(e.code or 0)
     finally:
         sys.argv = old
+    return 0
+
+
+def bench_model_parser() -> argparse.ArgumentParser:
+    ap = argparse.ArgumentParser(prog="llmx bench", description="prompt and decode rates of a model (the reference's `bench --model`)")
+    ap.add_argument("--model", default=None, action=_Once, help="a model folder")
+    ap.add_argument("--p", type=int, default=64, action=_Once, help="prompt tokens (default %(default)s)")
+    ap.add_argument("--n", type=int, default=64, action=_Once, help="decoded tokens (default %(default)s)")
+    ap.add_argument("--r", type=int, default=3, action=_Once, help="timed repetitions of each test (default %(default)s)")
+    ap.add_argument("--seqs", type=int, default=1, action=_Once, help="sequences decoding together (default %(default)s)")
+    ap.add_argument("--depth", type=int, default=0, action=_Once, help="tokens of history each test runs after; one sequence only (default %(default)s)")
+    _add_exec(ap)
+    return ap
+
+
+def cmd_bench_model(argv) -> int:
+    """`llmx bench --model DIR [--p 64] [--n 64] [--r 3] [--seqs 1] [--depth 0]`, the reference's model bench
+    (/root/reference/src/cli/main.cpp:67-75,1192-1287): the rate of a prompt of p tokens after `depth` tokens of
+    history, and of n decoded tokens (one sequence after the history; or `seqs` sequences together, each after the
+    prompt, with each step's logits read on the host as a server would), as mean and standard deviation over r runs
+    after one run that is not counted.  `--config JSON --random SEED` stands for the folder as elsewhere."""
+    import statistics
+    import torch
+    from .engine import StepEntry
+    a = bench_model_parser().parse_args(argv)
+    a.words = [a.model] if a.model is not None else []
+    _model_and_prompt(a, "bench")
+    for name in ("p", "n", "r", "seqs"):
+        if getattr(a, name) < 1:
+            raise SystemExit2(f"bench: --{name} must be at least 1")
+    if a.depth < 0 or (a.depth and a.seqs > 1):
+        raise SystemExit2("bench: --depth is at least 0 and goes with one sequence")
+    cfg = _config_of(a)
+    P, G, R, S, D = a.p, a.n, a.r, a.seqs, a.depth
+    reach = P + G if S > 1 else D + max(P, G)
+    pages = -(-reach // a.page_tokens) + 1
+    engine = _engine(a, cfg, kv_tokens=a.kv_tokens or S * pages * a.page_tokens, page_tokens=a.page_tokens, max_requests=S)
+    vocab = cfg.vocab_size
+    prompt, gen, history = _lcg_ids(P, vocab, 12345), _lcg_ids(G, vocab, 777), _lcg_ids(D, vocab, 4242)
+
+    def feed(request, ids, want_last):
+        for s in range(0, len(ids), a.ubatch):
+            part = ids[s:s + a.ubatch]
+            last = s + a.ubatch >= len(ids)
+            engine.step([StepEntry(request, part, [len(part) - 1] if want_last and last else [])])
+
+    def fresh(request):
+        engine.add_request(request)
+        if D:
+            feed(request, history, False)
+        torch.cuda.synchronize()
+
+    def timed(work, tokens):
+        t0 = time.perf_counter()
+        work()
+        torch.cuda.synchronize()
+        return tokens / (time.perf_counter() - t0)
+
+    def pp():
+        fresh(0)
+        rate = timed(lambda: feed(0, prompt, True), P)
+        engine.end_request(0)
+        return rate
+
+    def tg():
+        if S == 1:
+            fresh(0)
+            rate = timed(lambda: [engine.step([StepEntry(0, [t], [0])]) for t in gen], G)
+            engine.end_request(0)
+            return rate
+        for q in range(S):
+            engine.add_request(q)
+            feed(q, prompt, True)
+        torch.cuda.synchronize()
+        rate = timed(lambda: [engine.step([StepEntry(q, [t], [0]) for q in range(S)]).cpu() for t in gen], G * S)
+        for q in range(S):
+            engine.end_request(q)
+        return rate
+
+    def report(what, n, rates):
+        sd = statistics.stdev(rates) if len(rates) > 1 else 0.0
+        at = f" @ d{D}" if D else ""
+        print(f"bench: {what}{n}{at}  {statistics.mean(rates):8.2f} +- {sd:.2f} tok/s  ({len(rates)} runs)")
+
+    pp()
+    tg()
+    report("pp", P, [pp() for _ in range(R)])
+    report(f"x{S} tg" if S > 1 else "tg", G, [tg() for _ in range(R)])
     return 0
 
 
@@ -308,7 +410,7 @@ def build_parser():
     r.add_argument("--bias-range", type=float, default=0.0)
     r.add_argument("--storage", choices=["bfloat16", "float32"], default="bfloat16")
     r.set_defaults(run=cmd_random)
-    b = sub.add_parser("bench", help="decode and prefill throughput of a random-weight model (see bench.py)")
+    b = sub.add_parser("bench", help="--model DIR --p --n --r --seqs --depth: prompt and decode rates of a model; without a model: bench.py's record")
     b.add_argument("rest", nargs=argparse.REMAINDER)
     b.set_defaults(run=lambda a: cmd_bench(a.rest))
     return ap

@@ -75,3 +75,31 @@ def test_config_and_random_name_a_model_without_a_folder(tmp_path, capsys):
     bad.write_text(json.dumps({"architectures": ["MiniMaxM3ForCausalLM"], "head_dim": 16}))
     rc, _, err = run(["generate", "--config", str(bad), "--random", "0", "1,2"], capsys)
     assert rc == 1 and "missing key" in err
+
+
+def test_cache_types_and_device_are_the_reference_flags_with_this_engines_limits(tmp_path, capsys):
+    """`--cache-type-k/-ctk`, `--cache-type-v/-ctv` and `--device` exist as in the reference
+    (/root/reference/src/cli/main.cpp:120,544-555); the cache has the activations' type and the device is a GPU, and
+    anything else is a usage error before a model is read."""
+    rc, _, err = run(["generate", str(tmp_path), "1,2", "-ctk", "f32"], capsys)
+    assert rc == 2 and "--cache-type-k f32" in err and "--dtype bf16" in err
+    rc, _, err = run(["generate", str(tmp_path), "1,2", "--dtype", "f32", "--cache-type-v", "f16"], capsys)
+    assert rc == 2 and "--cache-type-v f16" in err
+    rc, _, err = run(["logits", str(tmp_path), "1,2", "--device", "cpu"], capsys)
+    assert rc == 2 and "runs on a GPU only" in err
+    # the matching type passes these checks (and then fails on the empty folder, not on usage)
+    rc, _, err = run(["generate", str(tmp_path), "1,2", "--dtype", "f32", "-ctk", "f32", "-ctv", "f32", "--device", "cuda:0"], capsys)
+    assert rc == 1 and "cache-type" not in err
+
+
+def test_bench_with_a_model_is_the_reference_bench(capsys):
+    """`bench --model` is parsed here (the reference's --p --n --r --seqs --depth, main.cpp:67-75); without a model
+    the flags go on to bench.py."""
+    rc, _, err = run(["bench", "--model", "m", "--p", "0"], capsys)
+    assert rc == 2 and "--p must be at least 1" in err
+    rc, _, err = run(["bench", "--model", "m", "--seqs", "2", "--depth", "8"], capsys)
+    assert rc == 2 and "goes with one sequence" in err
+    rc, _, err = run(["bench", "--model", "m", "--p", "4", "--p", "5"], capsys)
+    assert rc == 2 and "given twice" in err
+    rc, _, err = run(["bench", "--config", "c.json", "--n", "3"], capsys)
+    assert rc == 2 and "--config and --random go together" in err

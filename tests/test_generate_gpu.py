@@ -200,6 +200,33 @@ def test_command_line_runs_a_configuration_with_random_weights(tmp_path):
     assert int(lg.stdout.strip().split("\n")[-1].split()[0]) == want[0]
 
 
+def test_command_line_bench_of_a_model(tmp_path):
+    """`llmx bench --model DIR --p --n --r --seqs --depth` prints the reference's lines (`bench: pp16 ...`,
+    `bench: tg8 ...`, `bench: x3 tg8 ...`, ` @ d40` after a history; /root/reference/src/cli/main.cpp:1261-1270) and
+    leaves no request open between its runs (every run opens its requests anew in a pool made for one run)."""
+    import re
+    exe = os.path.join(ROOT, "bin", "llmx")
+    one = subprocess.run([exe, "bench", "--model", model_folder("A16"), "--p", "16", "--n", "8", "--r", "2", "--depth", "40", "--ubatch", "12"],
+                         capture_output=True, text=True, timeout=300)
+    assert one.returncode == 0, one.stderr[-2000:]
+    lines = [l for l in one.stdout.strip().split("\n") if l.startswith("bench: ")]
+    assert len(lines) == 2
+    assert re.fullmatch(r"bench: pp16 @ d40 +[0-9.]+ \+- [0-9.]+ tok/s  \(2 runs\)", lines[0]), lines[0]
+    assert re.fullmatch(r"bench: tg8 @ d40 +[0-9.]+ \+- [0-9.]+ tok/s  \(2 runs\)", lines[1]), lines[1]
+    import json
+    from helpers import TINY_B
+    from llmx_amd import MiniMaxM3Config
+    path = tmp_path / "config.json"
+    path.write_text(json.dumps(MiniMaxM3Config(**TINY_B).to_json()))
+    many = subprocess.run([exe, "bench", "--config", str(path), "--random", "1", "--p", "9", "--n", "5", "--r", "1", "--seqs", "3", "--dtype", "f32",
+                           "--page-tokens", "8"], capture_output=True, text=True, timeout=300)
+    assert many.returncode == 0, many.stderr[-2000:]
+    lines = [l for l in many.stdout.strip().split("\n") if l.startswith("bench: ")]
+    assert lines[0].startswith("bench: pp9 ") and lines[1].startswith("bench: x3 tg5 ") and lines[1].endswith("(1 runs)")
+    bad = subprocess.run([exe, "bench", "--model", model_folder("A16"), "--seqs", "2", "--depth", "5"], capture_output=True, text=True, timeout=120)
+    assert bad.returncode == 2 and "--depth" in bad.stderr
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_many_requests_through_a_small_pool_equal_their_runs_alone(dtype):
     """Thirty requests of drawn lengths, counts and settings, through pages for about three of them: requests wait for
