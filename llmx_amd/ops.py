@@ -183,16 +183,30 @@ class NormedRows:
 _NO_NORM = (0, 0, 0.0, 0)
 
 
-def gemm_takes_normed_rows(rows: int, w: torch.Tensor, c_dtype: torch.dtype, epilogue: int = EPI_STORE, grouped: bool = False) -> bool:
-    """Whether gemm / grouped_gemm would form `rows` normed rows itself for this product (the weight-streaming kernel runs
+NORMED_ROWS_PAY = 1   # rows up to which a product that norms its own rows beats the norm kernel (measured: 1 row 3.07 -> 2.98 ms a step,
+                      # 2 rows 4.03 -> 4.23, 4 rows 6.01 -> 6.11: the rows are formed one after the other in every workgroup)
+
+
+def gemm_can_norm_rows(rows: int, w: torch.Tensor, c_dtype: torch.dtype, epilogue: int = EPI_STORE, grouped: bool = False) -> bool:
+    """Whether gemm / grouped_gemm can form `rows` normed rows itself for this product (the weight-streaming kernel runs
     and the rows fit its LDS)."""
     K = w.shape[-1]
     return (w.dtype == torch.bfloat16 and epilogue != EPI_ADD and K % 8 == 0 and bool(lib().llmx_gemm_skinny_normed_ok(rows, K))
             and (grouped and rows <= SKINNY_MAX_GROUPED_ROWS or not grouped))
 
 
-def gemm_f32_takes_normed_rows(rows: int, w: torch.Tensor) -> bool:
+def gemm_f32_can_norm_rows(rows: int, w: torch.Tensor) -> bool:
     return bool(lib().llmx_gemm_skinny_f32_normed_ok(rows, w.shape[1]))
+
+
+def gemm_takes_normed_rows(rows: int, w: torch.Tensor, c_dtype: torch.dtype, epilogue: int = EPI_STORE, grouped: bool = False) -> bool:
+    """What a part answers a block that offers a deferred norm: the product can form the rows, and for so few rows that
+    it pays."""
+    return rows <= NORMED_ROWS_PAY and gemm_can_norm_rows(rows, w, c_dtype, epilogue, grouped)
+
+
+def gemm_f32_takes_normed_rows(rows: int, w: torch.Tensor) -> bool:
+    return rows <= NORMED_ROWS_PAY and gemm_f32_can_norm_rows(rows, w)
 
 
 def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False) -> None:
@@ -203,7 +217,7 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
     if isinstance(a, NormedRows):
-        if not gemm_takes_normed_rows(M, w, c.dtype, epilogue):
+        if not gemm_can_norm_rows(M, w, c.dtype, epilogue):
             raise KernelError("gemm: normed rows are not taken for this product")
         _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *a.args(), _stream()),
@@ -244,7 +258,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
     if token_rows is None:
         token_rows = n_pairs
     if isinstance(a, NormedRows):
-        if active is None or n_active is None or not gemm_takes_normed_rows(a.shape[0], w, c.dtype, epilogue, grouped=True):
+        if active is None or n_active is None or not gemm_can_norm_rows(a.shape[0], w, c.dtype, epilogue, grouped=True):
             raise KernelError("grouped_gemm: normed rows are not taken for this product")
         _check(lib().llmx_gemm_skinny(0, _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), G, min(G, n_pairs), _dev(active, "active", torch.int32, (G,)),
@@ -548,7 +562,7 @@ def gemm_f32(a, w: torch.Tensor, c: torch.Tensor, add: bool = False, parts: Opti
     if w.shape[1] != K or tuple(c.shape) != (M, N):
         raise KernelError(f"gemm_f32 shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, c {tuple(c.shape)}")
     normed = isinstance(a, NormedRows)    # the product reads norm(x), unrounded, formed by its own workgroups
-    if normed and not gemm_f32_takes_normed_rows(M, w):
+    if normed and not gemm_f32_can_norm_rows(M, w):
         raise KernelError("gemm_f32: normed rows are not taken for this product")
     if K % 4:
         if parts is not None:

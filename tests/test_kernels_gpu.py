@@ -277,8 +277,9 @@ def test_products_that_norm_their_rows_give_the_bits_of_norm_then_product(rows, 
     h32 = torch.empty(rows, K, dtype=torch.float32, device=DEV)
     o.rmsnorm(x, nw, eps, h, h32)
     w = rnd(N, K, dtype=torch.bfloat16, seed=1, scale=0.2)
-    assert o.gemm_takes_normed_rows(rows, w, torch.float32) and not o.gemm_takes_normed_rows(5, w, torch.float32)
-    assert not o.gemm_takes_normed_rows(rows, w, torch.float32, o.EPI_ADD)
+    assert o.gemm_can_norm_rows(rows, w, torch.float32) and not o.gemm_can_norm_rows(5, w, torch.float32)
+    assert not o.gemm_can_norm_rows(rows, w, torch.float32, o.EPI_ADD)
+    assert o.gemm_takes_normed_rows(rows, w, torch.float32) == (rows <= o.NORMED_ROWS_PAY)   # what parts answer: only where it pays
     want, got = torch.empty(rows, N, dtype=torch.float32, device=DEV), torch.full((rows, N), 7.0, dtype=torch.float32, device=DEV)
     o.gemm(h, w, want)
     o.gemm(lazy, w, got)
@@ -291,7 +292,7 @@ def test_products_that_norm_their_rows_give_the_bits_of_norm_then_product(rows, 
     with pytest.raises(o.KernelError):
         o.gemm(lazy, w, got, o.EPI_ADD)
     # float32 (the router's product), also as partial sums
-    if N <= 1536 and o.gemm_f32_takes_normed_rows(rows, w):
+    if N <= 1536 and o.gemm_f32_can_norm_rows(rows, w):
         w32 = rnd(N, K, seed=2, scale=0.2)
         want, got = torch.empty(rows, N, dtype=torch.float32, device=DEV), torch.zeros(rows, N, dtype=torch.float32, device=DEV)
         slices = o.gemm_f32_slices(N, K)
