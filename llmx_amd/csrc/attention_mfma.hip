@@ -10,7 +10,9 @@
 //   o^T[dim][col] = V^T[16 dims x 32 keys] . P^T[32 keys x 16 cols], 4 chunks of 32 keys added in key order
 // The value pages are stored transposed ([dim][token]) so that V^T's rows are contiguous, and a chunk's 32 keys are
 // assigned to the product's k-slots in the order the score accumulators hold them: no data moves between lanes
-// except the softmax's reductions over the 4 lanes of a column.
+// except the softmax's reductions over the 4 lanes of a column.  The keys of a chunk are dealt to the rows of its two
+// score tiles so that this order is the keys' own (chunk_key below): a lane's 8 weights of a chunk belong to 8
+// consecutive keys, and the values' operand is 16 contiguous bytes of a dim's row.
 // The segments' (m, l, o) are folded in key order with one formula (fold_segment).  A long context of a decoding row is
 // shared out over several items that write their segments' (m, l, o), which a second kernel folds; a prompt tile folds
 // its segments in registers.  Every form calls the same functions with the same values, so a column's result is the
@@ -43,8 +45,14 @@ __device__ __forceinline__ bool frag_in(int s, int g) {
     return g < 2;
 }
 
-// Scores of one chunk (32 keys, two tiles of 16) against the tile's columns.  kf: the keys, qf: the columns' queries.
-// Lane (column c = l % 16, group g = l / 16) gets keys 16u + 4g + i of the chunk in s[u][i].
+// Which of a chunk's 32 keys sits in row r of the chunk's score tile u: 8 (r / 4) + 4 u + r % 4.  The product hands lane
+// (column c, group g) the rows 4g .. 4g + 3 of a tile, so the lane gets the keys 8g + 4u + i: over both tiles the keys
+// 8g .. 8g + 7, which are the k-slots 8g .. 8g + 7 that the lane feeds the value product.
+__device__ __forceinline__ int chunk_key(int u, int r) { return 8 * (r >> 2) + 4 * u + (r & 3); }
+
+// Scores of one chunk (32 keys, two tiles of 16 rows) against the tile's columns.  kf: the keys (row r of tile u holds
+// key chunk_key(u, r)), qf: the columns' queries.  Lane (column c = l % 16, group g = l / 16) gets keys 8g + 4u + i of
+// the chunk in s[u][i].
 template <int DT>
 __device__ __forceinline__ void chunk_scores(const bf16x8_t (&kf)[2][(DT + 1) / 2], const bf16x8_t (&qf)[(DT + 1) / 2], f32x4_t& s0, f32x4_t& s1) {
     constexpr int QS = (DT + 1) / 2;
@@ -57,7 +65,7 @@ __device__ __forceinline__ void chunk_scores(const bf16x8_t (&kf)[2][(DT + 1) / 
     }
 }
 
-// Softmax of a column over one segment.  s[2v + u][i]: the score of key 32v + 16u + 4g + i; ok bit 8v + 4u + i says
+// Softmax of a column over one segment.  s[2v + u][i]: the score of key 32v + 8g + 4u + i; ok bit 8v + 4u + i says
 // whether that key counts for the lane's column (MASKED false: all 128 count for every column and the selects fall
 // away; the sums are the same).  Gives the segment's maximum m, its sum l and the weights as the value product's
 // operands pf[v] (chunk v).  A column without a key that counts gets m = -inf, l = 0, weights 0.
@@ -115,7 +123,7 @@ __device__ __forceinline__ void fold_segment(const f32x4_t (&o)[DT], float m, fl
 }
 
 // The keys of a segment that count for a lane's column: key in [lo_col, p_col], below key_end; bit 8v + 4u + i for key
-// seg0 + 32v + 16u + 4g + i.
+// seg0 + 32v + 8g + 4u + i.
 __device__ __forceinline__ uint32_t segment_mask(int seg0, int g, bool col_ok, int lo_col, int p_col, int key_end) {
     uint32_t ok = 0u;
     if (!col_ok) return ok;
@@ -123,7 +131,7 @@ __device__ __forceinline__ uint32_t segment_mask(int seg0, int g, bool col_ok, i
     for (int t = 0; t < 8; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int key = seg0 + 16 * t + 4 * g + i;
+            const int key = seg0 + 32 * (t >> 1) + 8 * g + 4 * (t & 1) + i;
             if (key <= p_col && key >= lo_col && key < key_end) ok |= 1u << (4 * t + i);
         }
     return ok;
@@ -228,12 +236,14 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
             }
         }
     };
-    // K fragments of chunk v of the segment: lane (key c of each tile, dims 32s + 8g ..)
+    // K fragments of chunk v of the segment: lane (row c of each score tile: key chunk_key(u, c) of the chunk, which
+    // lies in the chunk's second 16 keys (their own page) from row 8 on; dims 32s + 8g ..)
     auto load_keys = [&](const int (&pages)[8], const int (&subs)[8], int v, bf16x8_t (&kf)[2][QS]) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int page = pages[2 * v + u];
-            const bf16_t* src = a.k_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * bt + subs[2 * v + u] + c) * D + 8 * g;
+            const int page = c >= 8 ? pages[2 * v + 1] : pages[2 * v];
+            const int sub = c >= 8 ? subs[2 * v + 1] : subs[2 * v];
+            const bf16_t* src = a.k_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * bt + sub + (chunk_key(u, c) & 15)) * D + 8 * g;
 #pragma unroll
             for (int s = 0; s < QS; ++s) {
                 u32x4_t x = {0u, 0u, 0u, 0u};
@@ -242,17 +252,16 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
             }
         }
     };
-    // V^T fragments of chunk v: lane (dim 16dt + c, keys 4g .. 4g+3 of each tile)
+    // V^T fragments of chunk v: lane (dim 16dt + c, keys 8g .. 8g + 7 of the chunk: 16 bytes of the dim's row in the
+    // page of the chunk's first or second 16 keys)
     auto load_values = [&](const int (&pages)[8], const int (&subs)[8], int v, bf16x8_t (&vf)[DT]) {
-        const int page0 = pages[2 * v], page1 = pages[2 * v + 1];
-        const bf16_t* src0 = a.v_cache + (((size_t)(page0 < 0 ? 0 : page0) * Hkv + kvh) * D + c) * bt + subs[2 * v] + 4 * g;
-        const bf16_t* src1 = a.v_cache + (((size_t)(page1 < 0 ? 0 : page1) * Hkv + kvh) * D + c) * bt + subs[2 * v + 1] + 4 * g;
+        const int page = g >= 2 ? pages[2 * v + 1] : pages[2 * v];
+        const int sub = g >= 2 ? subs[2 * v + 1] : subs[2 * v];
+        const bf16_t* src = a.v_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * D + c) * bt + sub + 8 * (g & 1);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            u32x2_t v0 = {0u, 0u}, v1 = {0u, 0u};
-            if (page0 >= 0) v0 = *reinterpret_cast<const u32x2_t*>(src0 + (size_t)16 * dt * bt);
-            if (page1 >= 0) v1 = *reinterpret_cast<const u32x2_t*>(src1 + (size_t)16 * dt * bt);
-            const u32x4_t x = {v0[0], v0[1], v1[0], v1[1]};
+            u32x4_t x = {0u, 0u, 0u, 0u};
+            if (page >= 0) x = *reinterpret_cast<const u32x4_t*>(src + (size_t)16 * dt * bt);
             vf[dt] = __builtin_bit_cast(bf16x8_t, x);
         }
     };
@@ -288,11 +297,8 @@ __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_atten
         if (seg0 + AM_SEG - 1 <= p_first && seg0 >= lo_last && all_in) {
             segment_softmax<false>(s, 0xffffffffu, a.scale, m, l, pf);   // every key counts for every column
         } else {
-            uint32_t ok = segment_mask(seg0, g, col_ok, lo_col, p_col, key_end);
-#pragma unroll
-            for (int tl = 0; tl < 8; ++tl)
-                if (pages[tl] < 0) ok &= ~(0xfu << (4 * tl));
-            segment_softmax<true>(s, ok, a.scale, m, l, pf);
+            // (a tile without a page lies wholly at or after key_end, which the mask leaves out)
+            segment_softmax<true>(s, segment_mask(seg0, g, col_ok, lo_col, p_col, key_end), a.scale, m, l, pf);
         }
         f32x4_t o[DT];
 #pragma unroll
@@ -380,10 +386,8 @@ __global__ void __launch_bounds__(256) paged_attention_split4_kernel(AttnMfmaArg
     struct Loaded {
         bf16x8_t kf[2][QS];
         bf16x8_t vf[4][2];
-        int tile_in;   // bit tl: tile tl of the segment holds keys of the item
     };
     auto fetch = [&](int seg0, Loaded& x) {
-        x.tile_in = 0;
         int pages[8], subs[8];
 #pragma unroll
         for (int tl = 0; tl < 8; ++tl) {
@@ -391,19 +395,19 @@ __global__ void __launch_bounds__(256) paged_attention_split4_kernel(AttnMfmaArg
             const bool in = key0 < key_end;
             pages[tl] = in ? table[key0 / bt] : -1;
             subs[tl] = key0 % bt;
-            if (in) x.tile_in |= 1 << tl;
         }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            // tile 2 wave + u; selected without indexing the arrays by a run-time value
+            // row c of score tile u of chunk `wave`: key chunk_key(u, c), in the chunk's first (rows below 8) or second
+            // 16 keys; the page selected without indexing the arrays by a run-time value
             int page = -1, sub = 0;
 #pragma unroll
             for (int tl = 0; tl < 8; ++tl)
-                if (tl == 2 * wave + u) {
+                if (tl == 2 * wave + (c >= 8 ? 1 : 0)) {
                     page = pages[tl];
                     sub = subs[tl];
                 }
-            const bf16_t* src = a.k_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * bt + sub + c) * D + 8 * g;
+            const bf16_t* src = a.k_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * bt + sub + (chunk_key(u, c) & 15)) * D + 8 * g;
 #pragma unroll
             for (int s = 0; s < QS; ++s) {
                 u32x4_t v = {0u, 0u, 0u, 0u};
@@ -413,16 +417,14 @@ __global__ void __launch_bounds__(256) paged_attention_split4_kernel(AttnMfmaArg
         }
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const int page0 = pages[2 * v], page1 = pages[2 * v + 1];
+            const int page = g >= 2 ? pages[2 * v + 1] : pages[2 * v];
+            const int sub = g >= 2 ? subs[2 * v + 1] : subs[2 * v];
 #pragma unroll
             for (int q = 0; q < 2; ++q) {
                 const int dim = 32 * wave + 16 * q + c;
-                const bf16_t* src0 = a.v_cache + (((size_t)(page0 < 0 ? 0 : page0) * Hkv + kvh) * D + dim) * bt + subs[2 * v] + 4 * g;
-                const bf16_t* src1 = a.v_cache + (((size_t)(page1 < 0 ? 0 : page1) * Hkv + kvh) * D + dim) * bt + subs[2 * v + 1] + 4 * g;
-                u32x2_t v0 = {0u, 0u}, v1 = {0u, 0u};
-                if (page0 >= 0) v0 = *reinterpret_cast<const u32x2_t*>(src0);
-                if (page1 >= 0) v1 = *reinterpret_cast<const u32x2_t*>(src1);
-                const u32x4_t both = {v0[0], v0[1], v1[0], v1[1]};
+                const bf16_t* src = a.v_cache + (((size_t)(page < 0 ? 0 : page) * Hkv + kvh) * D + dim) * bt + sub + 8 * (g & 1);
+                u32x4_t both = {0u, 0u, 0u, 0u};
+                if (page >= 0) both = *reinterpret_cast<const u32x4_t*>(src);
                 x.vf[v][q] = __builtin_bit_cast(bf16x8_t, both);
             }
         }
@@ -436,11 +438,9 @@ __global__ void __launch_bounds__(256) paged_attention_split4_kernel(AttnMfmaArg
         if (more) fetch(seg0 + AM_SEG, next);     // the next segment travels while this one is worked on
         f32x4_t s0, s1;
         chunk_scores<DT>(cur.kf, qf, s0, s1);
-        // the keys that count for the lane's column: bits 8 v + 4 u + i of the segment's mask, tiles without keys taken out
-        uint32_t ok = segment_mask(seg0, g, col_ok, lo_col, p_col, key_end);
-#pragma unroll
-        for (int tl = 0; tl < 8; ++tl)
-            if (!((cur.tile_in >> tl) & 1)) ok &= ~(0xfu << (4 * tl));
+        // the keys that count for the lane's column: bits 8 v + 4 u + i of the segment's mask (a tile without a page
+        // lies wholly at or after key_end, which the mask leaves out)
+        const uint32_t ok = segment_mask(seg0, g, col_ok, lo_col, p_col, key_end);
         const uint32_t mine = (ok >> (8 * wave)) & 0xffu;
         float top = -INFINITY;
 #pragma unroll
@@ -516,7 +516,7 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
     constexpr int QS = (DT + 1) / 2;
     constexpr int D = 16 * DT;
     constexpr int K_LD = D + 8;              // bf16 elements a key's row takes in LDS
-    constexpr int V_LD = AM_SEG + 4;         // bf16 elements a dim's row of 128 keys takes in LDS: 66 words, so 16 dims' 8-byte reads miss each other's banks
+    constexpr int V_LD = AM_SEG + 8;         // bf16 elements a dim's row of 128 keys takes in LDS: 68 words, so 16 dims' 16-byte reads miss each other's banks
     __shared__ __attribute__((aligned(16))) bf16_t Ks[AM_SEG * K_LD];
     __shared__ __attribute__((aligned(16))) bf16_t Vs[D * V_LD];
     __shared__ int ranges[4][2];
@@ -572,6 +572,9 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
     // (page and place in the page) are the same for all threads and are kept by a cursor that steps from tile to tile.
     constexpr int PER_TILE = (2 * D + 255) / 256;   // rounds a tile takes: 2 D chunks of keys (and of values)
     constexpr int ROUNDS = 8 * PER_TILE;
+    // Keys are placed in LDS in the order the score tiles want their rows: a chunk's key kc = 8a + 4u + b (chunk_key)
+    // lies in row 16u + 4a + b of the chunk's 32 rows, so row c of tile u is read as before.  For key k of a tile's 16
+    // that is row 4 (k / 8) + k % 4 + 16 ((k / 4) % 2), plus 8 in the chunk's second tile.
     u32x4_t stage[ROUNDS];
     int k_off[PER_TILE], k_lds[PER_TILE], v_off[PER_TILE], v_lds[PER_TILE];
 #pragma unroll
@@ -580,7 +583,7 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
         const bool in = ch < 2 * D;
         const int key = ch / (D / 8), dc = ch % (D / 8);
         k_off[r] = key * D + 8 * dc;
-        k_lds[r] = in ? key * K_LD + 8 * dc : -1;
+        k_lds[r] = in ? (4 * (key >> 3) + (key & 3) + 16 * ((key >> 2) & 1)) * K_LD + 8 * dc : -1;
         const int d = ch >> 1, half = ch & 1;
         v_off[r] = d * bt + 8 * half;
         v_lds[r] = in ? d * V_LD + 8 * half : -1;
@@ -614,7 +617,7 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
         for (int tl = 0; tl < 8; ++tl)
 #pragma unroll
             for (int r = 0; r < PER_TILE; ++r)
-                if (k_lds[r] >= 0) *reinterpret_cast<u32x4_t*>(&Ks[16 * tl * K_LD + k_lds[r]]) = stage[tl * PER_TILE + r];
+                if (k_lds[r] >= 0) *reinterpret_cast<u32x4_t*>(&Ks[(32 * (tl >> 1) + 8 * (tl & 1)) * K_LD + k_lds[r]]) = stage[tl * PER_TILE + r];
     };
     auto fetch_values = [&]() {   // of the segment whose keys were fetched last
 #pragma unroll
@@ -634,13 +637,9 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
         for (int tl = 0; tl < 8; ++tl)
 #pragma unroll
             for (int r = 0; r < PER_TILE; ++r)
-                if (v_lds[r] >= 0) {
-                    u32x2_t* dst = reinterpret_cast<u32x2_t*>(&Vs[v_lds[r] + 16 * tl]);
-                    dst[0] = u32x2_t{stage[tl * PER_TILE + r][0], stage[tl * PER_TILE + r][1]};
-                    dst[1] = u32x2_t{stage[tl * PER_TILE + r][2], stage[tl * PER_TILE + r][3]};
-                }
+                if (v_lds[r] >= 0) *reinterpret_cast<u32x4_t*>(&Vs[v_lds[r] + 16 * tl]) = stage[tl * PER_TILE + r];
     };
-    const int k_at = c * K_LD + 8 * g, v_at = c * V_LD + 4 * g;   // where the lane's fragments start
+    const int k_at = c * K_LD + 8 * g, v_at = c * V_LD + 8 * g;   // where the lane's fragments start
 
     if (block_begin >= block_end) return;
     fetch_keys(block_begin);
@@ -684,12 +683,8 @@ __global__ void __launch_bounds__(256, DT <= 8 ? 2 : 1) paged_attention_tiles_ke
             for (int v = 0; v < 4; ++v) {
                 bf16x8_t vf[DT];
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(&Vs[v_at + 16 * dt * V_LD + 32 * v]);
-                    const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(&Vs[v_at + 16 * dt * V_LD + 32 * v + 16]);
-                    const u32x4_t x = {v0[0], v0[1], v1[0], v1[1]};
-                    vf[dt] = __builtin_bit_cast(bf16x8_t, x);
-                }
+                for (int dt = 0; dt < DT; ++dt)   // keys 32v + 8g .. of dim 16dt + c
+                    vf[dt] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Vs[v_at + 16 * dt * V_LD + 32 * v]));
                 chunk_values<DT>(vf, pf[v], o);
             }
             fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
@@ -711,7 +706,8 @@ __device__ __forceinline__ void attention_load_to_lds(const void* base, uint32_t
 // KV head.  A segment's keys and values go from the pages straight into LDS (no registers in between), a whole segment
 // ahead: while segment n is worked on, segment n+1 is on its way into the other half of LDS; one barrier a segment.
 // LDS rows are not padded; the 16-byte chunks are placed so that the operand reads miss each other's banks:
-//   keys:   row = key (256 bytes), chunk c (8 dims) at place c ^ (key & 15)
+//   keys:   a row of 256 bytes a key, in the order the score tiles want them (a chunk's key 8a + 4u + b in row
+//           16u + 4a + b of the chunk's 32), chunk c (8 dims) at place c ^ (row & 15)
 //   values: per tile of 16 keys a block of 128 dims x 32 bytes, the two chunks of dim d swapped when (d >> 3) & 1
 // and the lane that fills a place fetches the chunk that belongs there.  Per column the arithmetic is that of the
 // kernels above (the same functions on the same values).
@@ -784,11 +780,13 @@ __global__ void __launch_bounds__(512) paged_attention_tiles128_kernel(AttnMfmaA
         const bf16_t* vb = a.v_cache + ((size_t)pg * Hkv + kvh) * D * bt + sub;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            // keys 4 j .. 4 j + 3 of the tile: lane is key 4 j + l / 16 (row 16 wave + that), place l % 16 holds chunk
-            // place ^ (key & 15)
+            // keys 4 j .. 4 j + 3 of the tile: lane is key 4 j + l / 16; as keys 16 (wave % 2) + 4 j + .. of their chunk
+            // they go to 4 rows in a run, from row 32 (wave / 2) + 16 (j % 2) + 8 (wave % 2) + 4 (j / 2); place l % 16
+            // holds chunk place ^ (row & 15)
             const int key = 4 * j + (lane >> 4);
-            const uint32_t off = (uint32_t)((key * D + 8 * ((lane & 15) ^ key)) * sizeof(bf16_t));
-            attention_load_to_lds(kb, off, &Ks[buf * K_SEG + (16 * wave + 4 * j) * D]);
+            const int row = 16 * (j & 1) + 8 * (wave & 1) + 4 * (j >> 1) + (lane >> 4);
+            const uint32_t off = (uint32_t)((key * D + 8 * ((lane & 15) ^ (row & 15))) * sizeof(bf16_t));
+            attention_load_to_lds(kb, off, &Ks[buf * K_SEG + (32 * (wave >> 1) + 16 * (j & 1) + 8 * (wave & 1) + 4 * (j >> 1)) * D]);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -806,12 +804,12 @@ __global__ void __launch_bounds__(512) paged_attention_tiles128_kernel(AttnMfmaA
     for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int s = 0; s < QS; ++s) k_rd[u][s] = (16 * u + c) * D + 8 * ((4 * s + g) ^ c);
-    // values: tile tl, dim d = 16 dt + c, keys 4 g .. 4 g + 3: chunk g / 2 at place (g / 2) ^ ((d >> 3) & 1), 8 bytes g % 2 of it
+    // values: keys 8 g .. 8 g + 7 of a chunk are in its tile g / 2, for dim d = 16 dt + c chunk g % 2 at place (g % 2) ^ ((d >> 3) & 1)
     int v_rd[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
         const int d = 16 * dt + c;
-        v_rd[dt] = d * 16 + 8 * ((g >> 1) ^ ((d >> 3) & 1)) + 4 * (g & 1);
+        v_rd[dt] = (g >> 1) * 16 * D + d * 16 + 8 * ((g & 1) ^ ((d >> 3) & 1));
     }
 
     if (block_begin >= block_end) return;
@@ -849,12 +847,8 @@ __global__ void __launch_bounds__(512) paged_attention_tiles128_kernel(AttnMfmaA
             for (int v = 0; v < 4; ++v) {
                 bf16x8_t vf[DT];
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(&vs[(2 * v) * 16 * D + v_rd[dt]]);
-                    const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(&vs[(2 * v + 1) * 16 * D + v_rd[dt]]);
-                    const u32x4_t x = {v0[0], v0[1], v1[0], v1[1]};
-                    vf[dt] = __builtin_bit_cast(bf16x8_t, x);
-                }
+                for (int dt = 0; dt < DT; ++dt)
+                    vf[dt] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(&vs[(2 * v) * 16 * D + v_rd[dt]]));
                 chunk_values<DT>(vf, pf[v], o);
             }
             fold_segment<DT>(o, m, l, o_tot, m_tot, l_tot);
