@@ -30,6 +30,10 @@ typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 #define AM_ITEM_INTS 8
 #define AM_SEG 128  // keys in a segment
 
+// One value of a fold: state * a + value * b with the second product rounded and the rest one fused multiply-add.
+// Every fold (the tiles' registers, the merge kernel's chain) goes through here.
+__device__ __forceinline__ float folded(float state, float a, float value, float b) { return fmaf(state, a, value * b); }
+
 // state (M, L, O) <- state folded with a segment's (m, l, o); one element of O at a time.  An empty segment changes nothing.
 __device__ __forceinline__ void fold_weights(float M, float m, float& a, float& b, float& Mn) {
     Mn = fmaxf(M, m);
@@ -114,11 +118,11 @@ __device__ __forceinline__ void fold_segment(const f32x4_t (&o)[DT], float m, fl
     }
     float fa, fb, mn;
     fold_weights(m_tot, m, fa, fb, mn);
-    l_tot = l_tot * fa + l * fb;
+    l_tot = folded(l_tot, fa, l, fb);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
-        o_tot[dt] = f32x4_t{o_tot[dt][0] * fa + o[dt][0] * fb, o_tot[dt][1] * fa + o[dt][1] * fb,
-                            o_tot[dt][2] * fa + o[dt][2] * fb, o_tot[dt][3] * fa + o[dt][3] * fb};
+        o_tot[dt] = f32x4_t{folded(o_tot[dt][0], fa, o[dt][0], fb), folded(o_tot[dt][1], fa, o[dt][1], fb),
+                            folded(o_tot[dt][2], fa, o[dt][2], fb), folded(o_tot[dt][3], fa, o[dt][3], fb)};
     m_tot = mn;
 }
 
@@ -702,8 +706,9 @@ __device__ __forceinline__ void attention_load_to_lds(const void* base, uint32_t
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(at), "v"(offset), "s"(base) : "memory", "m0");
 }
 
-// Prompt tiles of head_dim 128, the form for the sizes this engine serves: 8 waves hold 8 items of one request and one
-// KV head.  A segment's keys and values go from the pages straight into LDS (no registers in between), a whole segment
+// Prompt tiles of head_dim 128, the form for the sizes this engine serves: 12 waves hold 12 items of one request and one
+// KV head (three waves a SIMD: the registers just allow it, and one wave's vector instructions run beside another's
+// matrix instructions; measured against 8 waves: a 2,048-token portion at depth 63K 4.13 -> 3.57 ms).  A segment's keys and values go from the pages straight into LDS (no registers in between), a whole segment
 // ahead: while segment n is worked on, segment n+1 is on its way into the other half of LDS; one barrier a segment.
 // LDS rows are not padded; the 16-byte chunks are placed so that the operand reads miss each other's banks:
 //   keys:   a row of 256 bytes a key, in the order the score tiles want them (a chunk's key 8a + 4u + b in row
@@ -711,20 +716,21 @@ __device__ __forceinline__ void attention_load_to_lds(const void* base, uint32_t
 //   values: per tile of 16 keys a block of 128 dims x 32 bytes, the two chunks of dim d swapped when (d >> 3) & 1
 // and the lane that fills a place fetches the chunk that belongs there.  Per column the arithmetic is that of the
 // kernels above (the same functions on the same values).
-__global__ void __launch_bounds__(512) paged_attention_tiles128_kernel(AttnMfmaArgs a) {
-    constexpr int DT = 8, QS = 4, D = 128;
+#define AM_TILES128_WAVES 12
+__global__ void __launch_bounds__(64 * AM_TILES128_WAVES) paged_attention_tiles128_kernel(AttnMfmaArgs a) {
+    constexpr int DT = 8, QS = 4, D = 128, NW = AM_TILES128_WAVES;
     constexpr int K_SEG = AM_SEG * D, V_SEG = AM_SEG * D;   // elements of a segment's keys (values) in LDS
     __shared__ __attribute__((aligned(1024))) bf16_t Ks[2 * K_SEG];
     __shared__ __attribute__((aligned(1024))) bf16_t Vs[2 * V_SEG];
-    __shared__ int ranges[8][2];
+    __shared__ int ranges[NW][2];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int* it = a.items + ((size_t)blockIdx.x * 8 + wave) * AM_ITEM_INTS;
+    const int* it = a.items + ((size_t)blockIdx.x * NW + wave) * AM_ITEM_INTS;
     const int row0 = __builtin_amdgcn_readfirstlane(it[0]), n_rows = __builtin_amdgcn_readfirstlane(it[1]);
     const int h = __builtin_amdgcn_readfirstlane(it[2]);
-    const int lead_row = a.items[(size_t)blockIdx.x * 8 * AM_ITEM_INTS];   // the first item is never a filler
-    const int lead_head = a.items[(size_t)blockIdx.x * 8 * AM_ITEM_INTS + 2];
+    const int lead_row = a.items[(size_t)blockIdx.x * NW * AM_ITEM_INTS];   // the first item is never a filler
+    const int lead_head = a.items[(size_t)blockIdx.x * NW * AM_ITEM_INTS + 2];
     const int bt = a.page_tokens, Hkv = a.n_kv_heads;
     const int kvh = lead_head / (a.n_heads / Hkv);
     const int* table = a.tables + (size_t)a.row_entry[lead_row] * a.max_blocks;
@@ -749,7 +755,7 @@ __global__ void __launch_bounds__(512) paged_attention_tiles128_kernel(AttnMfmaA
     __syncthreads();
     int bb = 0x7fffffff, be = 0;
 #pragma unroll
-    for (int w = 0; w < 8; ++w) {
+    for (int w = 0; w < NW; ++w) {
         bb = min(bb, ranges[w][0]);
         be = max(be, ranges[w][1]);
     }
@@ -768,10 +774,11 @@ __global__ void __launch_bounds__(512) paged_attention_tiles128_kernel(AttnMfmaA
     float m_tot = -INFINITY, l_tot = 0.0f;
 
     // A segment's loads: 32 instructions for its keys (4 keys each: lane l is key l / 16, place l % 16) and 32 for its
-    // values (32 dims of one tile each: lane l is dim l / 2, place l % 2), 8 of them a wave: wave w brings the keys of
-    // tile w (4 instructions) and the values of tile w (4 instructions).  The tile's page comes from the block table.
+    // values (32 dims of one tile each: lane l is dim l / 2, place l % 2), 8 of them a wave: wave w of the first 8 brings
+    // the keys of tile w (4 instructions) and the values of tile w (4 instructions).  The tile's page comes from the block table.
     const uint32_t k_lane = (uint32_t)((((lane >> 4) * D) + 8 * ((lane & 15) ^ (lane >> 4))) * sizeof(bf16_t));   // + 4 j keys: see below
     auto issue = [&](int seg0, int buf) {
+        if (wave >= 8) return;                               // a segment has 8 tiles: the first 8 waves bring them
         const int key0 = seg0 + 16 * wave;                   // the wave's tile
         const int page = key0 < block_end ? __builtin_amdgcn_readfirstlane(table[key0 / bt]) : -1;
         const int pg = page < 0 ? 0 : page;                  // a tile past the keys reads page 0: its keys are masked
@@ -981,26 +988,26 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
                             O[0] = ring[r][0][0];
                             if constexpr (WIDE) O[1] = ring[r][1][0];
                         } else {
-                            L = L * fa[0][0] + fl[0][0] * fb[0][0];
-                            O[0] = O[0] * fa[0][0] + ring[r][0][0] * fb[0][0];
-                            if constexpr (WIDE) O[1] = O[1] * fa[0][0] + ring[r][1][0] * fb[0][0];
+                            L = folded(L, fa[0][0], fl[0][0], fb[0][0]);
+                            O[0] = folded(O[0], fa[0][0], ring[r][0][0], fb[0][0]);
+                            if constexpr (WIDE) O[1] = folded(O[1], fa[0][0], ring[r][1][0], fb[0][0]);
                         }
                         if (count == MERGE_DEPTH) {
 #pragma unroll
                             for (int u = 1; u < MERGE_DEPTH; ++u) {
                                 const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
-                                L = L * a + l * b;
-                                O[0] = O[0] * a + ring[r][0][u] * b;
-                                if constexpr (WIDE) O[1] = O[1] * a + ring[r][1][u] * b;
+                                L = folded(L, a, l, b);
+                                O[0] = folded(O[0], a, ring[r][0][u], b);
+                                if constexpr (WIDE) O[1] = folded(O[1], a, ring[r][1][u], b);
                             }
                         } else {
 #pragma unroll
                             for (int u = 1; u < MERGE_DEPTH; ++u) {
                                 if (u < count) {    // the same for every thread
                                     const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
-                                    L = L * a + l * b;
-                                    O[0] = O[0] * a + ring[r][0][u] * b;
-                                    if constexpr (WIDE) O[1] = O[1] * a + ring[r][1][u] * b;
+                                    L = folded(L, a, l, b);
+                                    O[0] = folded(O[0], a, ring[r][0][u], b);
+                                    if constexpr (WIDE) O[1] = folded(O[1], a, ring[r][1][u], b);
                                 }
                             }
                         }
@@ -1012,11 +1019,11 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
                         for (int u = 0; u < MERGE_DEPTH; ++u) {
                             const uint32_t code = (at + u < n) ? fc[u / 4][u % 4] : 0u;
                             const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
-                            const float l_fold = L * a + l * b, o0_fold = O[0] * a + ring[r][0][u] * b;
+                            const float l_fold = folded(L, a, l, b), o0_fold = folded(O[0], a, ring[r][0][u], b);
                             L = code == 2u ? l_fold : (code == 1u ? l : L);
                             O[0] = code == 2u ? o0_fold : (code == 1u ? ring[r][0][u] : O[0]);
                             if constexpr (WIDE) {
-                                const float o1_fold = O[1] * a + ring[r][1][u] * b;
+                                const float o1_fold = folded(O[1], a, ring[r][1][u], b);
                                 O[1] = code == 2u ? o1_fold : (code == 1u ? ring[r][1][u] : O[1]);
                             }
                         }
@@ -1037,7 +1044,7 @@ __global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restr
 // Rows part_o must have beyond its slots' (see the merge).
 extern "C" int llmx_attention_partial_pad() { return MERGE_PAD; }
 
-// `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 8: one workgroup each 8, or
+// `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 12: one workgroup each 12, or
 // each 4 for head sizes other than 128),
 // then the n_direct items that fold their segments themselves (slot < 0), then the n_partial items that write them
 // (slot >= 0).  wide_items: a decoding item is worked on by a workgroup of 4 waves instead of one wave (head_dim 128 only;
@@ -1048,7 +1055,7 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
                                          void* out, float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
                                          int page_tokens, int max_blocks, int window, int wide_items, hipStream_t stream) {
     if (n_shared + n_direct + n_partial <= 0) return 0;
-    if (n_shared % 8) return -2;
+    if (n_shared % 12) return -2;
     if (head_dim % 16 || head_dim > AM_MAX_D || page_tokens % 16 || n_heads % n_kv_heads) return -2;
     AttnMfmaArgs a{(const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, pos, row_entry, tables, items, (bf16_t*)out, part_o,
                    part_ml, scale, n_direct, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
@@ -1063,7 +1070,7 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
 #define AM_CASE(DT)                                                                                                          \
     case DT:                                                                                                                 \
         if (n_shared > 0 && DT == 8 && page_tokens % 16 == 0)                                                               \
-            hipLaunchKernelGGL(paged_attention_tiles128_kernel, dim3(n_shared / 8), dim3(512), 0, stream, sh);                          \
+            hipLaunchKernelGGL(paged_attention_tiles128_kernel, dim3(n_shared / AM_TILES128_WAVES), dim3(64 * AM_TILES128_WAVES), 0, stream, sh); \
         else if (n_shared > 0) hipLaunchKernelGGL((paged_attention_tiles_kernel<DT>), dim3(n_shared / 4), block, 0, stream, sh);        \
         if (n_direct > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, false>), dim3((n_direct + 3) / 4), block, 0, stream, a);  \
         if (n_partial > 0 && DT == 8 && wide_items)                                                                          \

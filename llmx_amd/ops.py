@@ -318,7 +318,7 @@ class AttentionPlan:
 
     def __init__(self, shared, items, merges, n_slots, device):
         import numpy as np
-        self.n_shared = len(shared)          # prompt tiles, 8 (or twice 4) to a workgroup that shares their keys
+        self.n_shared = len(shared)          # prompt tiles, 12 (or three times 4) to a workgroup that shares their keys
         self.n_direct = sum(1 for i in items if i[6] < 0)
         items = shared + [i for i in items if i[6] < 0] + [i for i in items if i[6] >= 0]   # those that fold their segments first
         self.n_items = len(items)
@@ -339,8 +339,8 @@ ATTENTION_WIDE_ITEMS = 1024     # up to this many decoding items a step, an item
 def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, window: int = 0) -> AttentionPlan:
     """row_counts[i]: rows of entry i in the step (entries' rows are consecutive, in order); contexts[i]: tokens the
     entry holds after the step.  Single-row entries become items per KV head (columns = its query heads) that share out
-    the context's 128-key segments when there are few rows; longer entries become tiles of 16 rows of one head, 8 tiles
-    that read the same KV head to a workgroup (two workgroups of 4 for head sizes other than 128).  How the context is shared out changes no result: segments are folded in
+    the context's 128-key segments when there are few rows; longer entries become tiles of 16 rows of one head, 12 tiles
+    that read the same KV head to a workgroup (three workgroups of 4 for head sizes other than 128).  How the context is shared out changes no result: segments are folded in
     key order either way."""
     ratio = n_heads // n_kv_heads
     head_chunks = [(kvh * ratio + c0, min(16, ratio - c0)) for kvh in range(n_kv_heads) for c0 in range(0, ratio, 16)]
@@ -371,11 +371,11 @@ def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, 
         for kvh in range(n_kv_heads):
             tiles = [[row0s[i] + r0, min(16, n - r0), h, 1, 0, 1, -1, 0]
                      for r0 in range(((n - 1) // 16) * 16, -1, -16) for h in range(kvh * ratio, (kvh + 1) * ratio)]
-            tiles += [[0, 0, 0, 1, 0, 1, -1, 0]] * (-len(tiles) % 8)
+            tiles += [[0, 0, 0, 1, 0, 1, -1, 0]] * (-len(tiles) % 12)
             per_head.append(tiles)
-        for b in range(0, len(per_head[0]), 8):      # the KV heads' workgroups take turns, so long ranges start first
+        for b in range(0, len(per_head[0]), 12):     # the KV heads' workgroups take turns, so long ranges start first
             for tiles in per_head:
-                shared += tiles[b:b + 8]
+                shared += tiles[b:b + 12]
     for i in single:
         for head0, nh in head_chunks:
             if n_splits == 1:
