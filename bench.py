@@ -12,6 +12,9 @@ step, one new token each, logits -> greedy token on the device -> ids read back 
   points               the same for every measured batch, flat: decode_b<B> (tok/s), decode_b<B>_ms, _gb (bytes to read),
                        _experts (distinct a layer) and _frac (of 8 TB/s); decode_b<B>_logits_to_host is the default batch
                        with every step's logits copied to pinned host memory, as the reference's bench reads them;
+                       generate_b<B>: the same batch through the product's own loop (scheduler, step, device sampler
+                       with temperature 0.8, top-k 40, top-p 0.95): tok/s of its steps that carried only decoded
+                       tokens, their mean rows (_rows_a_step) and time (_ms), the run's wall time and tokens;
   prefill              one 2,048-token prompt from an empty cache: tok/s, ms, `frac` = flops / time / the bf16 peak,
                        `hbm_frac` = the weights it has to read (the experts its tokens picked) / time / 8 TB/s, and the
                        first layer's feed-forward alone (first_layer_*): its rows are all different, so it touches every
@@ -59,6 +62,7 @@ def parse():
     ap.add_argument("--no-calibration", action="store_true", help="skip the copy, read and library-product rates of the card")
     ap.add_argument("--no-logits-to-host", action="store_true",
                     help="skip the extra point: the default batch with every step's logits copied to the host")
+    ap.add_argument("--no-generate", action="store_true", help="skip the extra point: the default batch through the scheduler and the sampler")
     ap.add_argument("--only-prefill", action="store_true", help="for profiling: measure the prefill alone and print its record")
     ap.add_argument("--only-long", action="store_true", help="for profiling: run the long-context configuration alone and print its record")
     return ap.parse_args()
@@ -298,6 +302,27 @@ def run_mixed_step(engine, cfg, sampler_out, context, portion, decoding, reps, t
     return {"ms": round(dt * 1e3, 3), "tok_s": round((decoding + portion) / dt, 1), "decoding": decoding, "portion": portion, "context": context}
 
 
+def run_generate(engine, cfg, batch, context, new_tokens, torch):
+    """The product's own loop: `batch` requests through the scheduler (prompts in portions beside decoding requests),
+    the step function and the device sampler with the reference's default settings (temperature 0.8, top-k 40, top-p
+    0.95), each request's context reaching `context` tokens.  Reports the steps that carried only decoded tokens."""
+    from llmx_amd import SamplingParams
+    from llmx_amd.engine.generation import Generator
+    from llmx_amd.engine.scheduler import Request
+    gen = Generator(engine, batch, PREFILL_TOKENS)
+    for i in range(batch):
+        gen.submit(Request(("generate", i), lcg_ids(context - new_tokens, cfg.vocab_size, 100 + i),
+                           SamplingParams(max_tokens=new_tokens, temp=0.8, top_k=40, top_p=0.95, seed=1 + i, ignore_eos=True)))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    gen.run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    st = gen.stats
+    return {"tok_s": round(st.decode_rows / max(st.decode_seconds, 1e-9), 2), "rows_a_step": round(st.decode_rows / max(st.decode_steps, 1), 2),
+            "ms": round(st.decode_seconds / max(st.decode_steps, 1) * 1e3, 4), "wall_s": round(wall, 2), "tokens": st.generated_tokens}
+
+
 def run_long(torch, steps_warm=4):
     """The long-context configuration: 30 layers, 2 requests of 65,536 prompt tokens fed in portions of 2,048, then 256
     decoded tokens each.  Returns its record."""
@@ -404,6 +429,10 @@ def main():
         pts[f"decode_b{a.batch}_logits_to_host"] = round(a.batch * a.steps / r["s"], 2)
     for b in points:
         add_point(f"decode_b{b}", decode_record(cfg, b, context, a.steps, run_decode(engine, sampler_out, b, context, a.steps, a.warmup, torch)))
+    if points and not a.no_generate:
+        g = run_generate(engine, cfg, a.batch, context, 2 * a.steps, torch)
+        for key, v in g.items():
+            pts[f"generate_b{a.batch}" if key == "tok_s" else f"generate_b{a.batch}_{key}"] = v
     result["points"] = pts
 
     if a.sweep:

@@ -25,6 +25,8 @@ class GenerationStats:
     steps: int = 0
     prompt_seconds: float = 0.0     # time of steps that carried prompt portions
     decode_seconds: float = 0.0     # time of steps that carried only decoded tokens
+    decode_steps: int = 0           # such steps
+    decode_rows: int = 0            # and the tokens they carried
 
 
 class Generator:
@@ -85,6 +87,8 @@ class Generator:
             self.stats.prompt_tokens += prompt_rows
         else:
             self.stats.decode_seconds += dt
+            self.stats.decode_steps += 1
+            self.stats.decode_rows += len(plan)
         sampled = {r.id: t for r, t in zip(reqs, tokens)}
         done = sch.advance(plan, sampled)
         for r, t in zip(reqs, tokens):
