@@ -14,7 +14,7 @@ step, one new token each, logits -> greedy token on the device -> ids read back 
                        with every step's logits copied to pinned host memory, as the reference's bench reads them;
                        generate_b<B>: the same batch through the product's own loop (scheduler, step, device sampler
                        with temperature 0.8, top-k 40, top-p 0.95): tok/s of its steps that carried only decoded
-                       tokens, their mean rows (_rows_a_step) and time (_ms), the run's wall time and tokens;
+                       tokens, their mean rows (_rows_a_step) and time (_ms);
   prefill              one 2,048-token prompt from an empty cache: tok/s, ms, `frac` = flops / time / the bf16 peak,
                        `hbm_frac` = the weights it has to read (the experts its tokens picked) / time / 8 TB/s, and the
                        first layer's feed-forward alone (first_layer_*): its rows are all different, so it touches every
@@ -313,14 +313,11 @@ def run_generate(engine, cfg, batch, context, new_tokens, torch):
     for i in range(batch):
         gen.submit(Request(("generate", i), lcg_ids(context - new_tokens, cfg.vocab_size, 100 + i),
                            SamplingParams(max_tokens=new_tokens, temp=0.8, top_k=40, top_p=0.95, seed=1 + i, ignore_eos=True)))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
     gen.run()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     st = gen.stats
     return {"tok_s": round(st.decode_rows / max(st.decode_seconds, 1e-9), 2), "rows_a_step": round(st.decode_rows / max(st.decode_steps, 1), 2),
-            "ms": round(st.decode_seconds / max(st.decode_steps, 1) * 1e3, 4), "wall_s": round(wall, 2), "tokens": st.generated_tokens}
+            "ms": round(st.decode_seconds / max(st.decode_steps, 1) * 1e3, 4)}
 
 
 def run_long(torch, steps_warm=4):
