@@ -1,6 +1,6 @@
 """Decode and prefill throughput of MiniMax-M3 at real layer sizes with random weights, on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--points 1,64] [--sweep] [--long]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--points 1,64] [--no-sweep] [--long]
 
 A step is one decode step of the whole batch: B requests, each at a context that reaches C tokens at the last timed
 step, one new token each, logits -> greedy token on the device -> ids read back (the reference's batched `tg`,
@@ -19,8 +19,9 @@ step, one new token each, logits -> greedy token on the device -> ids read back 
                        `hbm_frac` = the weights it has to read (the experts its tokens picked) / time / 8 TB/s, and the
                        first layer's feed-forward alone (first_layer_*): its rows are all different, so it touches every
                        expert and streams all their weights;
-  sweep (--sweep)      further sizes: batch 8 at 16k and 32k tokens of context, batch 16 and 32 at 4k, and the mixed step
-                       a scheduler issues: a 512-token prompt portion beside 8 decoding requests;
+  sweep                further sizes (left out with --no-sweep, or when --points is empty and --sweep is not given): batch 8
+                       at 16k and 32k tokens of context, batch 16 and 32 at 4k (tok/s, _ms, _experts, _frac), and the mixed
+                       step a scheduler issues: a 512-token prompt portion beside 8 decoding requests;
   long (--long)        the long-context configuration: 30 layers, 2 requests of 65,536 prompt tokens in portions of
                        2,048, then 256 decoded tokens each (the engine is freed and built again for it);
   calibration          what a device copy, a read-only pass and a square bf16 library product reach on this card.
@@ -56,7 +57,8 @@ def parse():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=0, help="tokens each sequence holds at the last timed step (0: the configuration's 4,096)")
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
-    ap.add_argument("--sweep", action="store_true", help="also measure further contexts and batches and the mixed prompt + decode step")
+    ap.add_argument("--sweep", action="store_true", help="measure further contexts and batches and the mixed prompt + decode step (the default whenever --points names a batch)")
+    ap.add_argument("--no-sweep", action="store_true", help="leave those out")
     ap.add_argument("--long", action="store_true", help="also run the long-context configuration (30 layers, 2 x 65,536 tokens, 256 decoded)")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-calibration", action="store_true", help="skip the copy, read and library-product rates of the card")
@@ -377,9 +379,10 @@ def main():
     context = a.context or CONTEXT
     layers = a.layers or FULL_LAYERS
     points = [int(p) for p in a.points.split(",") if p.strip()]
-    sweep = [(8, 16384), (8, 32768), (16, context), (32, context)] if a.sweep else []
-    kv_tokens = max([a.batch * context] + [b * context for b in points] + [b * c for b, c in sweep] + ([9 * context] if a.sweep else []))
-    max_batch = max([a.batch] + points + [b for b, _ in sweep] + ([9] if a.sweep else []))
+    do_sweep = a.sweep or (bool(points) and not a.no_sweep)
+    sweep = [(8, 16384), (8, 32768), (16, context), (32, context)] if do_sweep else []
+    kv_tokens = max([a.batch * context] + [b * context for b in points] + [b * c for b, c in sweep] + ([9 * context] if do_sweep else []))
+    max_batch = max([a.batch] + points + [b for b, _ in sweep] + ([9] if do_sweep else []))
     cfg = real_config(layers, max([context] + [c for _, c in sweep]))
     t_setup = time.perf_counter()
     engine = Engine.from_random(cfg, RandomInit(seed=0, std=0.02), dtype="bfloat16", kv_tokens=kv_tokens, page_tokens=16, max_requests=max_batch)
@@ -432,13 +435,13 @@ def main():
             pts[f"generate_b{a.batch}" if key == "tok_s" else f"generate_b{a.batch}_{key}"] = v
     result["points"] = pts
 
-    if a.sweep:
+    if do_sweep:
         sw = {}
         for b, c in sweep:
             rec = decode_record(cfg, b, c, a.steps, run_decode(engine, sampler_out, b, c, a.steps, a.warmup, torch))
             name = f"decode_b{b}_ctx{c}"
             sw[name] = rec["tok_s"]
-            for key in ("ms", "gb", "experts", "frac"):
+            for key in ("ms", "experts", "frac"):
                 sw[f"{name}_{key}"] = rec[key]
         mixed = run_mixed_step(engine, cfg, sampler_out, context, 512, 8, 8, torch)
         sw["mixed_512_beside_8_ms"] = mixed["ms"]
