@@ -154,7 +154,7 @@ def cmd_generate(a) -> int:
         raise SystemExit2("generate: empty prompt")
     need = sum(len(p) + params.max_tokens for p in prompts[:a.max_seqs]) if len(prompts) > 1 else len(prompts[0]) + params.max_tokens
     kv_tokens = a.kv_tokens or max(need + a.page_tokens * a.max_seqs, max(len(p) for p in prompts) + params.max_tokens)
-    engine = _engine(a, cfg, kv_tokens=kv_tokens, page_tokens=a.page_tokens, max_requests=a.max_seqs)
+    engine = _engine(a, cfg, kv_tokens=kv_tokens, page_tokens=a.page_tokens, max_requests=a.max_seqs, step_tokens=a.ubatch)
     gen = Generator(engine, a.max_seqs, a.ubatch)
     for i, p in enumerate(prompts):
         import copy
