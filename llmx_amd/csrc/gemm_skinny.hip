@@ -234,8 +234,94 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_kernel(SkinnyArgs g) {
     }
 }
 
+// Dense products of 17 to 64 rows: two strips of 16 features a workgroup.  With several tiles of rows a step fetches
+// more bytes of rows (from the caches, again for every strip) than of weights; a workgroup that multiplies the rows'
+// fragments into two strips fetches them half as often.  A wave's steps, their rounds of four and the order in which
+// the waves' sums are added are those of the kernel above: the same bits.
+template <int KS, int MT, int EPI, typename TC>
+__global__ void __launch_bounds__(64 * KS) gemm_skinny_two_strips_kernel(SkinnyArgs g) {
+    static_assert(EPI != SK_SWIGLU, "one weight strip a feature strip");
+    __shared__ float red[KS > 1 ? KS : 1][MT * 2][256];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 15, kg = lane >> 4;
+    const int n0 = blockIdx.x * 32;
+    const int K = g.K;
+    const int steps_total = (K + 31) >> 5;
+    const int per = (steps_total + KS - 1) / KS;
+    const int s_begin = wave * per;
+    const int s_end = min(steps_total, s_begin + per);
+    const bf16_t* wp[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) wp[q] = g.W + (size_t)min(n0 + 16 * q + r, g.N - 1) * K + kg * 8;
+    const bf16_t* ap[MT];
+    bool a_in[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + r;
+        a_in[t] = m < g.M;
+        ap[t] = g.A + (size_t)(a_in[t] ? m : 0) * g.lda + kg * 8;
+    }
+    f32x4_t acc[MT][2];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int q = 0; q < 2; ++q) acc[t][q] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s = s_begin; s < s_end; s += 4) {
+        bf16x8_t wf[4][2], af[4][MT];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int k = (s + u) * 32 + kg * 8;
+            const bool in = (s + u) < s_end && k < K;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) wf[u][q] = load_frag(wp[q] + (size_t)(s + u) * 32, in);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) af[u][t] = load_frag(ap[t] + (size_t)(s + u) * 32, in && a_in[t]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int q = 0; q < 2; ++q) acc[t][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][q], af[u][t], acc[t][q], 0, 0, 0);
+    }
+    if (KS > 1) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int q = 0; q < 2; ++q) *reinterpret_cast<f32x4_t*>(&red[wave][t * 2 + q][lane * 4]) = acc[t][q];
+        __syncthreads();
+    }
+    if (wave != 0) return;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + r;      // lane: row m, features n0 + 16 q + 4 kg + 0..3
+        if (m >= g.M) continue;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            f32x4_t v = acc[t][q];
+            if (KS > 1) {
+                v = *reinterpret_cast<f32x4_t*>(&red[0][t * 2 + q][lane * 4]);
+#pragma unroll
+                for (int w = 1; w < KS; ++w) {
+                    const f32x4_t o = *reinterpret_cast<f32x4_t*>(&red[w][t * 2 + q][lane * 4]);
+                    v = f32x4_t{v[0] + o[0], v[1] + o[1], v[2] + o[2], v[3] + o[3]};
+                }
+            }
+            TC* c = (TC*)g.C + (size_t)m * g.ldc + n0 + 16 * q + 4 * kg;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (n0 + 16 * q + 4 * kg + i >= g.N) continue;
+                float x = v[i];
+                if (EPI == SK_ADD) x = ld(c + i) + x;
+                st(c + i, x);
+            }
+        }
+    }
+}
+
 // steps of K in a round of loads: with one tile of rows two rounds are in flight (see the kernel)
 #define SKINNY_ROUND(MT, EPI) 4
+#define SKINNY_TWO_STRIPS_MIN_WORKGROUPS 192
 
 template <int KS, int MT, int EPI, typename TC>
 static void launch_grouped(const SkinnyArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
@@ -250,10 +336,18 @@ static void launch_grouped(const SkinnyArgs& g, dim3 grid, bool grouped, hipStre
         }
         return;
     }
-    if (grouped)
+    if (grouped) {
         hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true, SKINNY_ROUND(MT, EPI), false>), grid, dim3(64 * KS), 0, stream, g);
-    else
-        hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false, SKINNY_ROUND(MT, EPI), false>), grid, dim3(64 * KS), 0, stream, g);
+        return;
+    }
+    if constexpr (MT > 1 && EPI != SK_SWIGLU) {
+        // several tiles of rows: two strips a workgroup where that still gives the chip enough workgroups
+        if ((g.N + 31) / 32 >= SKINNY_TWO_STRIPS_MIN_WORKGROUPS) {
+            hipLaunchKernelGGL((gemm_skinny_two_strips_kernel<KS, MT, EPI, TC>), dim3((g.N + 31) / 32), dim3(64 * KS), 0, stream, g);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false, SKINNY_ROUND(MT, EPI), false>), grid, dim3(64 * KS), 0, stream, g);
 }
 
 template <int KS, int MT>
