@@ -69,8 +69,9 @@ def test_rmsnorm(rows, width, eps):
 
 
 # ---------------------------------------------------------------------------
+# (the shapes of 17 to 64 rows and at least 6,113 features take the weight-streaming kernel's form with two strips a workgroup)
 GEMM_SHAPES = [(1, 16, 32), (2, 48, 96), (3, 100, 72), (17, 200, 3072), (64, 96, 192), (65, 130, 264), (8, 8192, 3072), (33, 3072, 6144),
-               (129, 72, 40), (300, 257, 136), (2048, 512, 3072)]
+               (129, 72, 40), (300, 257, 136), (2048, 512, 3072), (64, 8192, 3072), (23, 6150, 104), (40, 6200, 1000)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
