@@ -238,11 +238,13 @@ extern "C" int llmx_qknorm_rope_kvwrite(const float* qkv, const float* q_weight,
     QkvArgs a{qkv, q_weight, k_weight, cos_sin, pos, row_entry, tables, q_out, k_cache, v_cache, eps,
               n_heads, n_kv_heads, head_dim, rotary_dim, norm_mode, page_tokens, max_blocks, write_kv, q_slices, k_slices, pairing};
     if (rows > 256 && qw <= 32 * 256 && kw <= 32 * 256 && head_dim <= 256) {   // rows kept in registers
+        llmx_note_launch(LK_QKNORM_ROPE_KVWRITE_ROWS);
         if (dtype == LLMX_F32) launch_qkv_rows<float, float>(a, rows, qw, kw, stream);
         else launch_qkv_rows<bf16_t, bf16_t>(a, rows, qw, kw, stream);
         return LLMX_CHECK_LAUNCH();
     }
     const dim3 grid(rows, q_slices + k_slices);
+    llmx_note_launch(LK_QKNORM_ROPE_KVWRITE);
     if (dtype == LLMX_F32)
         hipLaunchKernelGGL((qknorm_rope_kvwrite_kernel<float, float>), grid, dim3(256), 0, stream, a);
     else
@@ -344,6 +346,7 @@ extern "C" int llmx_paged_attention_generic(const void* q, const void* k_cache, 
     if (rows <= 0) return 0;
     if (head_dim > ATT_MAX_D || n_heads % n_kv_heads) return -2;
     AttnArgs a{q, k_cache, v_cache, pos, row_entry, tables, out, scale, n_heads, n_kv_heads, head_dim, page_tokens, max_blocks, window};
+    llmx_note_launch(LK_ATTENTION_GENERIC);
     if (dtype == LLMX_F32)
         hipLaunchKernelGGL(paged_attention_generic_kernel<float>, dim3(rows, n_heads), dim3(64), 0, stream, a);
     else

@@ -1066,6 +1066,11 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
     b.items = a.items + (size_t)n_direct * AM_ITEM_INTS;
     b.n_items = n_partial;
     const dim3 block(256);
+    const bool tiles128 = n_shared > 0 && head_dim == 128, split4 = n_partial > 0 && head_dim == 128 && wide_items;
+    if (n_shared > 0) llmx_note_launch(tiles128 ? LK_ATTENTION_TILES128 : LK_ATTENTION_TILES);
+    if (n_direct > 0) llmx_note_launch(LK_ATTENTION_DIRECT);
+    if (n_partial > 0) llmx_note_launch(split4 ? LK_ATTENTION_SPLIT4 : LK_ATTENTION_PARTIAL);
+    if (n_merges > 0) llmx_note_launch(LK_ATTENTION_MERGE);
     switch (head_dim / 16) {
 #define AM_CASE(DT)                                                                                                          \
     case DT:                                                                                                                 \

@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "witness.h"
+
 #define LLMX_WAVE 64
 
 // dtype codes of the C ABI

@@ -161,6 +161,7 @@ extern "C" int llmx_gemm_generic(const void* A, int a_dtype, const void* W, int 
                                  long w_group_stride, int up_offset, hipStream_t stream) {
     if (N <= 0 || K <= 0) return 0;
     if (n_groups == 0 && M <= 0) return 0;
+    llmx_note_launch(n_groups ? LK_GEMM_GENERIC_GROUPED : LK_GEMM_GENERIC);
     GemmArgs g{A, W, C, M, N, K, lda, ldw, ldc, n_groups ? group_offsets : nullptr, list, a_div > 0 ? a_div : 1, w_group_stride, up_offset};
     dim3 grid;
     grid.x = (N + GT_BN - 1) / GT_BN;

@@ -323,48 +323,58 @@ __global__ void __launch_bounds__(64 * KS) gemm_skinny_two_strips_kernel(SkinnyA
 #define SKINNY_ROUND(MT, EPI) 4
 #define SKINNY_TWO_STRIPS_MIN_WORKGROUPS 192
 
+// Returns -2 (and launches nothing) for a combination that has no kernel: normed rows with several tiles of rows or
+// with an adding epilogue.
 template <int KS, int MT, int EPI, typename TC>
-static void launch_grouped(const SkinnyArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
+static int launch_grouped(const SkinnyArgs& g, dim3 grid, bool grouped, hipStream_t stream) {
     if (g.X) {
         // normed rows: one tile of rows, the rows kept in LDS
         if constexpr (MT == 1 && EPI != SK_ADD) {
             const size_t lds = (size_t)g.x_rows * g.K * sizeof(bf16_t);
+            llmx_note_launch(grouped ? LK_GEMM_SKINNY_GROUPED_NORMED : LK_GEMM_SKINNY_NORMED);
             if (grouped)
                 hipLaunchKernelGGL((gemm_skinny_kernel<KS, 1, EPI, TC, true, SKINNY_ROUND(MT, EPI), true>), grid, dim3(64 * KS), lds, stream, g);
             else
                 hipLaunchKernelGGL((gemm_skinny_kernel<KS, 1, EPI, TC, false, SKINNY_ROUND(MT, EPI), true>), grid, dim3(64 * KS), lds, stream, g);
+            return 0;
         }
-        return;
+        return -2;
     }
     if (grouped) {
+        llmx_note_launch(LK_GEMM_SKINNY_GROUPED);
         hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, true, SKINNY_ROUND(MT, EPI), false>), grid, dim3(64 * KS), 0, stream, g);
-        return;
+        return 0;
     }
     if constexpr (MT > 1 && EPI != SK_SWIGLU) {
         // several tiles of rows: two strips a workgroup where that still gives the chip enough workgroups
         if ((g.N + 31) / 32 >= SKINNY_TWO_STRIPS_MIN_WORKGROUPS) {
+            llmx_note_launch(LK_GEMM_SKINNY_TWO_STRIPS);
             hipLaunchKernelGGL((gemm_skinny_two_strips_kernel<KS, MT, EPI, TC>), dim3((g.N + 31) / 32), dim3(64 * KS), 0, stream, g);
-            return;
+            return 0;
         }
     }
+    llmx_note_launch(LK_GEMM_SKINNY);
     hipLaunchKernelGGL((gemm_skinny_kernel<KS, MT, EPI, TC, false, SKINNY_ROUND(MT, EPI), false>), grid, dim3(64 * KS), 0, stream, g);
+    return 0;
 }
 
 template <int KS, int MT>
 static int launch_epi(const SkinnyArgs& g, int epi, int c_dtype, dim3 grid, bool grouped, hipStream_t stream) {
+    int rc;
     if (epi == SK_SWIGLU) {
         if (MT != 1) return -2;
-        if (c_dtype == LLMX_BF16) launch_grouped<KS, 1, SK_SWIGLU, bf16_t>(g, grid, grouped, stream);
-        else launch_grouped<KS, 1, SK_SWIGLU, float>(g, grid, grouped, stream);
+        if (c_dtype == LLMX_BF16) rc = launch_grouped<KS, 1, SK_SWIGLU, bf16_t>(g, grid, grouped, stream);
+        else rc = launch_grouped<KS, 1, SK_SWIGLU, float>(g, grid, grouped, stream);
     } else if (epi == SK_ADD) {
         if (c_dtype != LLMX_F32) return -2;
-        launch_grouped<KS, MT, SK_ADD, float>(g, grid, grouped, stream);
+        rc = launch_grouped<KS, MT, SK_ADD, float>(g, grid, grouped, stream);
     } else if (epi == SK_STORE) {
-        if (c_dtype == LLMX_BF16) launch_grouped<KS, MT, SK_STORE, bf16_t>(g, grid, grouped, stream);
-        else launch_grouped<KS, MT, SK_STORE, float>(g, grid, grouped, stream);
+        if (c_dtype == LLMX_BF16) rc = launch_grouped<KS, MT, SK_STORE, bf16_t>(g, grid, grouped, stream);
+        else rc = launch_grouped<KS, MT, SK_STORE, float>(g, grid, grouped, stream);
     } else {
         return -2;
     }
+    if (rc) return rc;
     return LLMX_CHECK_LAUNCH();
 }
 

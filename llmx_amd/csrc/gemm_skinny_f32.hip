@@ -351,12 +351,14 @@ extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, in
     if (M > 64 && N >= 128 && K % 16 == 0 && ks >= 1 && ks <= 16) {
         const dim3 staged((N + RL_FEATS - 1) / RL_FEATS, (M + RL_ROWS - 1) / RL_ROWS, slices);
         if (staged.y > 65535) return -2;
+        llmx_note_launch(LK_GEMM_F32_STAGED);
         hipLaunchKernelGGL(gemm_rows_f32_lds_kernel, staged, dim3(512), 0, stream, g, ks);
         return LLMX_CHECK_LAUNCH();
     }
     if (M > 64 && N >= 64 && ks <= 8) {
         const dim3 wide((N + 63) / 64, (M + 63) / 64, slices);
         if (wide.y > 65535) return -2;
+        llmx_note_launch(LK_GEMM_F32_ROWS);
         switch (ks) {
             case 1: hipLaunchKernelGGL(gemm_rows_f32_kernel<1>, wide, dim3(64), 0, stream, g); break;
             case 2: hipLaunchKernelGGL(gemm_rows_f32_kernel<2>, wide, dim3(128), 0, stream, g); break;
@@ -374,6 +376,7 @@ extern "C" int llmx_gemm_skinny_f32(const float* A, const float* W, float* C, in
         else if (M <= 32) SKF_LAUNCH(KS, 2);                                                                                  \
         else SKF_LAUNCH(KS, 4);                                                                                               \
     } while (0)
+    if (ks == 1 || ks == 2 || ks == 4 || ks == 8 || ks == 16) llmx_note_launch(norm_w ? LK_GEMM_F32_NORMED : LK_GEMM_F32_SKINNY);
     switch (ks) {
         case 1: SKF_MT(1); break;
         case 2: SKF_MT(2); break;

@@ -797,6 +797,10 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
         const int feats = form_feats(form, epi);
         dim3 grid((N + feats - 1) / feats, grouped ? tiles_y : g.m_tiles, 1);
         if (grid.y > 65535) return -2;
+        llmx_note_launch(form == FORM_WIDE ? (grouped ? LK_GEMM_TILE_GROUPED_WIDE : LK_GEMM_TILE_WIDE)
+                         : form == FORM_128 ? LK_GEMM_TILE_GROUPED_128
+                         : form == FORM_64 ? (grouped ? LK_GEMM_TILE_GROUPED_64 : LK_GEMM_TILE_64)
+                                           : (grouped ? LK_GEMM_TILE_GROUPED_BOUNDED : LK_GEMM_TILE_BOUNDED));
         return tile_launch_typed(g, form, grid, grouped, epi, c_dtype, stream);
     };
     int rc;

@@ -190,6 +190,7 @@ extern "C" int llmx_route_topk(float* z, const float* parts, int slices, long sl
                                int rows, int n_experts, int k, int score, int normalize, float scale, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (n_experts > ROUTE_MAX_EXPERTS || k > ROUTE_MAX_K || k > n_experts || k <= 0 || (parts && (slices < 1 || slices > ROUTE_MAX_SLICES))) return -2;
+    llmx_note_launch(LK_ROUTE_TOPK);
     hipLaunchKernelGGL(route_topk_kernel, dim3(rows), dim3(64), 0, stream, z, parts, slices, slice_stride, bias, ids, weights, n_experts, k, score,
                        normalize, scale);
     return LLMX_CHECK_LAUNCH();
@@ -416,6 +417,7 @@ __global__ void __launch_bounds__(1024) moe_chunk_place_kernel(const int* __rest
 extern "C" int llmx_moe_align(const int* ids, int n_pairs, int n_experts, int* counts, int* offsets, int* list, int* active, int* n_active,
                               int* scratch, int* tiles128, hipStream_t stream) {
     if (n_pairs <= 0 || n_experts <= 0) return 0;
+    llmx_note_launch(LK_MOE_ALIGN);
     if (n_pairs <= ALIGN_SMALL_PAIRS && n_experts <= 1024) {
         hipLaunchKernelGGL(moe_align_small_kernel, dim3(1), dim3(1024), 0, stream, ids, n_pairs, n_experts, counts, offsets, list, active, n_active);
         return LLMX_CHECK_LAUNCH();
@@ -469,6 +471,7 @@ extern "C" int llmx_route_topk_align(float* z, const float* parts, int slices, l
     if (rows <= 0) return 0;
     if (rows > 16 || rows * k > ALIGN_SMALL_PAIRS || n_experts > 256 || k > 64 || k > n_experts || k <= 0) return -2;
     if (parts && (slices < 1 || slices > ROUTE_MAX_SLICES)) return -2;
+    llmx_note_launch(LK_ROUTE_TOPK_ALIGN);
     hipLaunchKernelGGL(route_topk_align_kernel, dim3(1), dim3(1024), 0, stream, z, parts, slices, slice_stride, bias, ids, weights, rows, n_experts, k,
                        normalize, scale,
                        counts, offsets, list, active, n_active);

@@ -13,6 +13,7 @@ __global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __r
 
 extern "C" int llmx_embed_gather(const void* table, int table_dtype, const int* ids, float* x, int rows, int width, hipStream_t stream) {
     if (rows <= 0) return 0;
+    llmx_note_launch(LK_EMBED_GATHER);
     if (table_dtype == LLMX_F32)
         hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(rows), dim3(256), 0, stream, (const float*)table, ids, x, width);
     else
@@ -76,6 +77,7 @@ __global__ void __launch_bounds__(RMS_THREADS) rmsnorm_kept_kernel(const float* 
 extern "C" int llmx_rmsnorm(const float* x, const int* pick, const float* w, float eps, void* out, int out_dtype, float* out32,
                             int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
+    llmx_note_launch(LK_RMSNORM);
     const bool kept = n <= RMS_THREADS * RMS_KEPT;
     if (out_dtype == LLMX_F32) {
         if (kept) hipLaunchKernelGGL(rmsnorm_kept_kernel<float>, dim3(rows), dim3(RMS_THREADS), 0, stream, x, pick, w, eps, (float*)out, out32, n);
@@ -143,6 +145,7 @@ __global__ void __launch_bounds__(256) moe_combine4_kernel(float* __restrict__ x
 extern "C" int llmx_moe_combine(float* x, const float* y, const int* ids, const float* w, int rows, int k, int width, int accumulate,
                                 hipStream_t stream) {
     if (rows <= 0) return 0;
+    llmx_note_launch(LK_MOE_COMBINE);
     if (rows > 64 && width % 4 == 0)
         hipLaunchKernelGGL(moe_combine4_kernel, dim3((width / 4 + 255) / 256, rows), dim3(256), 0, stream, x, y, ids, w, k, width, accumulate);
     else

@@ -115,6 +115,7 @@ __global__ void __launch_bounds__(64) argmax_merge_kernel(const float* __restric
 // `partial` holds rows * ceil(n / 8192) leaders (8 bytes each); it may be null for rows of at most 16384 scores.
 extern "C" int llmx_argmax_rows(const float* scores, const int* skip, int* out, void* partial, int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
+    llmx_note_launch(LK_ARGMAX_ROWS);
     if (n <= 2 * ARGMAX_SLICE || !partial) {
         hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, skip, out, n);
         return LLMX_CHECK_LAUNCH();
@@ -174,6 +175,7 @@ extern "C" int llmx_no_alloc_init(void) {
 extern "C" int llmx_argmax_rows_static(const float* scores, const int* skip, int* out, int rows, int n, hipStream_t stream) {
     no_alloc_error[0] = 0;
     if (rows <= 0) return 0;
+    llmx_note_launch(LK_ARGMAX_ROWS);
     if (n <= 0) {
         snprintf(no_alloc_error, sizeof no_alloc_error, "llmx_argmax_rows_static: rows of %d scores", n);
         return -2;
@@ -253,6 +255,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_all_kernel(const float*
 extern "C" int llmx_sample_all(const float* scores, const float* temp, const float* unit, const float* min_p, const int* skip, int* out,
                                int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
+    llmx_note_launch(LK_SAMPLE_ALL);
     hipLaunchKernelGGL(sample_all_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, unit, min_p, skip, out, n);
     return LLMX_CHECK_LAUNCH();
 }
@@ -279,6 +282,7 @@ __global__ void penalize_kernel(float* __restrict__ scores, const int* __restric
 extern "C" int llmx_penalize(float* scores, const int* rows, const int* ids, const int* counts, const float* penalty,
                              const float* presence, const float* frequency, int n_seen, int n, hipStream_t stream) {
     if (n_seen <= 0) return 0;
+    llmx_note_launch(LK_PENALIZE);
     hipLaunchKernelGGL(penalize_kernel, dim3((n_seen + 255) / 256), dim3(256), 0, stream, scores, rows, ids, counts, penalty, presence,
                        frequency, n_seen, n);
     return LLMX_CHECK_LAUNCH();
@@ -482,6 +486,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_topk_kernel(const float
 extern "C" int llmx_sample_topk(const float* scores, const float* temp, const int* top_k, const float* top_p, const float* min_p,
                                 const float* unit, const int* skip, int* out, int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
+    llmx_note_launch(LK_SAMPLE_TOPK);
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n);
     return LLMX_CHECK_LAUNCH();
 }
@@ -729,6 +734,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const flo
 extern "C" int llmx_sample_ranked(const float* scores, const float* temp, const int* top_k, const float* top_p, const float* min_p,
                                   const float* unit, const int* skip, int* out, int rows, int n, hipStream_t stream) {
     if (rows <= 0) return 0;
+    llmx_note_launch(LK_SAMPLE_RANKED);
     if (n <= 0 || n > (1 << 30)) return -2;
     hipLaunchKernelGGL(sample_ranked_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n);
     return LLMX_CHECK_LAUNCH();

@@ -79,6 +79,7 @@ def _declare(h) -> None:
         "llmx_sample_ranked": [P, P, P, P, P, P, P, P, I, I, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
     }
+    sigs.update({"llmx_note_launch": [I], "llmx_launch_kinds": [], "llmx_launch_name": [I], "llmx_take_launches": [P, I]})
     for name, args in sigs.items():
         try:
             fn = getattr(h, name)
@@ -86,6 +87,8 @@ def _declare(h) -> None:
             raise KernelError(f"the kernel library lacks {name}; build it again from the current sources") from None
         fn.argtypes = args
         fn.restype = c_int
+    h.llmx_launch_name.restype = ctypes.c_char_p
+    h.llmx_note_launch.restype = None
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -126,6 +129,24 @@ def _check(rc: int, what: str) -> None:
         raise KernelError(f"{what}: a size this kernel does not take")
     if rc != 0:
         raise KernelError(f"{what}: launch failed with HIP error {rc}")
+
+
+def launch_kinds() -> list:
+    """The names under which the library counts its launches: one for every kernel form of every entry point."""
+    h = lib()
+    return [h.llmx_launch_name(i).decode() for i in range(h.llmx_launch_kinds())]
+
+
+def take_launches() -> dict:
+    """Which kernel forms were launched since the last call, by name, with their counts (forms that were not are
+    left out); the counts are cleared.  The library counts on the host at every launch site, so this tells a test which
+    of several kernels with equal results ran (/root/reference/src/backends/backend.hpp:96-112 keeps such a record for
+    the same purpose).  A launch recorded into a HIP graph counts once, at the recording, not at replays."""
+    h = lib()
+    n = h.llmx_launch_kinds()
+    counts = (c_long * n)()
+    h.llmx_take_launches(counts, n)
+    return {h.llmx_launch_name(i).decode(): int(counts[i]) for i in range(n) if counts[i]}
 
 
 # ---------------------------------------------------------------------------

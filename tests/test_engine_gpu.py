@@ -427,11 +427,29 @@ def test_real_layer_widths(wide_folder, dtype):
     tol = 3e-5 if dtype == "float32" else BF16_TOL
     assert float((whole.double() - want).abs().max()) <= tol * float(want.abs().max())
     # in portions (70 rows take the tiled kernels, 2 and 13 the streaming ones) and token by token at the end
-    engine.add_request("p")
+    from llmx_amd import ops
+    engine.add_request("p")       # the observer stays set, so no step is recorded as a graph and every launch is counted
     cuts = [(0, 70), (70, 72), (72, 85), (85, 140)] + [(i, i + 1) for i in range(140, 150)]
-    rows = torch.cat([engine.step([StepEntry("p", tokens[a:b], list(range(b - a)))]).clone() for a, b in cuts]).cpu()
+    rows, launched = [], []
+    for a, b in cuts:
+        ops.take_launches()
+        rows.append(engine.step([StepEntry("p", tokens[a:b], list(range(b - a)))]).clone())
+        launched.append(ops.take_launches())
+    rows = torch.cat(rows).cpu()
     engine.end_request("p")
     assert torch.equal(rows, whole), f"portions differ from the whole prompt in {dtype}"
+    universal = {"gemm_generic", "gemm_generic.grouped", "attention.generic"}
+    if dtype == "bfloat16":
+        assert not any(universal & set(l) for l in launched), "a bfloat16 step at the real widths fell to the universal kernels"
+        assert {"gemm_tile.64", "gemm_tile.grouped_64", "attention.tiles128", "gemm_f32.staged"} <= set(launched[0])      # 70 rows
+        assert {"gemm_skinny", "gemm_skinny.grouped", "route_topk_align"} <= set(launched[1]) and not any(k.startswith("gemm_tile") for k in launched[1])
+        assert {"gemm_skinny", "gemm_skinny.grouped"} <= set(launched[2])                                            # 13 rows
+        # one row: the norms are formed inside the products, the context's segments go to workgroups of four waves
+        assert {"gemm_skinny.normed", "gemm_skinny.grouped_normed", "gemm_f32.normed", "attention.split4", "attention.merge"} <= set(launched[-1])
+        assert launched[-1].get("rmsnorm", 0) == 1                      # only the final norm runs as a kernel of its own
+    else:
+        assert all(universal <= set(l) for l in launched)
+        assert not any(k.startswith(("gemm_skinny", "gemm_tile", "attention.")) and k != "attention.generic" for l in launched for k in l)
 
 
 def test_a_long_portion_takes_the_wide_tiles_and_gives_the_bits_of_short_ones(wide_folder):
@@ -443,10 +461,19 @@ def test_a_long_portion_takes_the_wide_tiles_and_gives_the_bits_of_short_ones(wi
     tokens = [rng.randrange(1000) for _ in range(800)]
     want_rows = list(range(0, 800, 37)) + [799]
     engine = Engine.load(wide_folder, dtype="bfloat16", kv_tokens=2048, page_tokens=16, max_requests=2)
+    from llmx_amd import ops
     engine.add_request("w")
+    ops.take_launches()
     whole = engine.step([StepEntry("w", tokens, want_rows)]).clone()
+    launched = ops.take_launches()
     engine.end_request("w")
     assert bool(torch.isfinite(whole).all())
+    # QKV: 7 x 32 wide tiles fill the chip; the output projection (7 x 12) takes 64-row tiles; 6,400 pairs are launched
+    # in a 128-row form (wide for K = 3072, four waves for K = 1536) beside the 64-row form, chosen on the device
+    assert launched.get("gemm_tile.wide", 0) == 1 and launched.get("gemm_tile.64", 0) == 1
+    assert launched.get("gemm_tile.grouped_wide", 0) == 1 and launched.get("gemm_tile.grouped_128", 0) == 1
+    assert launched.get("gemm_tile.grouped_64", 0) == 2 and launched.get("attention.tiles128", 0) == 1
+    assert not {"gemm_generic", "gemm_generic.grouped", "attention.generic"} & set(launched)
     engine.add_request("p")
     rows = []
     for a, b in [(0, 300), (300, 330), (330, 650), (650, 799), (799, 800)]:

@@ -117,3 +117,24 @@ def test_attention_options_outside_what_is_built_are_refused_by_name():
         build_part("mixer", PartSpec("attention", {**base, "scale": 0.0}), ctx)
     a = build_part("mixer", PartSpec("attention", {**base, "scale": 0.3}), ctx)
     assert a.scale == pytest.approx(0.3) and build_part("mixer", PartSpec("attention", base), ctx).scale == pytest.approx(0.25)
+
+
+def test_the_launch_witness_counts_by_name_and_clears():
+    """The counters are host memory of the built library: noted launches come back by name once, then nothing; kinds
+    outside the list are ignored; an entry point that returns before it launches notes nothing."""
+    from llmx_amd import ops
+    kinds = ops.launch_kinds()
+    assert len(kinds) == len(set(kinds)) and {"gemm_skinny", "gemm_tile.wide", "gemm_generic", "attention.split4", "attention.generic"} <= set(kinds)
+    ops.take_launches()
+    h = ops.lib()
+    for name, times in (("gemm_tile.wide", 3), ("attention.merge", 1)):
+        for _ in range(times):
+            h.llmx_note_launch(kinds.index(name))
+    h.llmx_note_launch(-1)
+    h.llmx_note_launch(len(kinds))
+    assert h.llmx_launch_name(len(kinds)) is None
+    assert ops.take_launches() == {"gemm_tile.wide": 3, "attention.merge": 1}
+    assert ops.take_launches() == {}
+    # a product of no rows returns before its launch site
+    assert h.llmx_gemm_tile(0, 0, 0, 1, 0, 128, 64, 64, 128, 0, 1, 0, 0, 0, 0, 1, 0, 0, 0, 0) == 0
+    assert ops.take_launches() == {}
