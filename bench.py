@@ -1,6 +1,6 @@
 """Decode and prefill throughput of MiniMax-M3 at real layer sizes with random weights, on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--points 1,64] [--no-sweep] [--long]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C] [--points 1,64] [--no-sweep] [--no-long]
 
 A step is one decode step of the whole batch: B requests, each at a context that reaches C tokens at the last timed
 step, one new token each, logits -> greedy token on the device -> ids read back (the reference's batched `tg`,
@@ -20,10 +20,16 @@ step, one new token each, logits -> greedy token on the device -> ids read back 
                        first layer's feed-forward alone (first_layer_*): its rows are all different, so it touches every
                        expert and streams all their weights;
   sweep                further sizes (left out with --no-sweep, or when --points is empty and --sweep is not given): batch 8
-                       at 16k and 32k tokens of context, batch 16 and 32 at 4k (tok/s, _ms, _experts, _frac), and the mixed
-                       step a scheduler issues: a 512-token prompt portion beside 8 decoding requests;
-  long (--long)        the long-context configuration: 30 layers, 2 requests of 65,536 prompt tokens in portions of
-                       2,048, then 256 decoded tokens each (the engine is freed and built again for it);
+                       at 16k and 32k tokens of context, batch 16, 32 and 128 at 4k, batch 64 at 8k (tok/s, _ms, _frac;
+                       batch 64 at 16k would hold 103 GB of cache beside 178.6 GB of weights and does not fit the card);
+                       the mixed step a scheduler issues: a 512-token prompt portion beside 8 decoding requests;
+                       generate_b1: batch 1 through the product's own loop with the default sampler, beside decode_b1;
+                       prefill_8192: one prompt of 8,192 tokens in portions of 2,048 (tok/s, _ms, _frac of the bf16 peak);
+                       prefill_spread: 2,048 rows as 64 requests of 32 tokens in one step, whose rows pick most experts in
+                       every layer, so the step streams weights (_ms, _experts a layer, _frac of 8 TB/s);
+  long                 the long-context configuration (left out with --no-long or when another --layers, --batch or
+                       --context is asked for): 30 layers, 2 requests of 65,536 prompt tokens in portions of 2,048, then
+                       256 decoded tokens each (the first engine is freed and another built for it);
   calibration          what a device copy, a read-only pass and a square bf16 library product reach on this card.
 Token ids are a fixed LCG sequence; weights are N(0, 0.02) generated on the device.  The context before the timed steps
 is built by running each request's prompt through the model in portions of 2,048 tokens (`context_fill` gives its rate).
@@ -59,7 +65,8 @@ def parse():
     ap.add_argument("--points", default="1,64", help="other batch sizes to measure, comma separated ('' for none)")
     ap.add_argument("--sweep", action="store_true", help="measure further contexts and batches and the mixed prompt + decode step (the default whenever --points names a batch)")
     ap.add_argument("--no-sweep", action="store_true", help="leave those out")
-    ap.add_argument("--long", action="store_true", help="also run the long-context configuration (30 layers, 2 x 65,536 tokens, 256 decoded)")
+    ap.add_argument("--long", action="store_true", help="run the long-context configuration (30 layers, 2 x 65,536 tokens, 256 decoded) also beside a non-default run")
+    ap.add_argument("--no-long", action="store_true", help="leave the long-context configuration out of the default run")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-calibration", action="store_true", help="skip the copy, read and library-product rates of the card")
     ap.add_argument("--no-logits-to-host", action="store_true",
@@ -274,6 +281,54 @@ def run_prefill(engine, cfg, sampler_out, torch):
             "first_layer_hbm_frac": round(first_bytes / first / 1e9 / HBM_PEAK_GBS, 4)}
 
 
+def run_prefill_portions(engine, cfg, total, torch):
+    """One prompt of `total` tokens from an empty cache in portions of 2,048 to its last row's logits; best of two."""
+    from llmx_amd.engine import StepEntry
+    times = []
+    for rep in range(2):
+        rid = f"pp{rep}"
+        engine.add_request(rid)
+        ids = lcg_ids(total, cfg.vocab_size, 600 + rep)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for s in range(0, total, PREFILL_TOKENS):
+            part = ids[s:s + PREFILL_TOKENS]
+            engine.step([StepEntry(rid, part, [len(part) - 1] if s + len(part) == total else [])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.end_request(rid)
+    t = min(times)
+    return {"tok_s": round(total / t, 1), "ms": round(t * 1e3, 3), "frac": round(prefill_flops(cfg, total) / t / PEAK_FLOPS["bf16"], 4)}
+
+
+def run_prefill_spread(engine, cfg, requests, tokens_each, torch):
+    """`requests` prompts of `tokens_each` tokens in one step from an empty cache.  Short prompts of different tokens keep
+    their rows apart through the layers, so every layer's rows pick most of the experts: the step has to stream their
+    weights, where one long prompt's rows (which grow alike with random weights) pick few.  Best of two after a warm-up."""
+    from llmx_amd.engine import StepEntry
+    watcher = DistinctExperts()
+    times = []
+    for rep in range(3):
+        rids = [f"ps{rep}_{i}" for i in range(requests)]
+        entries = []
+        for i, rid in enumerate(rids):
+            engine.add_request(rid)
+            entries.append(StepEntry(rid, lcg_ids(tokens_each, cfg.vocab_size, 3000 + 97 * rep + i), [tokens_each - 1]))
+        engine.observer = watcher if rep == 0 else None
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step(entries)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.observer = None
+        for rid in rids:
+            engine.end_request(rid)
+    t = min(times[1:])
+    need = decode_bytes(cfg, 0, 0, watcher.mean)
+    return {"ms": round(t * 1e3, 3), "experts": round(watcher.mean, 1), "gb": round(need / 1e9, 1), "frac": round(need / t / 1e9 / HBM_PEAK_GBS, 4),
+            "tok_s": round(requests * tokens_each / t, 1)}
+
+
 def run_mixed_step(engine, cfg, sampler_out, context, portion, decoding, reps, torch):
     """The step a scheduler issues while a prompt arrives: `decoding` requests at `context` tokens take one token each
     beside a `portion`-token portion of another request's prompt.  Returns ms a step (mean of `reps`) and tokens a second."""
@@ -380,9 +435,11 @@ def main():
     layers = a.layers or FULL_LAYERS
     points = [int(p) for p in a.points.split(",") if p.strip()]
     do_sweep = a.sweep or (bool(points) and not a.no_sweep)
-    sweep = [(8, 16384), (8, 32768), (16, context), (32, context)] if do_sweep else []
+    # the long-context configuration belongs to the default run; a run at other sizes (a test, a profile) asks for it
+    do_long = a.long or (not a.no_long and not (a.layers or a.context) and a.batch == 8 and bool(points))
+    sweep = [(8, 16384), (8, 32768), (16, context), (32, context), (128, context), (64, 2 * context)] if do_sweep else []
     kv_tokens = max([a.batch * context] + [b * context for b in points] + [b * c for b, c in sweep] + ([9 * context] if do_sweep else []))
-    max_batch = max([a.batch] + points + [b for b, _ in sweep] + ([9] if do_sweep else []))
+    max_batch = max([a.batch] + points + [b for b, _ in sweep] + ([64] if do_sweep else []))
     cfg = real_config(layers, max([context] + [c for _, c in sweep]))
     t_setup = time.perf_counter()
     engine = Engine.from_random(cfg, RandomInit(seed=0, std=0.02), dtype="bfloat16", kv_tokens=kv_tokens, page_tokens=16, max_requests=max_batch)
@@ -441,18 +498,28 @@ def main():
             rec = decode_record(cfg, b, c, a.steps, run_decode(engine, sampler_out, b, c, a.steps, a.warmup, torch))
             name = f"decode_b{b}_ctx{c}"
             sw[name] = rec["tok_s"]
-            for key in ("ms", "experts", "frac"):
+            for key in ("ms", "frac"):
                 sw[f"{name}_{key}"] = rec[key]
         mixed = run_mixed_step(engine, cfg, sampler_out, context, 512, 8, 8, torch)
         sw["mixed_512_beside_8_ms"] = mixed["ms"]
         sw["mixed_512_beside_8_tok_s"] = mixed["tok_s"]
+        # batch 1 through the scheduler, the step and the device sampler, beside the bare step of decode_b1
+        g1 = run_generate(engine, cfg, 1, context, 2 * a.steps, torch)
+        sw["generate_b1"], sw["generate_b1_ms"] = g1["tok_s"], g1["ms"]
+        if "decode_b1_gb" in pts:
+            sw["generate_b1_frac"] = round(pts["decode_b1_gb"] / g1["ms"] / (HBM_PEAK_GBS / 1e3), 4)
+        if not a.no_prefill:
+            p8 = run_prefill_portions(engine, cfg, 4 * PREFILL_TOKENS, torch)
+            sw["prefill_8192"], sw["prefill_8192_ms"], sw["prefill_8192_frac"] = p8["tok_s"], p8["ms"], p8["frac"]
+            sp = run_prefill_spread(engine, cfg, 64, PREFILL_TOKENS // 64, torch)
+            sw["prefill_spread_ms"], sw["prefill_spread_experts"], sw["prefill_spread_frac"] = sp["ms"], sp["experts"], sp["frac"]
         result["sweep"] = sw
 
     if not a.no_prefill:
         result["prefill"] = run_prefill(engine, cfg, sampler_out, torch)
     if not a.no_calibration:
         result["calibration"] = calibrate(torch, sampler_out.device)
-    if a.long:
+    if do_long:
         del engine
         torch.cuda.empty_cache()
         result["long"] = run_long(torch)

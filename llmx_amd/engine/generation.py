@@ -53,11 +53,12 @@ class Generator:
         """One round: admit, plan, run, sample, advance.  Returns the requests that finished in it.
 
         When the round fails (a refused step, a kernel error) every running request is ended in the engine before the
-        error goes on, so that nothing stays open holding a slot and pages."""
+        error goes on, and retired in the scheduler (finish reason "error", its reservation returned), so that nothing stays open holding a
+        slot and pages and the generator can go on with the requests that wait."""
         try:
             return self._round(on_token)
         except BaseException:
-            for r in self.scheduler.running:
+            for r in self.scheduler.fail_running():
                 if self.engine.has_request(r.id):
                     self.engine.end_request(r.id)
             raise

@@ -40,7 +40,7 @@ class Request:
     generated: List[int] = field(default_factory=list)
     fed: int = 0                       # tokens of prompt + generated already in the cache
     state: str = "waiting"             # waiting | running | finished
-    finish_reason: Optional[str] = None  # "eos" | "stop" | "length"
+    finish_reason: Optional[str] = None  # "eos" | "stop" | "length" | "error"
     reserved: List[int] = field(default_factory=list)
     rng: XorShift64 = None
     order: int = -1                    # order of admission
@@ -172,6 +172,20 @@ class Scheduler:
             r.state = "finished"
             self.finished[r.id] = r
         return done
+
+    def fail_running(self) -> List[Request]:
+        """The round failed: every running request is retired with finish reason "error" and its reservation returned;
+        requests that wait stay in the queue.  Returns the retired requests."""
+        failed = list(self.running)
+        for r in failed:
+            for i, n in enumerate(r.reserved):
+                self.reserved[i] -= n
+            r.reserved = []
+            r.state = "finished"
+            r.finish_reason = "error"
+            self.finished[r.id] = r
+        self.running.clear()
+        return failed
 
     @property
     def idle(self) -> bool:

@@ -21,6 +21,7 @@ class Sampler:
     def __init__(self, vocab_size: int, device: torch.device):
         self.vocab = vocab_size
         self.device = device
+        self._kept = None     # (key, settings) of the last rows sampled
 
     def _f32(self, values) -> torch.Tensor:
         return torch.tensor(np.asarray(values, dtype=np.float32), device=self.device)
@@ -50,38 +51,52 @@ class Sampler:
         if rows:
             ops.penalize(logits, self._i32(rows), self._i32(ids), self._i32(counts), self._f32([p.penalty for p in params]),
                          self._f32([p.presence_penalty for p in params]), self._f32([p.frequency_penalty for p in params]))
-        skip = None
-        if eos is not None and any(p.ignore_eos for p in params):
-            skip = self._i32([eos if p.ignore_eos else -1 for p in params])
+        st = self._settings(params, eos)
+        skip = st["skip"]
         out = torch.empty(W, dtype=torch.int32, device=self.device)
-        if all(p.greedy for p in params):
+        if st["greedy"]:
             ops.argmax_rows(logits, out, skip)
             return out.tolist()
-        units = [0.0 if p.greedy else rng.unit() for p, rng in zip(params, rngs)]
-        temp = self._f32([p.temp for p in params])
-        unit = self._f32(units)
-        min_p = self._f32([p.min_p for p in params])
-        # ids a draw can give: all, less a masked end token; a top_k that leaves them all is no top_k
-        m = [self.vocab - (1 if (eos is not None and p.ignore_eos and 0 <= eos < self.vocab and self.vocab > 1) else 0) for p in params]
-        # which kernel takes a row: everything kept and no nucleus: the walk over the whole row; a top-k of at most
-        # MAX_EXACT_TOP_K: ranked whole in LDS; anything else (a larger top-k, a nucleus over the whole row): the search
-        # by histograms.  With mixed settings each kernel in use runs over all rows and a row takes the result of its own.
-        def kernel_of(p, mr):
-            if p.greedy or ((p.top_k <= 0 or p.top_k >= mr) and p.top_p >= 1.0):
-                return "all"
-            return "topk" if 0 < p.top_k <= MAX_EXACT_TOP_K else "ranked"
-        which = [kernel_of(p, mr) for p, mr in zip(params, m)]
+        unit = self._f32([0.0 if p.greedy else rng.unit() for p, rng in zip(params, rngs)])
+        temp, min_p, which = st["temp"], st["min_p"], st["which"]
         results = {}
         if "all" in which:
             ops.sample_all(logits, temp, unit, out, min_p, skip)
             results["all"] = out
-        if "topk" in which or "ranked" in which:
-            top_k, top_p = self._i32([p.top_k for p in params]), self._f32([p.top_p for p in params])
-            for name, kernel in (("topk", ops.sample_topk), ("ranked", ops.sample_ranked)):
-                if name in which:
-                    results[name] = torch.zeros(W, dtype=torch.int32, device=self.device)
-                    kernel(logits, temp, top_k, top_p, min_p, unit, results[name], skip)
+        for name, kernel in (("topk", ops.sample_topk), ("ranked", ops.sample_ranked)):
+            if name in which:
+                results[name] = torch.zeros(W, dtype=torch.int32, device=self.device)
+                kernel(logits, temp, st["top_k"], st["top_p"], min_p, unit, results[name], skip)
         if len(results) == 1:
             return next(iter(results.values())).tolist()
         lists = {name: t.tolist() for name, t in results.items()}
         return [lists[name][row] for row, name in enumerate(which)]
+
+    def _settings(self, params: Sequence[SamplingParams], eos: Optional[int]) -> dict:
+        """The rows' settings as device tensors, and which kernel takes each row.  They change only when the set of
+        running requests does, so the last set is kept: a decode loop then uploads one tensor a step (the uniforms)."""
+        key = (eos, tuple((p.temp, p.top_k, p.top_p, p.min_p, p.ignore_eos) for p in params))
+        if self._kept is not None and self._kept[0] == key:
+            return self._kept[1]
+        st = {"greedy": all(p.greedy for p in params), "skip": None}
+        if eos is not None and any(p.ignore_eos for p in params):
+            st["skip"] = self._i32([eos if p.ignore_eos else -1 for p in params])
+        if not st["greedy"]:
+            # ids a draw can give: all, less a masked end token; a top_k that leaves them all is no top_k
+            m = [self.vocab - (1 if (eos is not None and p.ignore_eos and 0 <= eos < self.vocab and self.vocab > 1) else 0) for p in params]
+
+            # which kernel takes a row: everything kept and no nucleus: the walk over the whole row; a top-k of at most
+            # MAX_EXACT_TOP_K: ranked whole in LDS; anything else (a larger top-k, a nucleus over the whole row): the
+            # search by histograms.  With mixed settings each kernel in use runs over all rows and a row takes the
+            # result of its own.
+            def kernel_of(p, mr):
+                if p.greedy or ((p.top_k <= 0 or p.top_k >= mr) and p.top_p >= 1.0):
+                    return "all"
+                return "topk" if 0 < p.top_k <= MAX_EXACT_TOP_K else "ranked"
+            st["which"] = [kernel_of(p, mr) for p, mr in zip(params, m)]
+            st["temp"] = self._f32([p.temp for p in params])
+            st["min_p"] = self._f32([p.min_p for p in params])
+            if "topk" in st["which"] or "ranked" in st["which"]:
+                st["top_k"], st["top_p"] = self._i32([p.top_k for p in params]), self._f32([p.top_p for p in params])
+        self._kept = (key, st)
+        return st

@@ -55,8 +55,27 @@ def test_the_record_of_one_real_layer():
     assert pre["tokens"] == 2048 and abs(pre["value"] - 2048 * 1e3 / pre["ms"]) < 0.01 * pre["value"]
     assert abs(pre["frac"] - pre["tflop"] * 1e12 / (pre["ms"] * 1e-3) / 2.5e15) < 2e-3
     assert 0 < pre["hbm_frac"] < 1 and pre["first_layer_experts"] > 200 and 0 < pre["first_layer_hbm_frac"] < 1
+    # the bytes a step has to read, written out here for batch 8 at one layer: the attention's four projections, the
+    # router, bias and norm weights in float32, the experts the step touched (three matrices each), the head and the
+    # final norm, eight embedding rows, and keys and values of eight requests at the mean context of the timed steps
+    experts = pts["decode_b8_experts"]
+    want_bytes = ((6144 + 2 * 1024) * 3072 * 2 + 3072 * 6144 * 2            # q, k, v and o projections in bfloat16
+                  + 256 * 3072 * 4 + 256 * 4                               # router matrix and correction bias in float32
+                  + (2 * 3072 + 6144 + 1024) * 4                           # two layer norms, the q and k projection norms
+                  + experts * 3 * 1536 * 3072 * 2                          # gate, up and down of each distinct expert
+                  + 200064 * 3072 * 2 + 3072 * 4                           # head and final norm
+                  + 8 * 3072 * 2                                           # embedding rows
+                  + 8 * (4096 - 3 / 2) * 2 * 1024 * 2)                     # keys and values of 8 requests (8 heads of 128)
+    assert abs(pts["decode_b8_gb"] - want_bytes / 1e9) <= 0.006, (pts["decode_b8_gb"], want_bytes / 1e9)
+    assert roof["bytes_gb"] == pts["decode_b8_gb"]
     sw = rec["sweep"]
-    assert len(sw) <= 20 and all(not isinstance(v, (dict, list)) for v in sw.values())
-    for name in ("decode_b8_ctx16384", "decode_b8_ctx32768", "decode_b16_ctx4096", "decode_b32_ctx4096"):
+    assert all(not isinstance(v, (dict, list)) for v in sw.values())
+    for name in ("decode_b8_ctx16384", "decode_b8_ctx32768", "decode_b16_ctx4096", "decode_b32_ctx4096", "decode_b128_ctx4096",
+                 "decode_b64_ctx8192"):
         assert sw[name] > 0 and sw[name + "_ms"] > 0 and 0 < sw[name + "_frac"] < 1
     assert sw["mixed_512_beside_8_ms"] > 0
+    assert sw["generate_b1"] > 0 and sw["generate_b1_ms"] > 0 and 0 < sw["generate_b1_frac"] < 1
+    assert sw["prefill_8192"] > 0 and sw["prefill_8192_ms"] > 0 and 0 < sw["prefill_8192_frac"] < 1
+    # 64 short prompts of different tokens pick most of the 256 experts, where one long prompt's rows pick few
+    assert sw["prefill_spread_ms"] > 0 and sw["prefill_spread_experts"] > 150 and 0 < sw["prefill_spread_frac"] < 1
+    assert "long" not in rec        # the long-context configuration belongs to the default run only

@@ -441,7 +441,7 @@ def test_real_layer_widths(wide_folder, dtype):
     universal = {"gemm_generic", "gemm_generic.grouped", "attention.generic"}
     if dtype == "bfloat16":
         assert not any(universal & set(l) for l in launched), "a bfloat16 step at the real widths fell to the universal kernels"
-        assert {"gemm_tile.64", "gemm_tile.grouped_64", "attention.tiles128", "gemm_f32.staged"} <= set(launched[0])      # 70 rows
+        assert {"gemm_tile.64", "gemm_tile.grouped_64", "attention.tiles128", "gemm_f32.skinny"} <= set(launched[0])      # 70 rows
         assert {"gemm_skinny", "gemm_skinny.grouped", "route_topk_align"} <= set(launched[1]) and not any(k.startswith("gemm_tile") for k in launched[1])
         assert {"gemm_skinny", "gemm_skinny.grouped"} <= set(launched[2])                                            # 13 rows
         # one row: the norms are formed inside the products, the context's segments go to workgroups of four waves

@@ -52,6 +52,10 @@ def test_a_failing_round_leaves_no_request_open():
     with pytest.raises(RuntimeError, match="the step failed"):
         gen.step()
     assert eng.cache.pages_in_use() == 0 and eng.cache.slots.in_use == 0 and eng.cache.live() == []
-    # the same ids can be opened again: nothing of the failed run is left
-    eng.add_request(0)
-    eng.add_request(1)
+    # the scheduler retired them too: reservations returned, nothing running, both finished with reason "error"
+    sch = gen.scheduler
+    assert sch.reserved == [0] and sch.idle and not sch.running
+    assert {r.finish_reason for r in sch.finished.values()} == {"error"} and set(sch.finished) == {0, 1}
+    # the scheduler goes on: a request submitted after the failure finds every seat and page free
+    gen.submit(Request(2, list(range(5)), SamplingParams(max_tokens=1, temp=0.0)))
+    assert [r.id for r in sch.admit()] == [2]
