@@ -107,7 +107,7 @@ class StepState:
         self.token_ids = self.positions = self.row_entry = self.entry_slots = self.pick = None
         self._tables: List[torch.Tensor] = []
         self.max_rows_per_entry = 0
-        self._plans = {}
+        self._shared: Dict = {}
         self.run_index = -1          # which item of the run order is running
         self.observer = None         # callable(step, kind, **tensors) that sees what parts choose to show, or None
 
@@ -117,20 +117,15 @@ class StepState:
     def tables(self, group: int) -> torch.Tensor:
         return self._tables[group]
 
-    def attention_plan(self, n_heads: int, n_kv_heads: int, window: int = 0):
-        """The matrix-core attention kernel's work items for this step's rows (shared by layers with the same heads)."""
-        key = (n_heads, n_kv_heads, window)
-        plan = self._plans.get(key)
-        if plan is None:
-            from .. import ops
-            plan = ops.attention_plan([e.n for e in self.entries], [e.past + e.n for e in self.entries], n_heads, n_kv_heads, self.device,
-                                      window)
-            self._plans[key] = plan
-        return plan
-
-    def plan_requests(self):
-        """The (heads, kv heads, window) attention plans were asked for in this step."""
-        return list(self._plans.keys())
+    def shared(self, key, make):
+        """Something a part wants once a step: `make()` is called at the key's first use in this step; every later use
+        (another layer with the same sizes) gets the same object.  A kernel's work plan for the step's rows, a second
+        stream of positions, anything that depends on the step and not on the layer."""
+        try:
+            return self._shared[key]
+        except KeyError:
+            value = self._shared[key] = make()
+            return value
 
     def observe(self, kind: str, **tensors) -> None:
         """Shows intermediate tensors (a router's picks, for instance) to the engine's observer, when one is set."""

@@ -18,8 +18,8 @@ import torch
 from .. import ops
 from ..cache import CacheManager, GroupSpec, OutOfPages
 from ..models import registry
-from ..parts.base import BuildContext, LayerCache
-from ..parts.spec import KVNeed, ModelSpec, StateNeed
+from ..parts.base import BuildContext, LayerCache, Part
+from ..parts.spec import ModelSpec, PagedNeed, StateNeed
 from ..weights import ModelFiles, RandomInit, load as load_weights
 from ..weights.loader import device_dtype
 from ..weights.random_init import fill_random, stored_dtype
@@ -42,10 +42,10 @@ def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
 class _StepGraph:
     """A recorded decode step: the graph, where its logits appear, and what must not have moved since."""
 
-    def __init__(self, graph, logits, plans, workspace_generation, uploader_generation):
+    def __init__(self, graph, logits, shared, workspace_generation, uploader_generation):
         self.graph = graph
         self.logits = logits
-        self.plans = plans      # kept alive: the graph's kernels read their work items
+        self.shared = shared    # kept alive: what the parts made for the step (work plans the graph's kernels read)
         self.generations = (workspace_generation, uploader_generation)
 
     def stale(self, engine: "Engine") -> bool:
@@ -79,7 +79,7 @@ class Engine:
         self.step_tokens = step_tokens
         self.max_positions = min(spec.max_positions, self.kv_tokens)
         torch.cuda.set_device(self.device)
-        ctx = BuildContext(self.act_dtype, self.device, self.max_positions)
+        ctx = BuildContext(self.act_dtype, self.device, self.max_positions, self.page_tokens)
         self.model = BuiltModel(spec, ctx)
         self._loaded = False
         if weights is not None:
@@ -95,7 +95,8 @@ class Engine:
             and all(getattr(b, "graph_safe", False) for b in self.model.blocks)
         self._graphs: Dict[tuple, "_StepGraph"] = {}
         self._graph_seen: Dict[tuple, int] = {}
-        self._plan_requests: set = set()      # the (heads, kv heads, window) the mixers ask attention plans for
+        # the parts that have a say in a recorded step's key (see Part.graph_key)
+        self._keyed_parts = [p for p in self.model.parts() if type(p).graph_key is not Part.graph_key]
         self.graph_replays = 0                # steps that ran as a replay (for tests and measurement)
 
     # -- construction -----------------------------------------------------------
@@ -133,14 +134,16 @@ class Engine:
         return cls(config, registry.assemble(config), dtype, weights=generate, **options)
 
     def _make_cache(self) -> None:
+        """Allocates what the mixers' needs list: for every group of equal paged needs a page pool and, for each of the
+        need's tensors, one arena [caches of the group, pages, *page shape]; for every state need [slots, *shape]."""
         needs = self.model.cache_needs()
         n_pages = self.kv_tokens // self.page_tokens
-        keys: List[KVNeed] = []
+        keys: List[PagedNeed] = []
         self._group_of: List[int] = []          # cache number -> group (or -1)
         self._index_in_group: List[int] = []
         counts: List[int] = []
         for need in needs:
-            if isinstance(need, KVNeed):
+            if isinstance(need, PagedNeed):
                 if need not in keys:
                     keys.append(need)
                     counts.append(0)
@@ -157,9 +160,11 @@ class Engine:
         # a model with per-request state steps into a second slot, so that a step that fails leaves the state as it was
         self._stateful = any(isinstance(need, StateNeed) for need in needs)
         self.cache = CacheManager(groups, self.max_requests, shadow_slots=self._stateful)
-        # [cache in group, K|V, page, kv head, token in page * head dim]; keys are [token][dim], values [dim][token]
-        self._kv = [torch.zeros((counts[g], 2, groups[g].n_pages, need.kv_heads, self.page_tokens * need.head_dim), dtype=self.act_dtype,
-                                device=self.device) for g, need in enumerate(keys)]
+        self._paged: List[Dict[str, torch.Tensor]] = []
+        for g, need in enumerate(keys):
+            self._paged.append({t.name: torch.zeros((counts[g], groups[g].n_pages, *t.page_shape(self.page_tokens)),
+                                                    dtype=getattr(torch, t.dtype) if t.dtype else self.act_dtype, device=self.device)
+                                for t in need.tensors})
         self._state: List[Optional[torch.Tensor]] = []
         for need in needs:
             if isinstance(need, StateNeed):
@@ -170,11 +175,9 @@ class Engine:
         for e in self.spec.run_order:
             g = self._group_of[e.cache]
             if g >= 0:
-                store = self._kv[g][self._index_in_group[e.cache]]
-                need = keys[g]
-                self._layer_caches.append(LayerCache(
-                    group=g, k=store[0].view(groups[g].n_pages, need.kv_heads, self.page_tokens, need.head_dim),
-                    v=store[1].view(groups[g].n_pages, need.kv_heads, need.head_dim, self.page_tokens), writes=e.writes))
+                at = self._index_in_group[e.cache]
+                self._layer_caches.append(LayerCache(group=g, tensors={name: arena[at] for name, arena in self._paged[g].items()},
+                                                     writes=e.writes))
             else:
                 self._layer_caches.append(LayerCache(state=self._state[e.cache], writes=e.writes))
 
@@ -338,12 +341,11 @@ class Engine:
 
         # A step of single decoded tokens launches a few hundred short kernels; replayed as one HIP graph they follow
         # each other without the host.  A graph holds addresses and launch sizes, so it is keyed by all that fixes
-        # them (rows, wanted places, widths of the block tables, the attention plans) and dropped when scratch storage
-        # moves.  The row plan is copied to the device before the replay, outside the graph; the graph holds kernels only.
+        # them (rows, wanted places, widths of the block tables, what the parts add: Part.graph_key) and dropped when
+        # scratch storage moves.  The row plan is copied to the device before the replay, outside the graph; the graph holds kernels only.
         key = None
         if self.graphs and self.observer is None and len(pick) > 0 and all(v.n == 1 for v in views):
-            plans = tuple(step.attention_plan(*req) for req in sorted(self._plan_requests))
-            key = (T, tuple(pick), tuple(a.shape for a in arrays[5:]), tuple(id(p) for p in plans))
+            key = (T, tuple(pick), tuple(a.shape for a in arrays[5:]), tuple(p.graph_key(step) for p in self._keyed_parts))
             graph = self._graphs.get(key)
             if graph is not None and not graph.stale(self):
                 graph.graph.replay()
@@ -354,14 +356,13 @@ class Engine:
                 self._graphs.clear()
                 self._graph_seen.clear()
         if key is not None and self._graph_seen.get(key, 0) >= 1:
-            graph = self._capture(step, key, plans)
+            graph = self._capture(step, key)
             if graph is not None:
                 graph.graph.replay()
                 self.graph_replays += 1
                 self._uploader.mark()
                 return graph.logits
         logits = self._forward(step)
-        self._plan_requests.update(step.plan_requests())
         if key is not None:
             if len(self._graph_seen) > 256:
                 self._graph_seen.clear()
@@ -384,7 +385,7 @@ class Engine:
         self.model.head.forward(step, rows, logits)
         return logits
 
-    def _capture(self, step: StepState, key: tuple, plans: tuple) -> Optional["_StepGraph"]:
+    def _capture(self, step: StepState, key: tuple) -> Optional["_StepGraph"]:
         """Records the step's launches (a step of this shape ran before, so every scratch tensor exists) into a graph."""
         before = (self._workspace.generation, self._uploader.generation)
         graph = torch.cuda.CUDAGraph()
@@ -400,7 +401,7 @@ class Engine:
             return None            # storage moved while recording: the graph holds stale addresses
         if len(self._graphs) >= 32:
             self._graphs.pop(next(iter(self._graphs)))
-        record = _StepGraph(graph, logits, plans, *before)
+        record = _StepGraph(graph, logits, dict(step._shared), *before)
         self._graphs[key] = record
         return record
 
@@ -415,4 +416,4 @@ class Engine:
         return total
 
     def cache_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self._kv) + sum(t.numel() * t.element_size() for t in self._state if t is not None)
+        return sum(t.numel() * t.element_size() for arenas in self._paged for t in arenas.values()) + sum(t.numel() * t.element_size() for t in self._state if t is not None)

@@ -8,7 +8,7 @@ import torch
 
 from ..parts import base as parts_base
 from ..parts.base import BuildContext, build_part
-from ..parts.spec import KVNeed, ModelSpec, StateNeed, TensorSpec
+from ..parts.spec import ModelSpec, PagedNeed, StateNeed, TensorSpec
 
 
 def build_block(spec, ctx: BuildContext):
@@ -47,9 +47,9 @@ class BuiltModel:
         if getattr(self.head, "tied", False):
             self.head.tie(self.embedding.table())
 
-    def cache_needs(self) -> List[Union[KVNeed, StateNeed, None]]:
+    def cache_needs(self) -> List[Union[PagedNeed, StateNeed, None]]:
         """For each cache number of the run order, what its writer keeps."""
-        needs: Dict[int, Union[KVNeed, StateNeed, None]] = {}
+        needs: Dict[int, Union[PagedNeed, StateNeed, None]] = {}
         for e in self.spec.run_order:
             need = self.blocks[e.layer].mixer.cache_need()
             if e.writes:

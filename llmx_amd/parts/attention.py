@@ -84,6 +84,19 @@ class Attention(Mixer):
     def takes_deferred_norm(self, step):
         return ops.gemm_takes_normed_rows(step.rows, self.wqkv, torch.float32)
 
+    def _plan(self, step):
+        """The matrix-core attention kernel's work items for this step's rows: made once a step and shared by every
+        layer with the same heads and window."""
+        window = int(self.window or 0)
+        return step.shared(("attention.plan", self.heads, self.kv_heads, window),
+                           lambda: ops.attention_plan([e.n for e in step.entries], [e.past + e.n for e in step.entries], self.heads,
+                                                      self.kv_heads, step.device, window))
+
+    def graph_key(self, step):
+        # a recorded step holds the plan's addresses and launch sizes; the universal kernel has no plan
+        page = self.ctx.page_tokens
+        return self._plan(step) if page and ops.attention_mfma_ok(step.act_dtype, self.head_dim, page) else None
+
     def forward(self, step, h, out, accumulate, cache: LayerCache, h32=None):
         T = step.rows
         act = step.act_dtype
@@ -96,9 +109,7 @@ class Attention(Mixer):
                                 self.eps, self.heads, self.kv_heads, self.head_dim, rotary, self.norm_mode, write_kv=cache.writes,
                                 pairing=self.pairing)
         o = step.buf("attention.out", (T, self.q_width), act)
-        plan = None
-        if ops.attention_mfma_ok(act, self.head_dim, cache.k.shape[2]):
-            plan = step.attention_plan(self.heads, self.kv_heads, int(self.window or 0))
+        plan = self._plan(step) if ops.attention_mfma_ok(act, self.head_dim, cache.k.shape[2]) else None
         ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
                             window=int(self.window or 0), plan=plan, scratch=step.buf)
         ops.gemm(o, self.wo, out, ops.EPI_ADD if accumulate else ops.EPI_STORE)

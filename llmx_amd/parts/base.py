@@ -13,7 +13,8 @@ What a part sees of a step (the `step` argument, an `engine.batch.StepState`):
   step.entry_slots                int32 [n_entries] on the device: each entry's state slot
   step.tables(group)              int32 [n_entries, max_blocks]: page ids of each entry in cache group `group`
   step.buf(name, shape, dtype)    a scratch tensor that lives until the step ends (same name, same storage)
-  step.attention_plan(heads, kv_heads)  work items of the matrix-core attention kernel for this step's rows
+  step.shared(key, make)          something a part wants once a step (a kernel's work plan, a second position stream):
+                                  make() is called at the key's first use in the step, later uses get the same object
   step.run_index                  which item of the run order is running
   step.observe(kind, **tensors)   shows intermediate tensors to an observer, when the engine has one (tests, probes)
 """
@@ -25,7 +26,7 @@ from typing import Callable, Dict, List, Optional, Sequence, Set, Union
 
 import torch
 
-from .spec import KVNeed, PartSpec, StateNeed, TensorSpec
+from .spec import PagedNeed, PartSpec, StateNeed, TensorSpec
 
 
 @dataclass
@@ -34,6 +35,7 @@ class BuildContext:
     act_dtype: torch.dtype        # float32: the true 32-bit path; bfloat16: the serving path
     device: torch.device
     max_positions: int            # positions the engine can reach (context or the cache's tokens, whichever is smaller)
+    page_tokens: Optional[int] = None   # tokens a cache page holds (None where no cache is made: listing tensors)
 
     @property
     def exact(self) -> bool:
@@ -64,6 +66,13 @@ class Part:
     def name(self, suffix: str) -> str:
         return self.prefix + suffix
 
+    def graph_key(self, step):
+        """What, beyond the step's shape (rows, wanted places, block-table widths), fixes the launches this part makes
+        for `step`: a hashable that the engine folds into the key under which it records and replays a decode step as
+        a HIP graph.  A part whose launches follow a plan made per step (`step.shared`) returns the plan: a step with
+        another plan is then another graph, and the graph keeps the plan alive.  None: nothing more."""
+        return None
+
 
 class Norm(Part):
     def forward(self, step, x: torch.Tensor, out: Optional[torch.Tensor], out32: Optional[torch.Tensor] = None,
@@ -91,12 +100,22 @@ class PositionEncoding(Part):
 
 @dataclass
 class LayerCache:
-    """What one run-order entry's mixer gets of the cache: pages of keys and values, or per-request state."""
+    """What one run-order entry's mixer gets of the cache: its paged tensors by the names of its need, or per-request
+    state."""
     group: int = -1                          # cache group of the pages (index for step.tables)
-    k: Optional[torch.Tensor] = None         # [pages, kv_heads, page_tokens, head_dim]
-    v: Optional[torch.Tensor] = None         # [pages, kv_heads, head_dim, page_tokens] (transposed within the page)
+    tensors: Optional[Dict[str, torch.Tensor]] = None   # name -> [pages, *CacheTensor.page_shape(page_tokens)]
     writes: bool = True                      # False: this entry reads pages another entry wrote
     state: Optional[torch.Tensor] = None     # [slots, *StateNeed.shape]
+
+    @property
+    def k(self) -> torch.Tensor:
+        """Keys of an attention cache: [pages, kv_heads, page_tokens, head_dim]."""
+        return self.tensors["k"]
+
+    @property
+    def v(self) -> torch.Tensor:
+        """Values of an attention cache: [pages, kv_heads, head_dim, page_tokens] (transposed within the page)."""
+        return self.tensors["v"]
 
 
 class Mixer(Part):
@@ -107,7 +126,7 @@ class Mixer(Part):
         """Whether, for this step, forward accepts a Norm.deferred() description as h and h32 in place of tensors."""
         return False
 
-    def cache_need(self) -> Union[KVNeed, StateNeed, None]:
+    def cache_need(self) -> Union[PagedNeed, StateNeed, None]:
         return None
 
     def forward(self, step, h: torch.Tensor, out: torch.Tensor, accumulate: bool, cache: LayerCache,

@@ -20,13 +20,33 @@ class TensorSpec:
     into: (target name, target shape, index): the tensor is one slice of a larger device tensor that the part reads
           instead; the loader allocates the target once and copies each file tensor from the host straight into
           target[index], so the slices are never on the device beside their fused copy.
+    dtype: the tensor's type on the device ("float32" | "bfloat16" | "int32"), whatever the file stores and whichever
+          path runs; None: what the role says.  A part whose parameter is of a kind the roles do not know (a decay
+          kept in float32, a table of 32-bit ids) states it here; loader and random weights follow it.
+    init: how random weights fill it: ("normal", mean, std) | ("uniform", low, high) | ("constant", value); None: what
+          the role says (matrices N(0, std), norm weights 1 + N(0, norm_std), biases U(-range, range) of the run's
+          RandomInit).
     """
     name: str
     shape: Tuple[int, ...]
     role: str = "matrix"
     into: Optional[Tuple[str, Tuple[int, ...], tuple]] = None
+    dtype: Optional[str] = None
+    init: Optional[Tuple] = None
 
     ROLES = ("matrix", "table", "norm", "bias", "router", "int")
+    DTYPES = ("float32", "bfloat16", "int32")
+    INITS = ("normal", "uniform", "constant")
+
+    def __post_init__(self):
+        if self.role not in self.ROLES:
+            raise ValueError(f"tensor {self.name}: role {self.role!r} is not one of {self.ROLES}")
+        if self.dtype is not None and self.dtype not in self.DTYPES:
+            raise ValueError(f"tensor {self.name}: dtype {self.dtype!r} is not one of {self.DTYPES}")
+        if self.init is not None:
+            kind = self.init[0] if self.init else None
+            if kind not in self.INITS or len(self.init) != (2 if kind == "constant" else 3):
+                raise ValueError(f"tensor {self.name}: init {self.init!r} is not (\"normal\", mean, std), (\"uniform\", low, high) or (\"constant\", value)")
 
 
 @dataclass
@@ -67,11 +87,45 @@ class RunEntry:
 
 
 @dataclass(frozen=True)
-class KVNeed:
-    """A mixer that keeps keys and values of every position (window None) or of the last `window` positions."""
-    kv_heads: int
-    head_dim: int
+class CacheTensor:
+    """One tensor a mixer keeps for every token of a request, in pages.
+
+    shape:      the values of one token, e.g. (kv_heads, head_dim) for keys, (latent_width,) for one latent a token;
+    dtype:      a torch dtype name, or None for the engine's activation type;
+    token_axis: where a page's token axis sits among `shape`'s axes: a page of this tensor has `shape` with
+                `page_tokens` put in at that place.  (kv_heads, head_dim) with token_axis 1 gives pages
+                [kv_heads, page_tokens, head_dim] (keys: a token's dims lie together); token_axis 2 gives
+                [kv_heads, head_dim, page_tokens] (values stored transposed within the page).
+    """
+    name: str
+    shape: Tuple[int, ...]
+    dtype: Optional[str] = None
+    token_axis: int = 0
+
+    def page_shape(self, page_tokens: int) -> Tuple[int, ...]:
+        if not 0 <= self.token_axis <= len(self.shape):
+            raise ValueError(f"cache tensor {self.name}: token_axis {self.token_axis} outside its {len(self.shape)} axes")
+        return tuple(self.shape[:self.token_axis]) + (int(page_tokens),) + tuple(self.shape[self.token_axis:])
+
+
+@dataclass(frozen=True)
+class PagedNeed:
+    """A mixer that keeps tensors of every position (window None) or of the last `window` positions, in pages.  The
+    engine allocates what is listed (one arena a tensor and cache group) and knows nothing else of it; mixers with equal
+    needs share a cache group: one page pool and one block table a request."""
+    tensors: Tuple[CacheTensor, ...]
     window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a paged cache need lists at least one tensor and no name twice, not {names}")
+
+
+def KVNeed(kv_heads: int, head_dim: int, window: Optional[int] = None) -> PagedNeed:
+    """The need of softmax attention: keys [kv_heads, token, head_dim] and values [kv_heads, head_dim, token] (transposed
+    within the page) in the activation type."""
+    return PagedNeed((CacheTensor("k", (int(kv_heads), int(head_dim)), None, 1), CacheTensor("v", (int(kv_heads), int(head_dim)), None, 2)), window)
 
 
 @dataclass(frozen=True)

@@ -19,7 +19,7 @@ from typing import Dict, Iterable, List, Tuple
 import torch
 
 from ..parts.spec import TensorSpec
-from .safetensors_io import SafetensorsError, SafetensorsFile
+from .safetensors_io import SafetensorsError, SafetensorsFile, parse_json_unique
 
 
 class WeightsError(ValueError):
@@ -41,9 +41,19 @@ class ModelFiles:
         index = folder / "model.safetensors.index.json"
         single = folder / "model.safetensors"
         if index.exists():
-            weight_map = json.loads(index.read_text()).get("weight_map")
+            try:
+                root = parse_json_unique(index.read_text(), f"safetensors index {index}")
+            except json.JSONDecodeError as e:
+                raise WeightsError(f"weights: {index} is not JSON: {e}") from None
+            weight_map = root.get("weight_map") if isinstance(root, dict) else None
             if not isinstance(weight_map, dict):
-                raise WeightsError(f"weights: {index} has no weight_map")
+                raise WeightsError(f"weights: {index} has no weight_map object")
+            for tensor, file_name in weight_map.items():
+                if not isinstance(file_name, str):
+                    raise WeightsError(f"weights: {index}: the weight_map value of {tensor} is not a file name")
+                # a file named by an index sits beside it (/root/reference/src/format/safetensors.hpp:134-137)
+                if file_name in ("", ".", "..") or any(c in file_name for c in "/\\:"):
+                    raise WeightsError(f"weights: {index} names a file outside its directory: {file_name}")
             names = sorted(set(weight_map.values()))
             self.files = [SafetensorsFile(folder / n) for n in names]
             held = {t for f in self.files for t in f.names()}
@@ -83,6 +93,9 @@ _INTS = (torch.int32, torch.int64)
 
 
 def device_dtype(spec: TensorSpec, stored: torch.dtype, exact: bool) -> torch.dtype:
+    """The type a tensor has on the device: what its spec states, else what its role says."""
+    if spec.dtype is not None:
+        return getattr(torch, spec.dtype)
     if spec.role == "int":
         return torch.int32
     if spec.role in ("norm", "bias", "router") or exact:
@@ -90,8 +103,13 @@ def device_dtype(spec: TensorSpec, stored: torch.dtype, exact: bool) -> torch.dt
     return torch.bfloat16 if stored == torch.bfloat16 else torch.float32
 
 
-def check(specs: List[TensorSpec], held: Dict[str, Tuple[torch.dtype, Tuple[int, ...]]]) -> None:
-    """Raises one WeightsError naming every tensor that is missing, unexpected, of a wrong shape or of a wrong type."""
+def _wants_ints(spec: TensorSpec) -> bool:
+    return spec.dtype == "int32" if spec.dtype is not None else spec.role == "int"
+
+
+def check(specs: List[TensorSpec], held: Dict[str, Tuple[torch.dtype, Tuple[int, ...]]], exact: bool = False) -> None:
+    """Raises one WeightsError naming every tensor that is missing, unexpected, of a wrong shape or of a wrong type,
+    and every fused target whose slices (`TensorSpec.into`) would arrive in different device types."""
     wanted = {s.name: s for s in specs}
     if len(wanted) != len(specs):
         seen, twice = set(), []
@@ -109,9 +127,15 @@ def check(specs: List[TensorSpec], held: Dict[str, Tuple[torch.dtype, Tuple[int,
         dtype, shape = held[n]
         if tuple(shape) != tuple(s.shape):
             wrong_shape.append((n, tuple(shape), tuple(s.shape)))
-        if dtype not in (_INTS if s.role == "int" else _FLOATS):
+        if dtype not in (_INTS if _wants_ints(s) else _FLOATS):
             wrong_type.append((n, str(dtype)))
-    if missing or unexpected or wrong_shape or wrong_type:
+    # the slices of one fused tensor must agree in their device type: found here, before anything is allocated
+    fused: Dict[str, Dict[str, List[str]]] = {}
+    for n, s in wanted.items():
+        if s.into is not None and n in held:
+            fused.setdefault(s.into[0], {}).setdefault(str(device_dtype(s, held[n][0], exact)), []).append(n)
+    mixed = {target: kinds for target, kinds in fused.items() if len(kinds) > 1}
+    if missing or unexpected or wrong_shape or wrong_type or mixed:
         lines = ["weights: the file's tensors are not the model's"]
         if missing:
             lines.append(f"  missing ({len(missing)}): " + ", ".join(missing))
@@ -121,11 +145,15 @@ def check(specs: List[TensorSpec], held: Dict[str, Tuple[torch.dtype, Tuple[int,
             lines.append(f"  wrong shape: {n} is {list(got)}, expected {list(want)}")
         for n, t in wrong_type:
             lines.append(f"  wrong type: {n} is stored as {t}")
+        for target, kinds in sorted(mixed.items()):
+            lines.append(f"  mixed types: the parts of {target} are stored in different types: "
+                         + "; ".join(f"{len(names)} as {kind} (first: {sorted(names)[0]})" for kind, names in sorted(kinds.items())))
+            wrong_type.extend((n, kind) for kind, names in kinds.items() for n in names)
         raise WeightsError("\n".join(lines), missing, unexpected, wrong_shape, wrong_type)
 
 
 def load(specs: List[TensorSpec], files: ModelFiles, device: torch.device, exact: bool) -> Dict[str, torch.Tensor]:
-    check(specs, {n: (files.entry(n).dtype, files.entry(n).shape) for n in files.names()})
+    check(specs, {n: (files.entry(n).dtype, files.entry(n).shape) for n in files.names()}, exact)
     out: Dict[str, torch.Tensor] = {}
     for s in specs:
         host = files.tensor(s.name)
@@ -136,7 +164,5 @@ def load(specs: List[TensorSpec], files: ModelFiles, device: torch.device, exact
         target, shape, index = s.into
         if target not in out:
             out[target] = torch.empty(shape, dtype=dtype, device=device)
-        elif out[target].dtype != dtype:
-            raise WeightsError(f"weights: {s.name} is stored as {host.dtype}, other parts of {target} in another type")
         out[target][index].copy_(host.to(dtype))
     return out

@@ -46,7 +46,14 @@ def tensor_key(seed: int, name: str) -> int:
 
 
 def distribution(spec: TensorSpec, init: RandomInit):
-    """(kind, a, b): kind 0 = a + b * normal, kind 1 = uniform in [a, b)."""
+    """(kind, a, b): kind 0 = a + b * normal, kind 1 = uniform in [a, b).  What the spec states, else what its role says."""
+    if spec.init is not None:
+        kind = spec.init[0]
+        if kind == "normal":
+            return 0, float(spec.init[1]), float(spec.init[2])
+        if kind == "uniform":
+            return 1, float(spec.init[1]), float(spec.init[2])
+        return 0, float(spec.init[1]), 0.0       # constant
     if spec.role == "norm":
         return 0, 1.0, init.norm_std
     if spec.role == "bias":
@@ -90,6 +97,9 @@ def host_values(spec: TensorSpec, init: RandomInit) -> torch.Tensor:
 
 
 def stored_dtype(spec: TensorSpec, init: RandomInit) -> torch.dtype:
+    """How a written folder stores the tensor: a stated type as it is, matrices and tables as the run asks."""
+    if spec.dtype is not None:
+        return getattr(torch, spec.dtype)
     if spec.role in ("matrix", "table"):
         return torch.bfloat16 if init.storage == "bfloat16" else torch.float32
     return torch.float32

@@ -3,9 +3,10 @@
 The container: an 8-byte little-endian header length, a JSON header whose
 entries hold exactly `dtype`, `shape` and `data_offsets`, then the data area.
 The reader keeps the reference's rules (/root/reference/src/format/safetensors.hpp:
-dtype map :52-64, entry rules :66-86, file rules :119-130): offsets span the
-shape, tensors tile the data area without gap or overlap and end at the file's
-end.  Tensors are returned as torch views over a memory map, so a large file
+dtype map :52-64, entry rules :66-86, file rules :107-130): no key twice in the
+header or in an entry, `__metadata__` an object of strings, offsets span the
+shape, tensors tile the data area without gap or overlap, each at a file offset
+aligned to its element (at most to 4 bytes), and end at the file's end.  Tensors are returned as torch views over a memory map, so a large file
 is never read whole.
 """
 
@@ -36,6 +37,19 @@ class SafetensorsError(ValueError):
     pass
 
 
+def parse_json_unique(text: str, what: str):
+    """json.loads that refuses an object that holds a key twice (the standard parser silently keeps the last one;
+    the reference refuses: /root/reference/src/format/safetensors.hpp:40-44,109)."""
+    def pairs(items):
+        seen = {}
+        for k, v in items:
+            if k in seen:
+                raise SafetensorsError(f"{what} repeats key {k}")
+            seen[k] = v
+        return seen
+    return json.loads(text, object_pairs_hook=pairs)
+
+
 @dataclass(frozen=True)
 class TensorEntry:
     name: str
@@ -61,12 +75,17 @@ class SafetensorsFile:
         if n > MAX_HEADER_BYTES or 8 + n > size:
             raise SafetensorsError(f"safetensors: {self.path} declares a header of {n} bytes, beyond the file or the limit")
         try:
-            header = json.loads(self._file.read(n).decode("utf-8"))
+            header = parse_json_unique(self._file.read(n).decode("utf-8"), f"safetensors header of {self.path}")
         except (UnicodeDecodeError, json.JSONDecodeError) as e:
             raise SafetensorsError(f"safetensors: {self.path} header is not JSON: {e}") from None
         if not isinstance(header, dict):
             raise SafetensorsError(f"safetensors: {self.path} header is not an object")
         self.metadata = header.pop("__metadata__", {})
+        if not isinstance(self.metadata, dict):
+            raise SafetensorsError(f"safetensors: __metadata__ of {self.path} is not an object")
+        for k, v in self.metadata.items():
+            if not isinstance(v, str):
+                raise SafetensorsError(f"safetensors: __metadata__ value of {k} in {self.path} is not a string")
         self.data_start = 8 + n
         data_bytes = size - self.data_start
         self.entries: Dict[str, TensorEntry] = {}
@@ -92,6 +111,9 @@ class SafetensorsFile:
         for e in sorted(self.entries.values(), key=lambda t: (t.begin, t.end)):
             if e.begin != at:
                 raise SafetensorsError(f"safetensors: {self.path} has a gap or an overlap before tensor {e.name}")
+            align = min(4, DTYPES[NAMES[e.dtype]][1])
+            if (self.data_start + e.begin) % align:
+                raise SafetensorsError(f"safetensors tensor {e.name} is not at a {align}-byte-aligned file offset in {self.path}")
             at = e.end
         if at != data_bytes:
             raise SafetensorsError(f"safetensors: {self.path} does not end where its last tensor ends")
@@ -125,12 +147,14 @@ class SafetensorsFile:
 
 
 def write_safetensors(path: str | Path, tensors: Mapping[str, torch.Tensor], metadata: Mapping[str, str] | None = None) -> None:
-    """Writes CPU tensors in the order given, each contiguous, data area aligned to 8 bytes."""
+    """Writes CPU tensors, each contiguous, the data area aligned to 8 bytes; wider elements first (in the order given
+    among equals), so that every tensor lies at an offset aligned to its element."""
     header = {}
     if metadata:
         header["__metadata__"] = dict(metadata)
     at = 0
-    for name, t in tensors.items():
+    ordered = sorted(tensors.items(), key=lambda item: -item[1].element_size())
+    for name, t in ordered:
         if t.dtype not in NAMES:
             raise SafetensorsError(f"safetensors: tensor {name} has dtype {t.dtype}, which the writer does not write")
         nbytes = t.numel() * t.element_size()
@@ -141,7 +165,7 @@ def write_safetensors(path: str | Path, tensors: Mapping[str, torch.Tensor], met
     with open(path, "wb") as f:
         f.write(struct.pack("<Q", len(blob)))
         f.write(blob)
-        for name, t in tensors.items():
+        for name, t in ordered:
             t = t.detach().cpu().contiguous()
             if t.numel():
                 f.write(t.view(torch.uint8).numpy().tobytes() if t.dim() else t.reshape(1).view(torch.uint8).numpy().tobytes())

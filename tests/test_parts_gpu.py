@@ -37,9 +37,9 @@ def make_step(dtype, entries, tables=(), page_tokens=4):
     return step
 
 
-def ctx(dtype, max_positions=256):
+def ctx(dtype, max_positions=256, page_tokens=None):
     from llmx_amd.parts import BuildContext
-    return BuildContext(dtype, DEV, max_positions)
+    return BuildContext(dtype, DEV, max_positions, page_tokens)
 
 
 def rnd(*shape, scale=1.0, seed=0):
@@ -113,8 +113,8 @@ def test_attention_part(dtype, page, heads, kv_heads, D, R, qk_norm):
         w[s.name] = t.to(torch.float32 if s.role == "norm" else dtype)
     att.load({k: v.to(DEV) for k, v in w.items()})
     n_pages = 16
-    cache = LayerCache(group=0, k=torch.zeros(n_pages, kv_heads, page, D, dtype=dtype, device=DEV),
-                       v=torch.zeros(n_pages, kv_heads, D, page, dtype=dtype, device=DEV), writes=True)
+    cache = LayerCache(group=0, tensors={"k": torch.zeros(n_pages, kv_heads, page, D, dtype=dtype, device=DEV),
+                                         "v": torch.zeros(n_pages, kv_heads, D, page, dtype=dtype, device=DEV)}, writes=True)
     h1, h2 = rnd(L1, E, seed=5), rnd(L2, E, seed=6)
     pages1 = list(range(3, 3 + -(-L1 // page)))[::-1]           # out of order on purpose
     pages2 = [0, 1, 2][: -(-L2 // page)]
@@ -236,8 +236,8 @@ def test_a_position_encoding_defined_here_serves_the_attention_part(dtype):
         att = build_part("mixer", PartSpec("attention", params, "a."), ctx(dtype))
         w = {s.name: rnd(*s.shape, scale=0.3, seed=i).to(dtype) for i, s in enumerate(att.tensor_specs(set()))}
         att.load({k: v.to(DEV) for k, v in w.items()})
-        cache = LayerCache(group=0, k=torch.zeros(8, kv_heads, page, D, dtype=dtype, device=DEV),
-                           v=torch.zeros(8, kv_heads, D, page, dtype=dtype, device=DEV), writes=True)
+        cache = LayerCache(group=0, tensors={"k": torch.zeros(8, kv_heads, page, D, dtype=dtype, device=DEV),
+                                             "v": torch.zeros(8, kv_heads, D, page, dtype=dtype, device=DEV)}, writes=True)
         h = rnd(L, E, seed=11).to(dtype)
         step = make_step(dtype, [(0, L, 0)], [[[7, 6, 5, 4, 3, 2, 1, 0]]], page)
         out = torch.zeros(L, E, dtype=torch.float32, device=DEV)
@@ -445,7 +445,7 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         assert json.loads((folder / "config.json").read_text())["architectures"] == ["ToyHybridForCausalLM"]
         engine = Engine.load(folder, dtype="float32", kv_tokens=64, page_tokens=4, max_requests=3)
         needs = engine.model.cache_needs()
-        assert [type(n).__name__ for n in needs] == ["KVNeed", "StateNeed", "KVNeed", "StateNeed"]
+        assert [type(n).__name__ for n in needs] == ["PagedNeed", "StateNeed", "PagedNeed", "StateNeed"]
         assert not engine.graphs, "a part that does not say graph_safe must keep the engine from recording graphs"
         weights, _ = {}, None
         from safetensors import safe_open
@@ -671,7 +671,7 @@ def test_run_order_names_a_layer_twice_and_shares_a_cache():
     files = ModelFiles(model_folder("A"))
     engine = Engine(cfg, spec, "float32", kv_tokens=128, page_tokens=4, max_requests=2,
                     weights=lambda e: load_weights(e.model.tensor_specs(set(files.names())), files, e.device, True))
-    assert len(engine._layer_caches) == 4 and engine._kv[0].shape[0] == 3
+    assert len(engine._layer_caches) == 4 and engine._paged[0]["k"].shape[0] == 3
     tokens = [5, 17, 3, 200, 41, 7, 99, 1, 2, 3, 4]
     engine.add_request("w")
     whole = engine.step([StepEntry("w", tokens, list(range(len(tokens))))]).clone()
@@ -710,6 +710,191 @@ def test_run_order_names_a_layer_twice_and_shares_a_cache():
     x = layer(x, 0, shared=(k0, v0))
     want = pm.rms_norm(x, w["model.norm.weight"].double(), config["rms_norm_eps"]) @ w["lm_head.weight"].double().T
     assert (whole.cpu().double() - want).abs().max() < 2e-5 * want.abs().max()
+
+
+# ---------------------------------------------------------------------------
+# A mixer whose cache is not keys and values: one float32 latent a token, in pages of its own group, and a parameter of
+# a kind no role knows (a gain drawn uniformly from [0.5, 1.5), kept in float32 in both paths).
+def define_latent_mixer():
+    from llmx_amd.parts import CacheTensor, Mixer, PagedNeed, TensorSpec, register
+
+    class LatentMixer(Mixer):
+        """c_t = h_t Wc^T (a latent of `latent` values, cached); out_t = gain * ((sum_s<=t softmax_s(c_t . c_s / sqrt(latent)) c_s) Wo^T)."""
+        wants_f32_input = True
+
+        def __init__(self, params, prefix, ctx):
+            super().__init__(params, prefix, ctx)
+            self.hidden, self.latent = params["hidden"], params["latent"]
+            self.page = ctx.page_tokens
+            self.wc = self.wo = self.gain = None
+
+        def cache_need(self):
+            return PagedNeed((CacheTensor("latent", (self.latent,), "float32", 0),))
+
+        def tensor_specs(self, available):
+            return [TensorSpec(self.name("down.weight"), (self.latent, self.hidden), "router"),
+                    TensorSpec(self.name("up.weight"), (self.hidden, self.latent), "router"),
+                    TensorSpec(self.name("gain"), (self.hidden,), "matrix", dtype="float32", init=("uniform", 0.5, 1.5))]
+
+        def load(self, tensors):
+            self.wc, self.wo, self.gain = (tensors[self.name(n)] for n in ("down.weight", "up.weight", "gain"))
+
+        def forward(self, step, h, out, accumulate, cache, h32=None):
+            # once a step, for every layer of this kind: each row's page and place in it, from the group's block tables
+            def places():
+                tables = step.tables(cache.group).cpu()
+                page, slot = [], []
+                for i, e in enumerate(step.entries):
+                    for pos in range(e.past, e.past + e.n):
+                        page.append(int(tables[i, pos // self.page]))
+                        slot.append(pos % self.page)
+                return torch.tensor(page, device=step.device), torch.tensor(slot, device=step.device), tables
+            page, slot, tables = step.shared(("latent.places", cache.group), places)
+            store = cache.tensors["latent"]                    # [pages, page_tokens, latent] float32
+            assert store.dtype == torch.float32 and tuple(store.shape[1:]) == (self.page, self.latent)
+            c = h32 @ self.wc.T
+            if cache.writes:
+                store[page, slot] = c
+            result = torch.empty((step.rows, self.hidden), dtype=torch.float32, device=step.device)
+            for i, e in enumerate(step.entries):
+                n_ctx = e.past + e.n
+                pages = tables[i, :-(-n_ctx // self.page)].to(step.device)
+                ctx_latents = store[pages].reshape(-1, self.latent)[:n_ctx]
+                scores = (c[e.row0:e.row0 + e.n] @ ctx_latents.T) / self.latent ** 0.5
+                causal = torch.arange(n_ctx, device=step.device)[None, :] <= torch.arange(e.past, n_ctx, device=step.device)[:, None]
+                weights = torch.softmax(scores.masked_fill(~causal, float("-inf")), dim=-1)
+                result[e.row0:e.row0 + e.n] = ((weights @ ctx_latents) @ self.wo.T) * self.gain
+            if accumulate:
+                out += result
+            else:
+                out.copy_(result)
+
+    register("mixer", "toy_latent", LatentMixer, replace=True)
+
+
+@dataclass(frozen=True)
+class LatentConfig:
+    vocab_size: int = 40
+    hidden_size: int = 32
+    latent: int = 6
+    layers: int = 4
+    architecture = "ToyLatentForCausalLM"
+
+    @classmethod
+    def from_json(cls, values):
+        return cls(**{k: v for k, v in values.items() if k != "architectures"})
+
+    def to_json(self):
+        return {"architectures": [self.architecture], "vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "latent": self.latent,
+                "layers": self.layers}
+
+
+def latent_assemble(c: LatentConfig):
+    from llmx_amd.parts import BlockSpec, ModelSpec, PartSpec, RunEntry
+    E = c.hidden_size
+    blocks = []
+    for i in range(c.layers):
+        p = f"layers.{i}."
+        norm = {"width": E, "eps": 1e-5}
+        if i % 2 == 0:
+            mixer = PartSpec("toy_latent", {"hidden": E, "latent": c.latent}, p + "latent.")
+        else:
+            mixer = PartSpec("attention", {"hidden": E, "heads": 4, "kv_heads": 2, "head_dim": 8, "qk_norm": "none"}, p + "attn.")
+        blocks.append(BlockSpec(PartSpec("rmsnorm", norm, p + "n1."), mixer, PartSpec("rmsnorm", norm, p + "n2."),
+                                PartSpec("dense_glu", {"hidden": E, "intermediate": 24}, p + "mlp.")))
+    return ModelSpec(architecture=c.architecture, vocab_size=c.vocab_size, hidden_size=E, max_positions=128,
+                     embedding=PartSpec("token_embedding", {"vocab": c.vocab_size, "hidden": E}, "embed."), blocks=blocks,
+                     run_order=[RunEntry(i, i) for i in range(c.layers)], final_norm=PartSpec("rmsnorm", {"width": E, "eps": 1e-5}, "norm."),
+                     head=PartSpec("linear", {"vocab": c.vocab_size, "hidden": E, "tied": True}, "head."))
+
+
+def latent_plain(weights, c: LatentConfig, tokens):
+    x = weights["embed.weight"].double()[tokens]
+    T = len(tokens)
+    for i in range(c.layers):
+        p = f"layers.{i}."
+        h = pm.rms_norm(x, weights[p + "n1.weight"].double(), 1e-5)
+        if i % 2 == 0:
+            lat = h @ weights[p + "latent.down.weight"].double().T
+            scores = (lat @ lat.T) / c.latent ** 0.5
+            scores = scores.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float("-inf"))
+            x = x + ((torch.softmax(scores, dim=-1) @ lat) @ weights[p + "latent.up.weight"].double().T) * weights[p + "latent.gain"].double()
+        else:
+            q = (h @ weights[p + "attn.q_proj.weight"].double().T).view(T, 4, 8)
+            k = (h @ weights[p + "attn.k_proj.weight"].double().T).view(T, 2, 8)
+            v = (h @ weights[p + "attn.v_proj.weight"].double().T).view(T, 2, 8)
+            x = x + pm.causal_attention(q, k, v).reshape(T, 32) @ weights[p + "attn.o_proj.weight"].double().T
+        h = pm.rms_norm(x, weights[p + "n2.weight"].double(), 1e-5)
+        gate_up = torch.cat([weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.up_proj.weight"]]).double()
+        x = x + pm.swiglu_expert(h, gate_up, weights[p + "mlp.down_proj.weight"].double())
+    return pm.rms_norm(x, weights["norm.weight"].double(), 1e-5) @ weights["embed.weight"].double().T
+
+
+def test_a_mixer_that_caches_one_latent_a_token_and_brings_a_parameter_of_its_own_kind(tmp_path):
+    """The engine allocates what a mixer's need lists (here one float32 latent a token, where attention lists keys and
+    values of the activation type), the loader and the random-weights mode follow what a tensor's spec states (a gain
+    kept in float32, drawn uniformly from [0.5, 1.5)), and `step.shared` gives a part what it wants once a step: no file
+    under llmx_amd changes for any of it."""
+    from safetensors import safe_open
+    from llmx_amd import Engine, RandomInit
+    from llmx_amd.engine import StepEntry
+    from llmx_amd.models import register_architecture, unregister_architecture
+    from llmx_amd.parts import unregister
+    from llmx_amd.weights.folder import write_random_model
+    define_latent_mixer()
+    register_architecture("ToyLatentForCausalLM", LatentConfig, latent_assemble, replace=True)
+    try:
+        c = LatentConfig()
+        folder = write_random_model(tmp_path / "latent", c, RandomInit(seed=9, std=0.2, norm_std=0.05, storage="bfloat16"))
+        with safe_open(str(folder / "model.safetensors"), framework="pt") as f:
+            weights = {n: f.get_tensor(n) for n in f.keys()}
+        gain = weights["layers.0.latent.gain"]
+        assert gain.dtype == torch.float32 and float(gain.min()) >= 0.5 and float(gain.max()) < 1.5 and float(gain.std()) > 0.2
+        assert weights["layers.1.attn.q_proj.weight"].dtype == torch.bfloat16       # the run's storage rule, where no spec states a type
+        seqs = {"a": [3, 14, 15, 9, 2, 6, 5, 35, 8, 9, 7, 9, 3, 2, 38, 4, 6, 1, 0, 22, 31], "b": [2, 7, 18, 28, 18, 2, 8, 4, 5, 9, 0, 12]}
+        want = {r: latent_plain(weights, c, t) for r, t in seqs.items()}
+        for dtype, tol in (("float32", 2e-5), ("bfloat16", 3e-2)):
+            engine = Engine.load(folder, dtype=dtype, kv_tokens=64, page_tokens=4, max_requests=2)
+            needs = engine.model.cache_needs()
+            assert [len(n.tensors) for n in needs] == [1, 2, 1, 2] and len(engine.cache.groups) == 2
+            assert engine._paged[0]["latent"].dtype == torch.float32 and tuple(engine._paged[0]["latent"].shape) == (2, 16, 4, c.latent)
+            assert engine._paged[1]["k"].dtype == engine.act_dtype and tuple(engine._paged[1]["v"].shape) == (2, 16, 2, 8, 4)
+            assert engine.model.blocks[0].mixer.gain.dtype == torch.float32
+            every = lambda t: list(range(len(t)))
+            whole = {}
+            for r, t in seqs.items():
+                engine.add_request(r)
+                whole[r] = engine.step([StepEntry(r, t, every(t))]).clone()
+                engine.end_request(r)
+                assert (whole[r].cpu().double() - want[r]).abs().max() < tol * want[r].abs().max(), (dtype, r)
+            # portions of one beside single tokens of the other, over page edges, pages of ended requests used again
+            engine.add_request("a")
+            engine.add_request("b")
+            at, rows = {"a": 0, "b": 0}, {"a": [], "b": []}
+            for na, nb in [(5, 1), (2, 1), (1, 3), (6, 1), (3, 2), (2, 4), (2, 0)]:
+                entries = []
+                for r, n in (("a", na), ("b", nb)):
+                    n = min(n, len(seqs[r]) - at[r])
+                    if n:
+                        entries.append(StepEntry(r, seqs[r][at[r]:at[r] + n], list(range(n))))
+                out = engine.step(entries)
+                i = 0
+                for e in entries:
+                    rows[e.request].append(out[i:i + len(e.tokens)].clone())
+                    i += len(e.tokens)
+                    at[e.request] += len(e.tokens)
+            for r in seqs:
+                assert at[r] == len(seqs[r])
+                got = torch.cat(rows[r])
+                assert (got.cpu().double() - want[r]).abs().max() < tol * want[r].abs().max()
+                if dtype == "float32":
+                    assert (got - whole[r]).abs().max() < 1e-5 * whole[r].abs().max()
+            engine.end_request("a")
+            engine.end_request("b")
+            assert engine.cache.pages_in_use(0) == 0 and engine.cache.pages_in_use(1) == 0
+    finally:
+        unregister_architecture("ToyLatentForCausalLM")
+        unregister("mixer", "toy_latent")
 
 
 @pytest.mark.parametrize("dtype,page", [("float32", 4), ("bfloat16", 16)])
@@ -763,7 +948,7 @@ def test_window_attention_gives_pages_back(dtype, page):
                    weights=lambda e: load_weights(e.model.tensor_specs(set(files.names())), files, e.device, exact))
     pools = [g.n_pages for g in small.cache.groups]
     assert pools[0] == 160 // page and pools[1] == 2 * (-(-(W + 12) // page) + 1) < pools[0]
-    assert small._kv[1].shape[2] == pools[1]
+    assert small._paged[1]["k"].shape[1] == pools[1]
     small.add_request("q")
     small.add_request("other")
     cut = []

@@ -28,8 +28,12 @@ def test_written_file_reads_back(tmp_path):
         assert torch.equal(g.get_tensor("b"), tensors["b"])
 
 
-def raw_file(path, header: dict, data: bytes):
-    blob = json.dumps(header).encode()
+def raw_file(path, header, data: bytes, pad_to: int = 8):
+    """A file with this header (a dict, or JSON text as it stands) padded with spaces so that the data area begins at
+    a multiple of `pad_to` bytes."""
+    blob = header.encode() if isinstance(header, str) else json.dumps(header).encode()
+    while (8 + len(blob)) % pad_to:
+        blob += b" "
     path.write_bytes(struct.pack("<Q", len(blob)) + blob + data)
 
 
@@ -47,6 +51,64 @@ def test_reader_refusals(tmp_path, header, data, text):
     raw_file(tmp_path / "bad.safetensors", header, data)
     with pytest.raises(SafetensorsError, match=text):
         SafetensorsFile(tmp_path / "bad.safetensors")
+
+
+def test_a_key_twice_in_the_header_is_refused(tmp_path):
+    """The standard JSON parser would silently keep the last of two equal keys
+    (/root/reference/src/format/safetensors.hpp:40-44,69,109 refuse them)."""
+    entry = '{"dtype": "F32", "shape": [2], "data_offsets": [0, 8]}'
+    raw_file(tmp_path / "twice.safetensors", '{"t": %s, "t": %s}' % (entry, entry), b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="header of .*twice.safetensors repeats key t"):
+        SafetensorsFile(tmp_path / "twice.safetensors")
+    raw_file(tmp_path / "inner.safetensors", '{"t": {"dtype": "F32", "dtype": "F32", "shape": [2], "data_offsets": [0, 8]}}', b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="repeats key dtype"):
+        SafetensorsFile(tmp_path / "inner.safetensors")
+
+
+def test_metadata_must_be_an_object_of_strings(tmp_path):
+    entry = {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]}
+    raw_file(tmp_path / "m1.safetensors", {"__metadata__": {"format": "pt", "step": 3}, "t": entry}, b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="__metadata__ value of step .* is not a string"):
+        SafetensorsFile(tmp_path / "m1.safetensors")
+    raw_file(tmp_path / "m2.safetensors", {"__metadata__": ["pt"], "t": entry}, b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="__metadata__ of .* is not an object"):
+        SafetensorsFile(tmp_path / "m2.safetensors")
+
+
+def test_a_tensor_at_an_unaligned_file_offset_is_refused(tmp_path):
+    """Elements must lie at multiples of their size (of 4 bytes at most) in the file, so that the map can be read in place
+    (/root/reference/src/format/safetensors.hpp:123-126)."""
+    # a bfloat16 tensor of 3 elements pushes the float32 tensor behind it to an offset of 6
+    header = {"h": {"dtype": "BF16", "shape": [3], "data_offsets": [0, 6]}, "f": {"dtype": "F32", "shape": [2], "data_offsets": [6, 14]}}
+    raw_file(tmp_path / "odd.safetensors", header, b"\0" * 14)
+    with pytest.raises(SafetensorsError, match="tensor f is not at a 4-byte-aligned file offset"):
+        SafetensorsFile(tmp_path / "odd.safetensors")
+    # the same tensors with the data area one byte off: the bfloat16 tensor is the first to be refused
+    raw_file(tmp_path / "off.safetensors", {"h": {"dtype": "BF16", "shape": [3], "data_offsets": [0, 6]}}, b"\0" * 6, pad_to=1)
+    if (8 + len(json.dumps({"h": {"dtype": "BF16", "shape": [3], "data_offsets": [0, 6]}}))) % 2:
+        with pytest.raises(SafetensorsError, match="tensor h is not at a 2-byte-aligned file offset"):
+            SafetensorsFile(tmp_path / "off.safetensors")
+    # the writer orders wider elements first, so what it writes is always aligned
+    write_safetensors(tmp_path / "ok.safetensors", {"h": torch.zeros(3, dtype=torch.bfloat16), "f": torch.ones(2), "i": torch.zeros(1, dtype=torch.int64)})
+    f = SafetensorsFile(tmp_path / "ok.safetensors")
+    assert f.entries["i"].begin == 0 and f.entries["f"].begin == 8 and f.entries["h"].begin == 16 and torch.equal(f.tensor("f"), torch.ones(2))
+
+
+def test_an_index_that_names_a_file_outside_its_folder_is_refused(tmp_path):
+    """/root/reference/src/format/safetensors.hpp:134-137: a file named by an index sits beside it."""
+    write_safetensors(tmp_path / "part.safetensors", {"t": torch.zeros(2)})
+    for bad in ("../part.safetensors", "sub/part.safetensors", "..", ""):
+        (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"t": bad}}))
+        with pytest.raises(WeightsError, match="names a file outside its directory"):
+            ModelFiles(tmp_path)
+    (tmp_path / "model.safetensors.index.json").write_text('{"weight_map": {"t": "part.safetensors", "t": "part.safetensors"}}')
+    with pytest.raises(SafetensorsError, match="repeats key t"):
+        ModelFiles(tmp_path)
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"t": 3}}))
+    with pytest.raises(WeightsError, match="weight_map value of t is not a file name"):
+        ModelFiles(tmp_path)
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"t": "part.safetensors"}}))
+    assert list(ModelFiles(tmp_path).names()) == ["t"]
 
 
 def test_header_longer_than_file(tmp_path):
@@ -90,6 +152,40 @@ def test_types_on_the_device():
     assert device_dtype(m, bf, exact=True) == f32          # the 32-bit path widens everything
     assert device_dtype(n, bf, exact=False) == f32 and device_dtype(r, bf, exact=False) == f32
     assert device_dtype(i, torch.int64, exact=False) == torch.int32
+    # a type the spec states holds in both paths, whatever the file stores
+    decay = TensorSpec("d", (4,), "matrix", dtype="float32")
+    assert device_dtype(decay, bf, exact=False) == f32 and device_dtype(TensorSpec("t", (4,), "table", dtype="bfloat16"), f32, exact=True) == bf
+    with pytest.raises(ValueError, match="dtype 'float16' is not one of"):
+        TensorSpec("x", (1,), dtype="float16")
+    with pytest.raises(ValueError, match="role 'gate' is not one of"):
+        TensorSpec("x", (1,), "gate")
+    with pytest.raises(ValueError, match="init .* is not"):
+        TensorSpec("x", (1,), init=("lognormal", 0, 1))
+
+
+def test_a_spec_states_how_random_weights_fill_it():
+    """A parameter of a kind the roles do not know brings its own distribution; the run's RandomInit does not touch it."""
+    from llmx_amd.weights.random_init import distribution, stored_dtype
+    init = RandomInit(seed=3, std=0.02, norm_std=0.1, bias_range=0.5)
+    u = TensorSpec("layer.decay", (4096,), "matrix", dtype="float32", init=("uniform", 0.9, 0.999))
+    assert distribution(u, init) == (1, 0.9, 0.999) and stored_dtype(u, init) == torch.float32
+    v = host_values(u, init)
+    assert v.dtype == torch.float32 and float(v.min()) >= 0.9 and float(v.max()) < 0.999 and float(v.std()) > 0.02
+    n = host_values(TensorSpec("layer.gain", (4096,), "norm", init=("normal", 2.0, 0.25)), init)
+    assert abs(float(n.mean()) - 2.0) < 0.02 and abs(float(n.std()) - 0.25) < 0.02
+    c = host_values(TensorSpec("layer.one", (8,), "bias", init=("constant", -1.5)), init)
+    assert torch.equal(c, torch.full((8,), -1.5))
+    assert distribution(TensorSpec("w", (2, 2)), init) == (0, 0.0, 0.02)          # by role, as before
+
+
+def test_slices_of_one_fused_tensor_in_different_types_are_refused_before_anything_is_allocated():
+    specs = [TensorSpec(f"experts.{e}.down", (4, 4), into=("experts.down", (3, 4, 4), (e,))) for e in range(3)]
+    held = {"experts.0.down": (torch.bfloat16, (4, 4)), "experts.1.down": (torch.float32, (4, 4)), "experts.2.down": (torch.bfloat16, (4, 4))}
+    with pytest.raises(WeightsError, match="mixed types: the parts of experts.down are stored in different types") as err:
+        check(specs, held, exact=False)
+    assert sorted(n for n, _ in err.value.wrong_type) == sorted(held)
+    check(specs, held, exact=True)          # the 32-bit path widens every slice to float32: no mix
+    check(specs, {n: (torch.bfloat16, (4, 4)) for n in held}, exact=False)
 
 
 def test_folder_loads_on_the_cpu_with_every_tensor_consumed_once():
