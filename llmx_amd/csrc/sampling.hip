@@ -602,7 +602,9 @@ __device__ bool ranked_find(int n, KeyFn key, WeightFn weight, unsigned long lon
         passed += sh.found_before;
         const int count = sh.hist_c[fb];
         lo = lo + ((unsigned long long)fb << shift);
-        const unsigned long long bucket_hi = lo + ((1ull << shift) - 1ull);
+        // the bucket's last key; the top bucket of the whole key range ends at the largest key there is (no wrap)
+        const unsigned long long span = (1ull << shift) - 1ull;
+        const unsigned long long bucket_hi = lo > ~0ull - span ? ~0ull : lo + span;
         hi = bucket_hi < hi ? bucket_hi : hi;
         __syncthreads();
         if (count > RANKED_CAP) continue;   // the range has shrunk by at least 1,024 times; go on inside it
@@ -615,6 +617,7 @@ __device__ bool ranked_find(int n, KeyFn key, WeightFn weight, unsigned long lon
             sh.g_q[at] = weight(i);
         }
         __syncthreads();
+        if (sh.gathered != count) return false;   // cannot happen: the range is the bucket that was counted
         for (int r = tid; r < count; r += SAMPLE_THREADS) {
             const unsigned long long mine = sh.g_key[r];
             int better = 0;
@@ -659,7 +662,11 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const flo
     const float tmp = temp[r], p = top_p[r], cut = min_p ? min_p[r] : 0.0f;
     if (!(tmp > 0.0f)) return;   // a greedy row is not this kernel's: its entry of `out` is not written
     const unsigned long long all_lo = 1ull, all_hi = ~0ull;
-    auto key_of = [&](int i) -> unsigned long long { return i == sk ? 0ull : rank_key(s[i], i); };
+    // a NaN score takes no part, like the masked token (the arg-max never lets a NaN lead either)
+    auto key_of = [&](int i) -> unsigned long long {
+        const float v = s[i];
+        return i == sk || v != v ? 0ull : rank_key(v, i);
+    };
 
     // the best token: the largest key
     unsigned long long top = 0;
@@ -668,15 +675,27 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const flo
         top = k > top ? k : top;
     }
     top = block_max_u64(top, sh.wave_q);
+    if (top == 0ull) {   // nothing takes part (every score a NaN): the first id that is not masked, as the arg-max gives
+        if (tid == 0) out[r] = sk == 0 && n > 1 ? 1 : 0;
+        return;
+    }
     const int best = (int)(0xFFFFFFFFu - (uint32_t)top);
     const float best_score = s[best];
     // fixed-point weights: a row's sum stays below 2^62
     int scale_bits = 62;
     while ((1ll << (62 - scale_bits)) < (long long)n) --scale_bits;
     const double scale = (double)(1ull << scale_bits);
-    auto weight_of = [&](int i) -> unsigned long long { return (unsigned long long)((double)expf((s[i] - best_score) / tmp) * scale); };
+    // exp((score - best) / temp); a score equal to an infinite best (inf - inf) weighs 1 like the best itself, and a
+    // NaN (which takes no part anyway) weighs 0, so that no NaN is ever turned into an integer
+    auto rel_weight = [&](int i) -> float {
+        const float v = s[i];
+        if (v != v) return 0.0f;
+        const float d = v - best_score;
+        return d != d ? 1.0f : expf(d / tmp);
+    };
+    auto weight_of = [&](int i) -> unsigned long long { return (unsigned long long)((double)rel_weight(i) * scale); };
     auto cut_weight_of = [&](int i) -> unsigned long long {
-        const float w = expf((s[i] - best_score) / tmp);
+        const float w = rel_weight(i);
         return w < cut ? 0ull : (unsigned long long)((double)w * scale);
     };
 
@@ -716,7 +735,7 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const flo
         auto nucleus_key = [&](int i) -> unsigned long long {
             const unsigned long long k = key_of(i);
             if (k < nucleus_from) return 0ull;
-            return (cut > 0.0f && expf((s[i] - best_score) / tmp) < cut) ? 0ull : k;
+            return (cut > 0.0f && rel_weight(i) < cut) ? 0ull : k;
         };
         mine = 0;
         for (int i = tid; i < n; i += SAMPLE_THREADS)

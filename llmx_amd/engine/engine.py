@@ -124,9 +124,16 @@ class Engine:
             tensors = {}
             for s in eng.model.tensor_specs():
                 dt = device_dtype(s, stored_dtype(s, init), eng.act_dtype == torch.float32)
-                t = torch.empty(s.shape, dtype=dt, device=eng.device)
+                if s.into is None:
+                    t = tensors[s.name] = torch.empty(s.shape, dtype=dt, device=eng.device)
+                else:   # a slice of a fused tensor, filled in place with the values its own name gives
+                    target, shape, index = s.into
+                    if target not in tensors:
+                        tensors[target] = torch.empty(shape, dtype=dt, device=eng.device)
+                    t = tensors[target][index]
+                    if not t.is_contiguous() or tuple(t.shape) != tuple(s.shape):
+                        raise ValueError(f"random weights: {s.name} is not a contiguous slice of {target}")
                 fill_random(t, s, init)
-                tensors[s.name] = t
             if tensors_out is not None:
                 tensors_out.update(tensors)
             return tensors

@@ -59,10 +59,13 @@ class Attention(Mixer):
         return KVNeed(self.kv_heads, self.head_dim, self.window)
 
     def tensor_specs(self, available):
+        # one product for the three projections: the file's q, k and v go straight into the rows q | k | v of one tensor
+        fused, shape = self.name("qkv_proj.weight"), (self.q_width + 2 * self.kv_width, self.hidden)
+        q, kv = self.q_width, self.kv_width
         specs = [
-            TensorSpec(self.name("q_proj.weight"), (self.q_width, self.hidden)),
-            TensorSpec(self.name("k_proj.weight"), (self.kv_width, self.hidden)),
-            TensorSpec(self.name("v_proj.weight"), (self.kv_width, self.hidden)),
+            TensorSpec(self.name("q_proj.weight"), (q, self.hidden), into=(fused, shape, (slice(0, q),))),
+            TensorSpec(self.name("k_proj.weight"), (kv, self.hidden), into=(fused, shape, (slice(q, q + kv),))),
+            TensorSpec(self.name("v_proj.weight"), (kv, self.hidden), into=(fused, shape, (slice(q + kv, q + 2 * kv),))),
             TensorSpec(self.name("o_proj.weight"), (self.hidden, self.q_width)),
         ]
         if self.norm_mode == ops.QKNORM_PROJECTION:
@@ -71,11 +74,7 @@ class Attention(Mixer):
         return specs
 
     def load(self, tensors):
-        q, k, v = (tensors[self.name(n + "_proj.weight")] for n in "qkv")
-        if not (q.dtype == k.dtype == v.dtype):
-            raise ValueError(f"{self.prefix}: q, k and v projections are stored in different types")
-        # one product for the three projections: rows q | k | v
-        self.wqkv = torch.cat([q, k, v], dim=0).contiguous()
+        self.wqkv = tensors[self.name("qkv_proj.weight")]
         self.wo = tensors[self.name("o_proj.weight")]
         if self.norm_mode == ops.QKNORM_PROJECTION:
             self.q_norm = tensors[self.name("q_norm.weight")]

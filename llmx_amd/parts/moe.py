@@ -121,11 +121,13 @@ class DenseGLU(FeedForward):
 
     def tensor_specs(self, available):
         F, E = self.intermediate, self.hidden
-        return [TensorSpec(self.name("gate_proj.weight"), (F, E)), TensorSpec(self.name("up_proj.weight"), (F, E)),
+        fused = self.name("gate_up_proj.weight")     # gate rows, then up rows, filled from the file's two tensors
+        return [TensorSpec(self.name("gate_proj.weight"), (F, E), into=(fused, (2 * F, E), (slice(0, F),))),
+                TensorSpec(self.name("up_proj.weight"), (F, E), into=(fused, (2 * F, E), (slice(F, 2 * F),))),
                 TensorSpec(self.name("down_proj.weight"), (E, F))]
 
     def load(self, tensors):
-        self.w_gate_up = torch.cat([tensors[self.name("gate_proj.weight")], tensors[self.name("up_proj.weight")]], dim=0).contiguous()
+        self.w_gate_up = tensors[self.name("gate_up_proj.weight")]
         self.w_down = tensors[self.name("down_proj.weight")]
 
     def takes_deferred_norm(self, step):

@@ -32,14 +32,14 @@ def main(argv=None) -> int:
     ap.add_argument("--out", required=True, help="folder the logits files are written to")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time, each request's count rounded up to a multiple of 64")
-    ap.add_argument("--page-tokens", type=int, default=16, help="tokens a cache page holds (a divisor or a multiple of 64)")
+    ap.add_argument("--page-tokens", type=int, default=16, help="tokens a cache page holds")
     ap.add_argument("--max-requests", type=int, default=8, help="most requests live at a time")
     ap.add_argument("--routing", action="store_true", help="also write every step's expert picks and router logits")
     args = ap.parse_args(argv)
     if args.max_tokens <= 0:
         ap.error("--max-tokens must be positive")
-    if args.page_tokens <= 0 or (64 % args.page_tokens and args.page_tokens % 64):
-        ap.error("--page-tokens must divide 64 or be a multiple of it")
+    if args.page_tokens <= 0:
+        ap.error("--page-tokens must be positive")
 
     out = Path(args.out)
     out.mkdir(parents=True, exist_ok=True)
@@ -47,9 +47,13 @@ def main(argv=None) -> int:
     import numpy as np
     from llmx_amd.engine import Engine, StepEntry
 
-    # each request's count is rounded up to a multiple of the larger of 64 and the page
+    # --max-tokens counts each request rounded up to a multiple of 64 (to the engine's own page where that is larger).
+    # A request of n tokens holds ceil(n / page) pages, which for pages that do not divide 64 can be one page more than
+    # its rounded count holds; one page a request on top covers that for any page size.
     unit = max(64, args.page_tokens)
     kv_tokens = -(-args.max_tokens // unit) * unit
+    if unit % args.page_tokens:
+        kv_tokens += args.max_requests * args.page_tokens
     engine = Engine.load(args.model, dtype=args.dtype, kv_tokens=kv_tokens, page_tokens=args.page_tokens,
                          max_requests=args.max_requests)
     routed = []      # what the routed layers of the running step showed, in run order

@@ -21,27 +21,39 @@ def weight(score, best, temp):
 
 
 def sample(scores, temp, top_k, top_p, min_p, r, skip=None):
+    return prepare(scores, temp, top_k, top_p, min_p, skip)(r)
+
+
+def prepare(scores, temp, top_k, top_p, min_p, skip=None):
+    """draw(r) for one row and its settings: everything that does not depend on the uniform number r (the ranking, the
+    weights and their sums, the nucleus) is formed once, so that many draws of one row stay affordable."""
     n = len(scores)
     ids = [i for i in range(n) if i != skip]
     m = len(ids)
     ranked = sorted(ids, key=lambda i: (-scores[i], i))
     if temp <= 0.0:
-        return ranked[0]
+        return lambda r: ranked[0]
     keep = top_k if 0 < top_k < m else m
     best = scores[ranked[0]]
     cut = lambda w: 0.0 if w < f32(min_p) else w
+
+    def walk(order, w, total):
+        def draw(r):
+            target = f32(r) * total
+            acc = 0.0
+            for i in order:
+                acc += w[i]
+                if target < acc:
+                    return i
+            return ranked[0]
+        return draw
+
     if keep == m and top_p >= 1.0:
         w = {i: cut(weight(scores[i], best, temp)) for i in ids}
         total = 0.0
         for i in ids:
             total += w[i]
-        target = f32(r) * total
-        acc = 0.0
-        for i in ids:
-            acc += w[i]
-            if target < acc:
-                return i
-        return ranked[0]
+        return walk(ids, w, total)
     kept_ranked = ranked[:keep]
     kept = sorted(kept_ranked)
     w = {i: weight(scores[i], best, temp) for i in kept}
@@ -54,13 +66,7 @@ def sample(scores, temp, top_k, top_p, min_p, r, skip=None):
             for i in kept:
                 w[i] = cut(w[i])
                 total += w[i]
-        target = f32(r) * total
-        acc = 0.0
-        for i in kept:
-            acc += w[i]
-            if target < acc:
-                return i
-        return ranked[0]
+        return walk(kept, w, total)
     goal = f32(top_p) * total
     nucleus_weight, nucleus = 0.0, 0
     while True:
@@ -77,10 +83,4 @@ def sample(scores, temp, top_k, top_p, min_p, r, skip=None):
             nucleus_weight = 0.0
             for i in range(nucleus):
                 nucleus_weight += w[kept_ranked[i]]
-    target = f32(r) * nucleus_weight
-    acc = 0.0
-    for i in range(nucleus):
-        acc += w[kept_ranked[i]]
-        if target < acc:
-            return kept_ranked[i]
-    return ranked[0]
+    return walk(kept_ranked[:nucleus], w, nucleus_weight)

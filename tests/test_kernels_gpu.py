@@ -953,6 +953,73 @@ def test_ranked_sampler_matches_reference_draw_for_draw(V, draws):
     assert out.tolist() == [-5] * rows
 
 
+def test_ranked_sampler_over_the_whole_vocabulary_200_draws():
+    """The search by histograms forms its sums in 64-bit fixed point where the reference sums doubles: 200 draws a row at
+    the real vocabulary (a nucleus over the whole row; a top-k of 5,000; a nucleus with min_p inside a top-k of 50,000),
+    each the reference's token.  The reference's ranking and sums are formed once a row (sampler_reference.prepare)."""
+    o = ops()
+    from llmx_amd.sampling import XorShift64
+    V, draws = 200064, 200
+    settings = [dict(temp=0.8, top_k=0, top_p=0.9, min_p=0.0), dict(temp=1.0, top_k=5000, top_p=1.0, min_p=0.0),
+                dict(temp=1.3, top_k=50000, top_p=0.8, min_p=0.01)]
+    rows = len(settings)
+    logits = rnd(rows, V, scale=2.5, seed=77)
+    host = logits.cpu()
+    refs = [sampler_reference.prepare(host[r].tolist(), s["temp"], s["top_k"], s["top_p"], s["min_p"]) for r, s in enumerate(settings)]
+    f = lambda key: torch.tensor([s[key] for s in settings], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([s["top_k"] for s in settings], dtype=torch.int32, device=DEV)
+    logits = logits.to(DEV)
+    rng = XorShift64(2024)
+    seen = [set() for _ in settings]
+    for draw in range(draws):
+        units = [rng.unit() for _ in range(rows)]
+        out = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        o.sample_ranked(logits, f("temp"), top_k, f("top_p"), f("min_p"), torch.tensor(units, dtype=torch.float32, device=DEV), out)
+        got = out.tolist()
+        for r in range(rows):
+            want = refs[r](units[r])
+            assert got[r] == want, f"draw {draw}, row {r} ({settings[r]}): device {got[r]}, reference {want}"
+            seen[r].add(want)
+    assert all(len(s) > 50 for s in seen), "the draws did not spread over the kept tokens"
+
+
+def test_ranked_sampler_with_scores_that_are_not_finite():
+    """Rows holding NaN, +inf and -inf: a NaN takes no part (as in the arg-max), an infinite best weighs 1 against 0 of
+    every finite score, a row of nothing but NaN gives its first id that is not masked; the pick is always inside the row."""
+    o = ops()
+    V = 5000
+    logits = rnd(6, V, scale=2.0, seed=5)
+    nan, inf = float("nan"), float("inf")
+    logits[0, 17] = nan
+    logits[0, 4000] = nan
+    logits[1, 123] = inf
+    logits[2, 9] = nan
+    logits[2, 77] = inf
+    logits[2, 78] = inf
+    logits[3, :] = nan
+    logits[4, :] = nan
+    logits[5, 5:4990] = -inf
+    logits[5, 3] = nan
+    logits = logits.to(DEV)
+    skip = torch.tensor([-1, -1, -1, -1, 0, -1], dtype=torch.int32, device=DEV)
+    ones = lambda v: torch.full((6,), v, dtype=torch.float32, device=DEV)
+    picks = [set() for _ in range(6)]
+    for top_k_v, top_p_v in ((0, 0.9), (2000, 1.0), (0, 0.999)):
+        top_k = torch.full((6,), top_k_v, dtype=torch.int32, device=DEV)
+        for u in (0.0, 0.31, 0.77, 1.0 - 2.0 ** -24):
+            out = torch.full((6,), -1, dtype=torch.int32, device=DEV)
+            o.sample_ranked(logits, ones(1.0), top_k, ones(top_p_v), ones(0.0), ones(u), out, skip)
+            got = out.tolist()
+            assert all(0 <= g < V for g in got), got
+            for r, g in enumerate(got):
+                picks[r].add(g)
+    assert not picks[0] & {17, 4000} and len(picks[0]) > 1           # NaNs never drawn; the rest of the row is
+    assert picks[1] == {123}                                        # an infinite score takes all the weight
+    assert picks[2] <= {77, 78} and 77 in picks[2]                   # two infinite scores share it; the NaN has none
+    assert picks[3] == {0} and picks[4] == {1}                       # nothing takes part: the first id not masked
+    assert picks[5] <= set(range(5)) | set(range(4990, V)) and 3 not in picks[5]
+
+
 def test_sampler_sends_each_row_to_the_kernel_that_takes_it():
     """One call with greedy rows, rows that keep everything, small top-k sets and rows only the search by histograms
     takes: every row's token is the reference's for that row's settings and generator."""

@@ -42,6 +42,21 @@ def ctx(dtype, max_positions=256, page_tokens=None):
     return BuildContext(dtype, DEV, max_positions, page_tokens)
 
 
+def load_part(part, w):
+    """Hands a part the tensors `w` (by the names it lists) as the loader does: on the device, a tensor that is a slice
+    of a fused one (TensorSpec.into) copied into its place there."""
+    out = {}
+    for s in part.tensor_specs(set(w)):
+        if s.into is None:
+            out[s.name] = w[s.name].to(DEV)
+        else:
+            target, shape, index = s.into
+            if target not in out:
+                out[target] = torch.empty(shape, dtype=w[s.name].dtype, device=DEV)
+            out[target][index].copy_(w[s.name])
+    part.load(out)
+
+
 def rnd(*shape, scale=1.0, seed=0):
     g = torch.Generator().manual_seed(seed + sum(shape))
     return torch.randn(*shape, generator=g) * scale
@@ -106,12 +121,13 @@ def test_attention_part(dtype, page, heads, kv_heads, D, R, qk_norm):
               "position": PartSpec("rotary_neox_partial", {"rotary_dim": R, "theta": 1e4, "head_dim": D})}
     att = build_part("mixer", PartSpec("attention", params, "a."), ctx(dtype))
     need = att.cache_need()
-    assert (need.kv_heads, need.head_dim, need.window) == (kv_heads, D, None)
+    assert need.window is None and [(t.name, t.shape, t.dtype, t.page_shape(page)) for t in need.tensors] == \
+        [("k", (kv_heads, D), None, (kv_heads, page, D)), ("v", (kv_heads, D), None, (kv_heads, D, page))]
     w = {}
     for s in att.tensor_specs(set()):
         t = (1 + 0.1 * rnd(*s.shape, seed=len(w))) if s.role == "norm" else rnd(*s.shape, scale=0.3, seed=len(w))
         w[s.name] = t.to(torch.float32 if s.role == "norm" else dtype)
-    att.load({k: v.to(DEV) for k, v in w.items()})
+    load_part(att, w)
     n_pages = 16
     cache = LayerCache(group=0, tensors={"k": torch.zeros(n_pages, kv_heads, page, D, dtype=dtype, device=DEV),
                                          "v": torch.zeros(n_pages, kv_heads, D, page, dtype=dtype, device=DEV)}, writes=True)
@@ -195,7 +211,7 @@ def test_routed_experts_and_dense_glu_parts(dtype, T):
 
     glu = build_part("feed_forward", PartSpec("dense_glu", {"hidden": E, "intermediate": Fe}, "g."), ctx(dtype))
     gw = {s.name: rnd(*s.shape, scale=0.3, seed=3 + i).to(dtype) for i, s in enumerate(glu.tensor_specs(set()))}
-    glu.load({n: t.to(DEV) for n, t in gw.items()})
+    load_part(glu, gw)
     base = rnd(T, E, seed=4)
     out = base.clone().to(DEV)
     glu.forward(step, h.to(dtype).to(DEV), out, True)
@@ -235,7 +251,7 @@ def test_a_position_encoding_defined_here_serves_the_attention_part(dtype):
                   "position": PartSpec("toy_squeezed_rotary", {"head_dim": D, "theta": 100.0, "factor": 4.0})}
         att = build_part("mixer", PartSpec("attention", params, "a."), ctx(dtype))
         w = {s.name: rnd(*s.shape, scale=0.3, seed=i).to(dtype) for i, s in enumerate(att.tensor_specs(set()))}
-        att.load({k: v.to(DEV) for k, v in w.items()})
+        load_part(att, w)
         cache = LayerCache(group=0, tensors={"k": torch.zeros(8, kv_heads, page, D, dtype=dtype, device=DEV),
                                              "v": torch.zeros(8, kv_heads, D, page, dtype=dtype, device=DEV)}, writes=True)
         h = rnd(L, E, seed=11).to(dtype)

@@ -209,7 +209,7 @@ def test_whole_model_invariants(name):
     x = w["model.embed_tokens.weight"].double()[tokens]
     want = pm.rms_norm(x, w["model.norm.weight"].double(), cfg["rms_norm_eps"]) @ w["lm_head.weight"].double().T
     assert torch.allclose(bare, want, rtol=1e-10)
-    assert torch.allclose(pm.forward(cfg, w0, tokens[::-1])[::-1] if False else pm.forward(cfg, w0, list(reversed(tokens))).flip(0), want, rtol=1e-10)
+    assert torch.allclose(pm.forward(cfg, w0, list(reversed(tokens))).flip(0), want, rtol=1e-10)
 
 
 def test_greedy_and_rounding():

@@ -55,12 +55,17 @@ def test_static_argmax_equals_the_ordinary_entry_point_on_two_calls_in_a_row():
         partial = torch.empty(2 * rows * (-(-n // 8192)), dtype=torch.int32, device=DEV)
         assert h.llmx_argmax_rows(s.data_ptr(), skip_at, want.data_ptr(), partial.data_ptr(), rows, n, _stream()) == 0
         got = torch.full((rows,), -9, dtype=torch.int32, device=DEV)
+        # a warm-up call, so that nothing the first launch of a kernel makes the runtime load or reserve is counted
+        assert h.llmx_argmax_rows_static(s.data_ptr(), skip_at, got.data_ptr(), rows, n, _stream()) == 0, h.llmx_no_alloc_last_error()
+        got.fill_(-9)
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        before = torch.cuda.memory_allocated()           # torch's own allocator
+        free_before = torch.cuda.mem_get_info()[0]        # the device's free bytes: a hipMalloc inside the library would lower them
         rc = h.llmx_argmax_rows_static(s.data_ptr(), skip_at, got.data_ptr(), rows, n, _stream())
         assert rc == 0, h.llmx_no_alloc_last_error()
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == free_before, "the device's free memory changed across the call"
         assert got.tolist() == want.tolist()
         # and both are the arg-max: the first of the tied leaders unless it is skipped, never the NaN
         host = s.cpu()
