@@ -119,9 +119,10 @@ class Engine:
     def from_random(cls, config, init: RandomInit = RandomInit(), dtype="bfloat16", tensors_out: Optional[dict] = None,
                     **options) -> "Engine":
         """An engine whose weights are generated on the device from (seed, tensor name); nothing is read or written.
-        `tensors_out`, when given, receives the device tensors by name as the parts were handed them."""
+        `tensors_out`, when given, receives the device tensors by the names a model folder would hold (a tensor that
+        is a slice of a fused one as a view of it) and the fused tensors by the names the parts read them under."""
         def generate(eng: "Engine"):
-            tensors = {}
+            tensors, by_file_name = {}, {}
             for s in eng.model.tensor_specs():
                 dt = device_dtype(s, stored_dtype(s, init), eng.act_dtype == torch.float32)
                 if s.into is None:
@@ -134,8 +135,10 @@ class Engine:
                     if not t.is_contiguous() or tuple(t.shape) != tuple(s.shape):
                         raise ValueError(f"random weights: {s.name} is not a contiguous slice of {target}")
                 fill_random(t, s, init)
+                by_file_name[s.name] = t
             if tensors_out is not None:
                 tensors_out.update(tensors)
+                tensors_out.update(by_file_name)
             return tensors
 
         return cls(config, registry.assemble(config), dtype, weights=generate, **options)
