@@ -325,91 +325,194 @@ __device__ int block_exclusive_scan(int v, int* scratch, int* total) {
     return before + inc - v;
 }
 
+// What the selection shares between its threads.
+struct TopkShared {
+    int hist[256];
+    int scan_scratch[SAMPLE_WAVES];
+    uint32_t prefix;
+    int remaining;
+};
+
+// The `keep` best of the items c in [0, count) by (score descending, id ascending).  item(c) is the item's id, or -1
+// for an item that takes no part; ids rise with c.  A radix select over the scores' ordered bits finds the keep-th
+// score; items above it are kept, items equal to it lowest id first until `keep` are held.  emit(place, id, score) is
+// called for every kept item, places counting the kept items in item order.  Returns how many were kept (fewer than
+// `keep` when fewer take part).  Every thread of the block calls it with the same arguments.
+template <typename Item, typename Emit>
+__device__ int select_topk(const float* __restrict__ s, int count, Item item, int keep, Emit emit, TopkShared& sh) {
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        sh.prefix = 0;
+        sh.remaining = keep;
+    }
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 24 - 8 * pass;
+        if (tid < 256) sh.hist[tid] = 0;
+        __syncthreads();
+        const uint32_t prefix = sh.prefix;
+        const uint32_t mask = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8));
+        if (pass == 0) {
+            // the top byte (sign and seven exponent bits) takes few values over a row, so a wave's lanes meet in a
+            // few bins: the lanes that share a bin add their count once (plain LDS atomics would serialise them)
+            for (int c0 = 0; c0 < count; c0 += SAMPLE_THREADS) {
+                const int c = c0 + tid;
+                const int id = c < count ? item(c) : -1;
+                const int digit = id >= 0 ? (int)(ordered_bits(s[id]) >> 24) : -1;
+                unsigned long long todo = __ballot(digit >= 0);
+                while (todo) {
+                    const int leader = __ffsll((long long)todo) - 1;
+                    const int d = __shfl(digit, leader, 64);
+                    const unsigned long long same = __ballot(digit == d);
+                    if ((tid & 63) == leader) atomicAdd(&sh.hist[d], __popcll(same));
+                    todo &= ~same;
+                }
+            }
+        } else {
+            for (int c = tid; c < count; c += SAMPLE_THREADS) {
+                const int id = item(c);
+                if (id < 0) continue;
+                const uint32_t b = ordered_bits(s[id]);
+                if ((b & mask) == prefix) atomicAdd(&sh.hist[(b >> shift) & 255u], 1);
+            }
+        }
+        __syncthreads();
+        if (tid < 64) {
+            // the first bin from the top down to which the bins hold `left` items (bin 0 when they never do): lane l
+            // has bins 255 - 4l .. 252 - 4l, the lanes' sums are scanned, and the lane in which `left` is reached walks its four
+            const int left = sh.remaining, top = 255 - 4 * tid;
+            const int c0 = sh.hist[top], c1 = sh.hist[top - 1], c2 = sh.hist[top - 2], c3 = sh.hist[top - 3];
+            int incl = c0 + c1 + c2 + c3;
+            const int own = incl;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(incl, o, 64);
+                if (tid >= o) incl += up;
+            }
+            const unsigned long long reached = __ballot(incl >= left);
+            const int total = __shfl(incl, 63, 64);
+            if (reached == 0ull) {
+                if (tid == 63) {   // fewer items than wanted: every bin is kept; what is left is asked of bin 0
+                    sh.prefix = prefix;
+                    sh.remaining = left - (total - c3);
+                }
+            } else if (tid == __ffsll((long long)reached) - 1) {
+                int above = incl - own, bin = top;
+                const int c[4] = {c0, c1, c2, c3};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (above + c[j] >= left) {
+                        bin = top - j;
+                        break;
+                    }
+                    above += c[j];
+                }
+                if (bin == 0) above = total - c3;   // bin 0 is never skipped: as when nothing above it reaches `left`
+                sh.prefix = prefix | ((uint32_t)bin << shift);
+                sh.remaining = left - above;  // how many of this bin (finally: of the threshold's equals) are kept
+            }
+        }
+        __syncthreads();
+    }
+    const uint32_t threshold = sh.prefix;
+    const int need_equal = sh.remaining;
+
+    // the kept items in item order: thread t owns the contiguous items [t*c, (t+1)*c)
+    const int chunk = (count + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+    const int begin = min(count, tid * chunk), end = min(count, begin + chunk);
+    int n_equal = 0;
+    for (int c = begin; c < end; ++c) {
+        const int id = item(c);
+        if (id >= 0 && ordered_bits(s[id]) == threshold) ++n_equal;
+    }
+    int total_equal;
+    const int equal_before = block_exclusive_scan(n_equal, sh.scan_scratch, &total_equal);
+    int n_mine = 0;
+    {
+        int eq = equal_before;
+        for (int c = begin; c < end; ++c) {
+            const int id = item(c);
+            if (id < 0) continue;
+            const uint32_t b = ordered_bits(s[id]);
+            if (b > threshold || (b == threshold && eq++ < need_equal)) ++n_mine;
+        }
+    }
+    int n_kept;
+    int at = block_exclusive_scan(n_mine, sh.scan_scratch, &n_kept);
+    {
+        int eq = equal_before;
+        for (int c = begin; c < end; ++c) {
+            const int id = item(c);
+            if (id < 0) continue;
+            const float v = s[id];
+            const uint32_t b = ordered_bits(v);
+            if (b > threshold || (b == threshold && eq++ < need_equal)) emit(at++, id, v);
+        }
+    }
+    __syncthreads();
+    return n_kept;
+}
+
+// The row's settings as every stage reads them: the masked id (n for none), the ids taking part, the tokens kept.
+__device__ __forceinline__ void topk_row_settings(const int* skip, const int* top_k, int r, int n, int& sk, int& keep) {
+    sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
+    const int m = sk < n ? n - 1 : n;
+    keep = top_k[r];
+    if (keep <= 0 || keep > m) keep = m;  // the host sends only rows with keep <= SAMPLE_MAX_KEEP
+    if (keep > SAMPLE_MAX_KEEP) keep = SAMPLE_MAX_KEEP;
+}
+
+// Rows of many scores are searched by many workgroups.  Stage 1: workgroup (slice, row) keeps the `keep` best of its
+// slice of the row; whatever is among the row's `keep` best is among its slice's.  The slices' kept ids go to
+// cand[row][slice][0 .. stride) in id order, -1 where a slice keeps fewer, so that the row's candidates stay in id order.
+__global__ void __launch_bounds__(SAMPLE_THREADS) topk_slices_kernel(const float* __restrict__ scores, const int* __restrict__ top_k,
+                                                                    const int* __restrict__ skip, int* __restrict__ cand, int n,
+                                                                    int slice_len, int stride) {
+    __shared__ TopkShared sh;
+    const int r = blockIdx.y, sl = blockIdx.x, tid = threadIdx.x;
+    const float* s = scores + (size_t)r * n;
+    int sk, keep;
+    topk_row_settings(skip, top_k, r, n, sk, keep);
+    if (keep > stride) keep = stride;   // cannot happen: the host sizes the stride for the largest top_k it sends
+    const int begin = sl * slice_len, count = max(0, min(n, begin + slice_len) - begin);
+    int* mine = cand + ((size_t)r * gridDim.x + sl) * stride;
+    const int kept = select_topk(s, count, [&](int c) { return begin + c == sk ? -1 : begin + c; }, keep,
+                                 [&](int place, int id, float) { mine[place] = id; }, sh);
+    for (int i = kept + tid; i < stride; i += SAMPLE_THREADS) mine[i] = -1;
+}
+
+// The draw from a row's items: the `keep` best are selected and gathered in id order, weighted, and drawn from in the
+// reference's order by one thread.  ITEMS_ARE_IDS: the items are all the row's ids; else `items` lists candidate ids in
+// rising order with -1 for none (stage 2 of the search by slices).
+template <bool ITEMS_ARE_IDS>
 __global__ void __launch_bounds__(SAMPLE_THREADS) sample_topk_kernel(const float* __restrict__ scores, const float* __restrict__ temp,
                                                                     const int* __restrict__ top_k, const float* __restrict__ top_p,
                                                                     const float* __restrict__ min_p, const float* __restrict__ unit,
-                                                                    const int* __restrict__ skip, int* __restrict__ out, int n) {
-    __shared__ int hist[256];
-    __shared__ int scan_scratch[SAMPLE_WAVES];
-    __shared__ uint32_t prefix_s;
-    __shared__ int remaining_s;
+                                                                    const int* __restrict__ skip, int* __restrict__ out, int n,
+                                                                    const int* __restrict__ items, int n_items) {
+    __shared__ TopkShared sh;
     __shared__ int kept_id[SAMPLE_MAX_KEEP];
     __shared__ float kept_score[SAMPLE_MAX_KEEP];
     __shared__ float kept_w[SAMPLE_MAX_KEEP];
     __shared__ int ranked[SAMPLE_MAX_KEEP];  // ranked[i] = place in kept_* of the i-th best
     const int r = blockIdx.x, tid = threadIdx.x;
     const float* s = scores + (size_t)r * n;
-    const int sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
-    const int m = sk < n ? n - 1 : n;
-    int keep = top_k[r];
-    if (keep <= 0 || keep > m) keep = m;  // the host sends only rows with keep <= SAMPLE_MAX_KEEP
-    if (keep > SAMPLE_MAX_KEEP) keep = SAMPLE_MAX_KEEP;
+    int sk, keep;
+    topk_row_settings(skip, top_k, r, n, sk, keep);
 
-    // 1. radix select of the keep-th largest ordered score, 8 bits a pass from the top
-    if (tid == 0) {
-        prefix_s = 0;
-        remaining_s = keep;
-    }
-    for (int pass = 0; pass < 4; ++pass) {
-        const int shift = 24 - 8 * pass;
-        if (tid < 256) hist[tid] = 0;
-        __syncthreads();
-        const uint32_t prefix = prefix_s;
-        const uint32_t mask = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8));
-        for (int i = tid; i < n; i += SAMPLE_THREADS) {
-            if (i == sk) continue;
-            const uint32_t b = ordered_bits(s[i]);
-            if ((b & mask) == prefix) atomicAdd(&hist[(b >> shift) & 255u], 1);
+    // 1. and 2.: the kept tokens, in id order
+    auto keep_it = [&](int place, int id, float v) {
+        if (place < SAMPLE_MAX_KEEP) {
+            kept_id[place] = id;
+            kept_score[place] = v;
         }
-        __syncthreads();
-        if (tid == 0) {
-            int left = remaining_s, bin = 255;
-            for (; bin > 0; --bin) {
-                if (hist[bin] >= left) break;
-                left -= hist[bin];
-            }
-            prefix_s = prefix | ((uint32_t)bin << shift);
-            remaining_s = left;  // how many of this bin (finally: of the threshold's equals) are kept
-        }
-        __syncthreads();
-    }
-    const uint32_t threshold = prefix_s;
-    const int need_equal = remaining_s;
-
-    // 2. gather the kept tokens in id order: thread t owns the contiguous ids [t*c, (t+1)*c)
-    const int chunk = (n + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-    const int begin = min(n, tid * chunk), end = min(n, begin + chunk);
-    int n_equal = 0;
-    for (int i = begin; i < end; ++i)
-        if (i != sk && ordered_bits(s[i]) == threshold) ++n_equal;
-    int total_equal;
-    const int equal_before = block_exclusive_scan(n_equal, scan_scratch, &total_equal);
-    int n_mine = 0;
-    {
-        int eq = equal_before;
-        for (int i = begin; i < end; ++i) {
-            if (i == sk) continue;
-            const uint32_t b = ordered_bits(s[i]);
-            if (b > threshold || (b == threshold && eq++ < need_equal)) ++n_mine;
-        }
-    }
+    };
     int n_kept;
-    int at = block_exclusive_scan(n_mine, scan_scratch, &n_kept);
-    {
-        int eq = equal_before;
-        for (int i = begin; i < end; ++i) {
-            if (i == sk) continue;
-            const uint32_t b = ordered_bits(s[i]);
-            if (b > threshold || (b == threshold && eq++ < need_equal)) {
-                if (at < SAMPLE_MAX_KEEP) {
-                    kept_id[at] = i;
-                    kept_score[at] = s[i];
-                }
-                ++at;
-            }
-        }
+    if (ITEMS_ARE_IDS) {
+        n_kept = select_topk(s, n, [&](int c) { return c == sk ? -1 : c; }, keep, keep_it, sh);
+    } else {
+        const int* mine = items + (size_t)r * n_items;
+        n_kept = select_topk(s, n_items, [&](int c) { return mine[c]; }, keep, keep_it, sh);
     }
-    __syncthreads();
     if (n_kept > SAMPLE_MAX_KEEP) n_kept = SAMPLE_MAX_KEEP;
 
     // rank of each kept token: how many kept tokens are better (higher score, or equal score and lower id)
@@ -483,11 +586,40 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_topk_kernel(const float
     }
 }
 
+// Slices a row of n scores is searched in by llmx_sample_topk when it is given scratch (1: the row is searched whole).
+#define TOPK_SLICE_MIN 4096
+#define TOPK_MAX_SLICES 32
+static int topk_slices(int n) {
+    int s = n / TOPK_SLICE_MIN;
+    return s < 2 ? 1 : (s > TOPK_MAX_SLICES ? TOPK_MAX_SLICES : s);
+}
+
+// Ints of scratch llmx_sample_topk wants for rows of n scores whose largest top_k is max_keep (0: none).
+extern "C" long llmx_sample_topk_scratch(int rows, int n, int max_keep) {
+    const int slices = topk_slices(n);
+    if (slices < 2 || rows <= 0) return 0;
+    if (max_keep < 1 || max_keep > SAMPLE_MAX_KEEP) max_keep = SAMPLE_MAX_KEEP;
+    return (long)rows * slices * max_keep;
+}
+
+// cand: llmx_sample_topk_scratch(rows, n, max_keep) ints, or null: every row is then searched by one workgroup.
+// max_keep: no row's top_k is above it (rows whose top_k is 0 or above SAMPLE_MAX_KEEP are not this kernel's).
 extern "C" int llmx_sample_topk(const float* scores, const float* temp, const int* top_k, const float* top_p, const float* min_p,
-                                const float* unit, const int* skip, int* out, int rows, int n, hipStream_t stream) {
+                                const float* unit, const int* skip, int* out, int rows, int n, int* cand, int max_keep, hipStream_t stream) {
     if (rows <= 0) return 0;
     llmx_note_launch(LK_SAMPLE_TOPK);
-    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n);
+    if (rows > 65535 || n <= 0) return -2;
+    const int slices = topk_slices(n);
+    if (!cand || slices < 2) {
+        hipLaunchKernelGGL(sample_topk_kernel<true>, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out,
+                           n, (const int*)nullptr, 0);
+        return LLMX_CHECK_LAUNCH();
+    }
+    if (max_keep < 1 || max_keep > SAMPLE_MAX_KEEP) max_keep = SAMPLE_MAX_KEEP;
+    const int slice_len = (n + slices - 1) / slices;
+    hipLaunchKernelGGL(topk_slices_kernel, dim3(slices, rows), dim3(SAMPLE_THREADS), 0, stream, scores, top_k, skip, cand, n, slice_len, max_keep);
+    hipLaunchKernelGGL(sample_topk_kernel<false>, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n,
+                       (const int*)cand, slices * max_keep);
     return LLMX_CHECK_LAUNCH();
 }
 

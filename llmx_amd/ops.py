@@ -75,7 +75,7 @@ def _declare(h) -> None:
         "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P],
         "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
-        "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P],
+        "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P, I, P],
         "llmx_sample_ranked": [P, P, P, P, P, P, P, P, I, I, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
     }
@@ -87,6 +87,8 @@ def _declare(h) -> None:
             raise KernelError(f"the kernel library lacks {name}; build it again from the current sources") from None
         fn.argtypes = args
         fn.restype = c_int
+    h.llmx_sample_topk_scratch.argtypes = [I, I, I]
+    h.llmx_sample_topk_scratch.restype = c_long
     h.llmx_launch_name.restype = ctypes.c_char_p
     h.llmx_note_launch.restype = None
 
@@ -617,14 +619,19 @@ def sample_all(scores: torch.Tensor, temp: torch.Tensor, unit: torch.Tensor, out
 
 
 def sample_topk(scores: torch.Tensor, temp: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,
-                unit: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Tensor] = None) -> None:
-    """Top-k (1..1024 per row), top-p, min-p and the draw; rows whose top_k is outside 1..1024 must not be read from `out`."""
+                unit: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Tensor] = None, max_keep: int = 1024, slices: bool = True) -> None:
+    """Top-k (1..1024 per row), top-p, min-p and the draw; rows whose top_k is outside 1..1024 must not be read from `out`.
+    `max_keep`: no row's top_k is above it (it sizes the scratch).  Rows of many scores are searched by many workgroups
+    (each keeps the best of a slice, one more ranks the slices' candidates and draws); `slices=False` keeps a row to one
+    workgroup.  The token is the same either way."""
     rows, n = scores.shape
+    need = lib().llmx_sample_topk_scratch(rows, n, int(max_keep)) if slices else 0
+    cand = _scratch("sample_topk.candidates", need, torch.int32, scores.device) if need else None
     _check(lib().llmx_sample_topk(_dev(scores, "scores", torch.float32), _dev(temp, "temp", torch.float32, (rows,)),
                                   _dev(top_k, "top_k", torch.int32, (rows,)), _dev(top_p, "top_p", torch.float32, (rows,)),
                                   _dev(min_p, "min_p", torch.float32, (rows,)), _dev(unit, "unit", torch.float32, (rows,)),
-                                  _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()),
-           "sample_topk")
+                                  _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n,
+                                  _dev(cand, "candidates"), int(max_keep), _stream()), "sample_topk")
 
 
 def sample_ranked(scores: torch.Tensor, temp: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,

@@ -63,10 +63,12 @@ class Sampler:
         if "all" in which:
             ops.sample_all(logits, temp, unit, out, min_p, skip)
             results["all"] = out
-        for name, kernel in (("topk", ops.sample_topk), ("ranked", ops.sample_ranked)):
-            if name in which:
-                results[name] = torch.zeros(W, dtype=torch.int32, device=self.device)
-                kernel(logits, temp, st["top_k"], st["top_p"], min_p, unit, results[name], skip)
+        if "topk" in which:
+            results["topk"] = torch.zeros(W, dtype=torch.int32, device=self.device)
+            ops.sample_topk(logits, temp, st["top_k"], st["top_p"], min_p, unit, results["topk"], skip, max_keep=st["max_keep"])
+        if "ranked" in which:
+            results["ranked"] = torch.zeros(W, dtype=torch.int32, device=self.device)
+            ops.sample_ranked(logits, temp, st["top_k"], st["top_p"], min_p, unit, results["ranked"], skip)
         if len(results) == 1:
             return next(iter(results.values())).tolist()
         lists = {name: t.tolist() for name, t in results.items()}
@@ -98,5 +100,7 @@ class Sampler:
             st["min_p"] = self._f32([p.min_p for p in params])
             if "topk" in st["which"] or "ranked" in st["which"]:
                 st["top_k"], st["top_p"] = self._i32([p.top_k for p in params]), self._f32([p.top_p for p in params])
+                # the largest top_k among the rows the exact kernel takes: it sizes that kernel's candidate lists
+                st["max_keep"] = max([p.top_k for p, w in zip(params, st["which"]) if w == "topk"] or [1])
         self._kept = (key, st)
         return st

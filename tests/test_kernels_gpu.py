@@ -953,6 +953,55 @@ def test_ranked_sampler_matches_reference_draw_for_draw(V, draws):
     assert out.tolist() == [-5] * rows
 
 
+@pytest.mark.parametrize("V", [8192, 9001, 200064])
+def test_topk_sampler_searched_by_slices_gives_the_token_of_one_workgroup(V):
+    """Rows of many scores are searched by many workgroups (each keeps the best of a slice of the row, one more ranks the
+    slices' candidates and draws).  The token must be the one a single workgroup over the whole row gives, for every
+    top_k from 1 to 1,024, with rows of ties (where the lower id ranks first, also across slices), a masked id, a best
+    token at a slice's edge, and a top_k above what one slice holds of the row's best."""
+    o = ops()
+    from llmx_amd.sampling import XorShift64
+    settings = [dict(temp=0.8, top_k=40, top_p=0.95, min_p=0.0), dict(temp=1.0, top_k=1, top_p=1.0, min_p=0.0),
+                dict(temp=1.3, top_k=1024, top_p=1.0, min_p=0.0), dict(temp=0.7, top_k=1024, top_p=0.9, min_p=0.01),
+                dict(temp=1.0, top_k=7, top_p=1.0, min_p=0.2), dict(temp=1.1, top_k=300, top_p=0.5, min_p=0.0),
+                dict(temp=0.9, top_k=64, top_p=0.99, min_p=0.0), dict(temp=1.0, top_k=500, top_p=1.0, min_p=0.0)]
+    rows = len(settings)
+    logits = rnd(rows, V, scale=2.0, seed=V + 3)
+    logits[2] = torch.round(logits[2] * 2.0) / 2.0              # ties: steps of 0.5, far more equals than are kept
+    logits[5] = torch.round(logits[5])
+    logits[6, :] = -3.0                                         # the whole best set inside one slice
+    logits[6, 100:180] = torch.linspace(1.0, 2.0, 80)
+    slice_len = -(-V // max(1, min(32, V // 4096)))
+    logits[0, slice_len - 1] = 30.0                             # the best tokens on both sides of a slice's edge
+    logits[0, min(V - 1, slice_len)] = 30.0
+    skip_ids = [-1, int(logits[1].argmax()), -1, 11, -1, -1, -1, V - 1]
+    logits = logits.to(DEV)
+    skip = torch.tensor(skip_ids, dtype=torch.int32, device=DEV)
+    f = lambda key: torch.tensor([s[key] for s in settings], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([s["top_k"] for s in settings], dtype=torch.int32, device=DEV)
+    rng = XorShift64(V)
+    seen = set()
+    for draw in range(60):
+        units = [rng.unit() for _ in range(rows)]
+        if draw == 0:
+            units[:2] = [0.0, 1.0 - 2.0 ** -24]
+        unit = torch.tensor(units, dtype=torch.float32, device=DEV)
+        whole = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        o.sample_topk(logits, f("temp"), top_k, f("top_p"), f("min_p"), unit, whole, skip, slices=False)
+        for max_keep in (1024, 1024 if draw % 2 else max(s["top_k"] for s in settings)):
+            sliced = torch.full((rows,), -2, dtype=torch.int32, device=DEV)
+            o.sample_topk(logits, f("temp"), top_k, f("top_p"), f("min_p"), unit, sliced, skip, max_keep=max_keep)
+            assert sliced.tolist() == whole.tolist(), f"draw {draw}: by slices {sliced.tolist()}, whole {whole.tolist()}"
+        seen.update(whole.tolist())
+    assert len(seen) > 100
+    # one row with a small top_k and a scratch sized for it: the candidate lists are top_k wide
+    one = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    o.sample_topk(logits[:1], f("temp")[:1], top_k[:1], f("top_p")[:1], f("min_p")[:1], unit[:1], one, None, max_keep=40)
+    want = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    o.sample_topk(logits[:1], f("temp")[:1], top_k[:1], f("top_p")[:1], f("min_p")[:1], unit[:1], want, None, slices=False)
+    assert one.tolist() == want.tolist()
+
+
 def test_ranked_sampler_over_the_whole_vocabulary_200_draws():
     """The search by histograms forms its sums in 64-bit fixed point where the reference sums doubles: 200 draws a row at
     the real vocabulary (a nucleus over the whole row; a top-k of 5,000; a nucleus with min_p inside a top-k of 50,000),
