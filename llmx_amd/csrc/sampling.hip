@@ -252,11 +252,176 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_all_kernel(const float*
     if (tid == 0) out[r] = found >= 0 ? found : best;
 }
 
+// The same draw for wide rows by many workgroups.  Stage 1 (argmax_slices_kernel) leaves every slice's leader; stage 2
+// gives every slice of 8,192 scores a workgroup that merges the leaders (the row's best score is what the weights are
+// taken against) and sums its slice's weights in double: a thread sums 32 consecutive ids in id order, the threads'
+// sums are added in thread order; stage 3, one workgroup a row, adds the slices' sums in slice order, finds the slice
+// and the thread whose range holds the target from the same sums, and walks that range.  The reference adds all
+// weights in id order (sampler.hpp:341-352); a different order of double additions moves the target by parts in 1e16.
+__device__ int merged_leader(const float* __restrict__ s, const Leader* __restrict__ partial, int n_slices, int n, int sk) {
+    // every thread of the first wave takes part; the result is valid in every lane of that wave
+    Leader best{-INFINITY, -1};
+    for (int i = threadIdx.x & 63; i < n_slices; i += 64) {
+        const Leader c = partial[i];
+        if (beats(c, best)) best = c;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        Leader other{__shfl_xor(best.score, o, 64), __shfl_xor(best.id, o, 64)};
+        if (beats(other, best)) best = other;
+    }
+    const int first = sk == 0 ? 1 : 0;
+    const float lead = s[first];
+    return (lead != lead || best.id < 0) ? first : best.id;
+}
+
+#define SAMPLE_ALL_CHUNK (ARGMAX_SLICE / 256)
+// A slice's weights in LDS: the scores are read side by side (thread t takes ids t, t + 256, ...), the weights stored so
+// that thread t then finds its 32 consecutive ids (its share of the sums, in id order) without bank conflicts: one
+// float of padding every 32.  A masked id and ids past the row weigh 0.  Every thread of the block calls it.
+__device__ __forceinline__ int weight_slot(int j) { return j + (j >> 5); }
+__device__ void slice_weights(const float* __restrict__ s, int slice_begin, int n, int sk, float best_score, float tmp, float cut,
+                              float* __restrict__ wbuf) {
+#pragma unroll 4
+    for (int i = 0; i < SAMPLE_ALL_CHUNK; ++i) {
+        const int j = i * 256 + threadIdx.x, id = slice_begin + j;
+        float w = 0.0f;
+        if (id < n && id != sk) {
+            w = expf((s[id] - best_score) / tmp);
+            if (w < cut) w = 0.0f;
+        }
+        wbuf[weight_slot(j)] = w;
+    }
+    __syncthreads();
+}
+// The thread's 32 consecutive weights added in id order in double.
+__device__ __forceinline__ double thread_weight(const float* __restrict__ wbuf) {
+    double sum = 0.0;
+#pragma unroll 4
+    for (int i = 0; i < SAMPLE_ALL_CHUNK; ++i) sum += (double)wbuf[weight_slot(threadIdx.x * SAMPLE_ALL_CHUNK + i)];
+    return sum;
+}
+
+__global__ void __launch_bounds__(256) sample_all_sums_kernel(const float* __restrict__ scores, const float* __restrict__ temp,
+                                                             const float* __restrict__ min_p, const int* __restrict__ skip,
+                                                             const Leader* __restrict__ partial, double* __restrict__ slice_sums, int n,
+                                                             int n_slices) {
+    __shared__ float wbuf[ARGMAX_SLICE + ARGMAX_SLICE / 32];
+    __shared__ double sums[256];
+    __shared__ int best_s;
+    const int r = blockIdx.y, sl = blockIdx.x, tid = threadIdx.x;
+    const float tmp = temp[r];
+    if (!(tmp > 0.0f)) return;   // a greedy row needs no sums
+    const float* s = scores + (size_t)r * n;
+    const int sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
+    if (tid < 64) {
+        const int best = merged_leader(s, partial + (size_t)r * n_slices, n_slices, n, sk);
+        if (tid == 0) best_s = best;
+    }
+    __syncthreads();
+    slice_weights(s, sl * ARGMAX_SLICE, n, sk, s[best_s], tmp, min_p ? min_p[r] : 0.0f, wbuf);
+    sums[tid] = thread_weight(wbuf);
+    __syncthreads();
+    if (tid == 0) {
+        double total = 0.0;
+        for (int t = 0; t < 256; ++t) total += sums[t];
+        slice_sums[(size_t)r * n_slices + sl] = total;
+    }
+}
+
+__global__ void __launch_bounds__(256) sample_all_draw_kernel(const float* __restrict__ scores, const float* __restrict__ temp,
+                                                             const float* __restrict__ unit, const float* __restrict__ min_p,
+                                                             const int* __restrict__ skip, const Leader* __restrict__ partial,
+                                                             const double* __restrict__ slice_sums, int* __restrict__ out, int n, int n_slices) {
+    __shared__ float wbuf[ARGMAX_SLICE + ARGMAX_SLICE / 32];
+    __shared__ double sums[256];
+    __shared__ int best_s, found, slice_s;
+    __shared__ double before_s, target_s;
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float* s = scores + (size_t)r * n;
+    const int sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
+    if (tid < 64) {
+        const int best = merged_leader(s, partial + (size_t)r * n_slices, n_slices, n, sk);
+        if (tid == 0) {
+            best_s = best;
+            found = -1;
+            slice_s = -1;
+        }
+    }
+    __syncthreads();
+    const int best = best_s;
+    const float tmp = temp[r];
+    if (!(tmp > 0.0f)) {
+        if (tid == 0) out[r] = best;
+        return;
+    }
+    if (tid == 0) {
+        // the slice whose running sum first exceeds the target
+        const double* mine = slice_sums + (size_t)r * n_slices;
+        double total = 0.0;
+        for (int i = 0; i < n_slices; ++i) total += mine[i];
+        const double target = (double)unit[r] * total;
+        double acc = 0.0;
+        for (int i = 0; i < n_slices; ++i) {
+            if (target < acc + mine[i]) {
+                slice_s = i;
+                before_s = acc;
+                break;
+            }
+            acc += mine[i];
+        }
+        target_s = target;
+    }
+    __syncthreads();
+    const int sl = slice_s;
+    if (sl >= 0) {
+        slice_weights(s, sl * ARGMAX_SLICE, n, sk, s[best], tmp, min_p ? min_p[r] : 0.0f, wbuf);
+        const double mine = thread_weight(wbuf);   // the very sums stage 2 formed
+        sums[tid] = mine;
+        __syncthreads();
+        double before = before_s;
+        for (int t = 0; t < tid; ++t) before += sums[t];
+        const double target = target_s;
+        if (target >= before && target < before + mine) {
+            double acc = before;
+            for (int i = 0; i < SAMPLE_ALL_CHUNK; ++i) {
+                acc += (double)wbuf[weight_slot(tid * SAMPLE_ALL_CHUNK + i)];
+                if (target < acc) {
+                    found = sl * ARGMAX_SLICE + tid * SAMPLE_ALL_CHUNK + i;
+                    break;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (tid == 0) out[r] = found >= 0 ? found : best;
+}
+
+// Bytes of scratch llmx_sample_all wants for rows of n scores (0: a row is narrow enough for one workgroup).
+extern "C" long llmx_sample_all_scratch(int rows, int n) {
+    if (n <= 2 * ARGMAX_SLICE || rows <= 0) return 0;
+    return (long)rows * ((n + ARGMAX_SLICE - 1) / ARGMAX_SLICE) * (long)(sizeof(Leader) + sizeof(double));
+}
+
+// scratch: llmx_sample_all_scratch(rows, n) bytes, 8-byte aligned, or null: every row is then walked by one workgroup.
 extern "C" int llmx_sample_all(const float* scores, const float* temp, const float* unit, const float* min_p, const int* skip, int* out,
-                               int rows, int n, hipStream_t stream) {
+                               int rows, int n, void* scratch, hipStream_t stream) {
     if (rows <= 0) return 0;
     llmx_note_launch(LK_SAMPLE_ALL);
-    hipLaunchKernelGGL(sample_all_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, unit, min_p, skip, out, n);
+    if (n <= 0) return -2;
+    if (n <= 2 * ARGMAX_SLICE || !scratch) {
+        hipLaunchKernelGGL(sample_all_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, unit, min_p, skip, out, n);
+        return LLMX_CHECK_LAUNCH();
+    }
+    if (rows > 65535 || ((uintptr_t)scratch & 7)) return -2;
+    const int n_slices = (n + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
+    double* slice_sums = (double*)scratch;
+    Leader* partial = (Leader*)(slice_sums + (size_t)rows * n_slices);
+    hipLaunchKernelGGL(argmax_slices_kernel, dim3(n_slices, rows), dim3(256), 0, stream, scores, skip, partial, n, n_slices);
+    hipLaunchKernelGGL(sample_all_sums_kernel, dim3(n_slices, rows), dim3(256), 0, stream, scores, temp, min_p, skip, (const Leader*)partial, slice_sums,
+                       n, n_slices);
+    hipLaunchKernelGGL(sample_all_draw_kernel, dim3(rows), dim3(256), 0, stream, scores, temp, unit, min_p, skip, (const Leader*)partial,
+                       (const double*)slice_sums, out, n, n_slices);
     return LLMX_CHECK_LAUNCH();
 }
 

@@ -74,7 +74,7 @@ def _declare(h) -> None:
         "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P, F, P],
         "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P],
         "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
-        "llmx_sample_all": [P, P, P, P, P, P, I, I, P],
+        "llmx_sample_all": [P, P, P, P, P, P, I, I, P, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P, I, P],
         "llmx_sample_ranked": [P, P, P, P, P, P, P, P, I, I, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
@@ -89,6 +89,8 @@ def _declare(h) -> None:
         fn.restype = c_int
     h.llmx_sample_topk_scratch.argtypes = [I, I, I]
     h.llmx_sample_topk_scratch.restype = c_long
+    h.llmx_sample_all_scratch.argtypes = [I, I]
+    h.llmx_sample_all_scratch.restype = c_long
     h.llmx_launch_name.restype = ctypes.c_char_p
     h.llmx_note_launch.restype = None
 
@@ -610,12 +612,17 @@ def gemm_f32(a, w: torch.Tensor, c: torch.Tensor, add: bool = False, parts: Opti
 
 
 def sample_all(scores: torch.Tensor, temp: torch.Tensor, unit: torch.Tensor, out: torch.Tensor, min_p: Optional[torch.Tensor] = None,
-               skip: Optional[torch.Tensor] = None) -> None:
+               skip: Optional[torch.Tensor] = None, slices: bool = True) -> None:
+    """The temperature draw with every token kept.  Rows of many scores are summed by many workgroups (a slice of 8,192
+    scores each) and one more a row finds the token; `slices=False` keeps a row to one workgroup.  The orders of the
+    double additions differ between the two, so their targets can differ in the last bits of a double."""
     rows, n = scores.shape
+    need = lib().llmx_sample_all_scratch(rows, n) if slices else 0
+    scratch = _scratch("sample_all.slices", -(-need // 8), torch.float64, scores.device) if need else None
     _check(lib().llmx_sample_all(_dev(scores, "scores", torch.float32), _dev(temp, "temp", torch.float32, (rows,)),
                                  _dev(unit, "unit", torch.float32, (rows,)), _dev(min_p, "min_p", torch.float32, (rows,)),
-                                 _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()),
-           "sample_all")
+                                 _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n,
+                                 _dev(scratch, "scratch"), _stream()), "sample_all")
 
 
 def sample_topk(scores: torch.Tensor, temp: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,

@@ -1002,6 +1002,43 @@ def test_topk_sampler_searched_by_slices_gives_the_token_of_one_workgroup(V):
     assert one.tolist() == want.tolist()
 
 
+@pytest.mark.parametrize("V", [16385, 20000, 200064])
+def test_temperature_draw_by_slices_gives_the_token_of_one_workgroup(V):
+    """Rows of more than 16,384 scores are summed by a workgroup a slice of 8,192 and one more finds the token; the token is
+    the one a single workgroup walking the whole row finds (150 draws a row: the two add the same doubles in different
+    orders, which moves a target by parts in 1e16), with min_p, a masked id, a greedy row among the others, units at
+    both ends of their range, and against the reference's walk for a sample of the draws."""
+    o = ops()
+    from llmx_amd.sampling import XorShift64
+    temps, min_ps = [0.8, 1.3, 0.0, 2.5, 0.6], [0.0, 0.05, 0.0, 0.0, 0.3]
+    rows = len(temps)
+    logits = rnd(rows, V, scale=2.0, seed=V + 9)
+    logits[3, V - 1] = 9.0                      # the best token is the row's last, in a slice of its own remainder
+    skip_ids = [-1, 5, -1, -1, int(logits[4].argmax())]
+    host = logits.cpu()
+    logits = logits.to(DEV)
+    skip = torch.tensor(skip_ids, dtype=torch.int32, device=DEV)
+    temp, min_p = torch.tensor(temps, device=DEV), torch.tensor(min_ps, device=DEV)
+    rng = XorShift64(V + 1)
+    seen = set()
+    for draw in range(150):
+        units = [rng.unit() for _ in range(rows)]
+        if draw == 0:
+            units[0], units[1] = 0.0, 1.0 - 2.0 ** -24
+        unit = torch.tensor(units, dtype=torch.float32, device=DEV)
+        whole = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        sliced = torch.full((rows,), -2, dtype=torch.int32, device=DEV)
+        o.sample_all(logits, temp, unit, whole, min_p, skip, slices=False)
+        o.sample_all(logits, temp, unit, sliced, min_p, skip)
+        assert sliced.tolist() == whole.tolist(), f"draw {draw}: by slices {sliced.tolist()}, whole {whole.tolist()}"
+        if draw < 4:
+            for r in (0, 1, 4):
+                want = sampler_reference.sample(host[r].tolist(), temps[r], 0, 1.0, min_ps[r], units[r], skip=skip_ids[r] if skip_ids[r] >= 0 else None)
+                assert int(sliced[r]) == want
+        seen.update(sliced.tolist())
+    assert int(sliced[2]) == int(host[2].argmax()) and len(seen) > 100
+
+
 def test_ranked_sampler_over_the_whole_vocabulary_200_draws():
     """The search by histograms forms its sums in 64-bit fixed point where the reference sums doubles: 200 draws a row at
     the real vocabulary (a nucleus over the whole row; a top-k of 5,000; a nucleus with min_p inside a top-k of 50,000),
