@@ -865,180 +865,241 @@ __global__ void __launch_bounds__(64 * AM_TILES128_WAVES) paged_attention_tiles1
     if (col_ok) store_output<DT>(a.out + ((size_t)t * a.n_heads + h) * D, g, o_tot, l_tot);
 }
 
-// merge: one block per output (row, head).  merge item: {row, head, first_slot, column, slots}.  The row's segments are
-// folded in key order with the formula the attention kernel uses for a tile's segments.  The fold's weights depend on
-// the segments' maxima only, so they are formed for 512 segments at a time by all threads (a prefix maximum, then
-// fold_weights per segment); what is left of the chain is O = O * a + o * b per segment, with thread d owning dim d and
-// 64 segments' loads in flight (two rounds of 32 whose registers are asked for again as soon as they are folded).  A
-// round in which every segment folds (none empty, none the first) runs the bare chain; the others choose per segment.
-// Same operations on the same values as a sequential fold: the same bits.  Loads run up to MERGE_PAD segments past a
-// row's last one and are never used: part_o has that many rows more than its slots.
+// The merge's sizes: segments whose weights are formed at a time, segments a round, rounds in flight, and the rows
+// part_o has beyond its slots' (as many segments as the form that asks for all its loads at once covers).
 #define MERGE_CHUNK 512
 #define MERGE_DEPTH 32
 #define MERGE_RING 2
 #define MERGE_PAD (MERGE_DEPTH * MERGE_RING)
-template <bool WIDE>   // WIDE: head_dim above 128, two dims a thread
-__global__ void __launch_bounds__(128) attention_merge_kernel(const int* __restrict__ merges, const int* __restrict__ pos,
-                                                            const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                            bf16_t* __restrict__ out, int n_heads, int D, int window) {
-    static_assert(MERGE_CHUNK % (MERGE_DEPTH * MERGE_RING) == 0, "a chunk is a whole number of turns of the ring");
-    __shared__ __attribute__((aligned(16))) float seg_a[MERGE_CHUNK], seg_b[MERGE_CHUNK], seg_l[MERGE_CHUNK];
-    __shared__ __attribute__((aligned(16))) int seg_code[MERGE_CHUNK];   // 0: empty segment, 1: the first one that is not (the state becomes it), 2: fold
-    // a round is plain when its first segment folds or is the row's first, every other one folds, and nothing but the
-    // row's end follows them: 1 (the first folds) or 2 (the first starts the state); 0 otherwise
-    __shared__ int round_plain[MERGE_CHUNK / MERGE_DEPTH];
-    __shared__ float wave_top[2];
+#define MERGE_CROWD_COLUMNS 1536   // above this many workgroups of short columns, no wave of its own for the sums
+#define MERGE_NARROW_COLUMNS 192   // up to this many workgroups of 128 dims, long columns are merged by workgroups of 64 dims instead
+
+// A chunk's weights in LDS.  code: 0 an empty segment, 1 the first one that is not (the state becomes it), 2 fold.
+// lb: the segment's sum times b (code 2) or the sum itself (code 1).  A round is plain when its first segment folds or
+// is the row's first, every other one folds, and nothing but the row's end follows them: 1 (the first folds) or 2 (the
+// first starts the state); 0 otherwise.
+struct __attribute__((aligned(16))) MergeWeights {
+    float a[MERGE_CHUNK], b[MERGE_CHUNK], lb[MERGE_CHUNK];
+    int code[MERGE_CHUNK];
+    int round_plain[MERGE_CHUNK / MERGE_DEPTH];
+    float wave_top[4];
+    float l_total;
+};
+
+// One round of the merge's chain for the values: O folded with the MERGE_DEPTH segments from `at` on (chunk-relative;
+// the chunk has n segments), whose values of the thread's dim are v.
+__device__ __forceinline__ void fold_round_o(float& O, const float (&v)[MERGE_DEPTH], const MergeWeights& w, int plain, int at, int n) {
+    f32x4_t fa[MERGE_DEPTH / 4], fb[MERGE_DEPTH / 4];
+    if (plain && n - at >= MERGE_DEPTH) {      // the bare chain
+#pragma unroll
+        for (int u = 0; u < MERGE_DEPTH / 4; ++u) {
+            fa[u] = *reinterpret_cast<const f32x4_t*>(&w.a[at + 4 * u]);
+            fb[u] = *reinterpret_cast<const f32x4_t*>(&w.b[at + 4 * u]);
+        }
+        O = plain == 2 ? v[0] : folded(O, fa[0][0], v[0], fb[0][0]);
+#pragma unroll
+        for (int u = 1; u < MERGE_DEPTH; ++u) O = folded(O, fa[u / 4][u % 4], v[u], fb[u / 4][u % 4]);
+    } else {
+        u32x4_t fc[MERGE_DEPTH / 4];
+#pragma unroll
+        for (int u = 0; u < MERGE_DEPTH / 4; ++u) {
+            if (at + 4 * u < n) {     // the same for every thread
+                fa[u] = *reinterpret_cast<const f32x4_t*>(&w.a[at + 4 * u]);
+                fb[u] = *reinterpret_cast<const f32x4_t*>(&w.b[at + 4 * u]);
+                fc[u] = *reinterpret_cast<const u32x4_t*>(&w.code[at + 4 * u]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t code = (at + 4 * u + i < n) ? fc[u][i] : 0u;
+                    const float o = folded(O, fa[u][i], v[4 * u + i], fb[u][i]);
+                    O = code == 2u ? o : (code == 1u ? v[4 * u + i] : O);
+                }
+            }
+        }
+    }
+}
+
+// The same round for the sum L (the same in every thread of the wave that keeps it).
+__device__ __forceinline__ void fold_round_l(float& L, const MergeWeights& w, int plain, int at, int n) {
+    f32x4_t fa[MERGE_DEPTH / 4], fl[MERGE_DEPTH / 4];
+    if (plain && n - at >= MERGE_DEPTH) {
+#pragma unroll
+        for (int u = 0; u < MERGE_DEPTH / 4; ++u) {
+            fa[u] = *reinterpret_cast<const f32x4_t*>(&w.a[at + 4 * u]);
+            fl[u] = *reinterpret_cast<const f32x4_t*>(&w.lb[at + 4 * u]);
+        }
+        L = plain == 2 ? fl[0][0] : fmaf(L, fa[0][0], fl[0][0]);
+#pragma unroll
+        for (int u = 1; u < MERGE_DEPTH; ++u) L = fmaf(L, fa[u / 4][u % 4], fl[u / 4][u % 4]);
+    } else {
+        u32x4_t fc[MERGE_DEPTH / 4];
+#pragma unroll
+        for (int u = 0; u < MERGE_DEPTH / 4; ++u) {
+            if (at + 4 * u < n) {
+                fa[u] = *reinterpret_cast<const f32x4_t*>(&w.a[at + 4 * u]);
+                fl[u] = *reinterpret_cast<const f32x4_t*>(&w.lb[at + 4 * u]);
+                fc[u] = *reinterpret_cast<const u32x4_t*>(&w.code[at + 4 * u]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t code = (at + 4 * u + i < n) ? fc[u][i] : 0u;
+                    const float l = fmaf(L, fa[u][i], fl[u][i]);
+                    L = code == 2u ? l : (code == 1u ? fl[u][i] : L);
+                }
+            }
+        }
+    }
+}
+
+// A chunk's weights: each of the first THREADS threads takes MERGE_CHUNK / THREADS segments of the chunk from c0 on, finds
+// the maximum of everything before each of them (earlier chunks: M; earlier threads: a scan; its own earlier segments)
+// and writes the segment's fold weights, its sum's term and its code, and each round's kind.  M becomes the maximum with
+// the chunk.  Two barriers, which every thread of the workgroup comes to.
+template <int THREADS>
+__device__ __forceinline__ void merge_chunk_weights(const float* base_ml, int c0, int n_seg, float& M, MergeWeights& w) {
+    constexpr int PER = MERGE_CHUNK / THREADS, WAVES = THREADS / 64, HOLD = MERGE_DEPTH / PER;   // HOLD threads hold a round
+    static_assert(MERGE_CHUNK % THREADS == 0 && MERGE_DEPTH % PER == 0 && 64 % HOLD == 0 && WAVES <= 4, "a round lies in whole threads of one wave");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int* mi = merges + (size_t)blockIdx.x * AM_ITEM_INTS;
+    const bool works = tid < THREADS;     // whole waves
+    float mv[PER], lv[PER], before[PER];
+    float excl = -INFINITY;
+    if (works) {
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int sg = c0 + PER * tid + u;
+            const bool in = sg < n_seg;
+            mv[u] = in ? base_ml[(size_t)sg * 2] : -INFINITY;
+            lv[u] = in ? base_ml[(size_t)sg * 2 + 1] : 0.0f;
+        }
+        float incl = mv[0];
+#pragma unroll
+        for (int u = 1; u < PER; ++u) incl = fmaxf(incl, mv[u]);
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const float o = __shfl_up(incl, d, 64);
+            if (lane >= d) incl = fmaxf(incl, o);
+        }
+        if (lane == 63) w.wave_top[wave] = incl;
+        excl = __shfl_up(incl, 1, 64);
+        if (lane == 0) excl = -INFINITY;
+    }
+    __syncthreads();
+    float all = w.wave_top[0];
+#pragma unroll
+    for (int v = 1; v < WAVES; ++v) {
+        if (v <= wave) excl = fmaxf(excl, w.wave_top[v - 1]);
+        all = fmaxf(all, w.wave_top[v]);
+    }
+    if (works) {
+        float run = fmaxf(M, excl);
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            before[u] = run;
+            run = fmaxf(run, mv[u]);
+        }
+        bool folds = true;
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int at = PER * tid + u;
+            const bool round_first = (at % MERGE_DEPTH) == 0;
+            int code = 0;
+            float fa = 1.0f, fb = 0.0f, lb = 0.0f;
+            if (mv[u] != -INFINITY) {
+                code = before[u] == -INFINITY ? 1 : 2;
+                lb = lv[u];
+                if (code == 2) {
+                    float mn;
+                    fold_weights(before[u], mv[u], fa, fb, mn);
+                    lb = lv[u] * fb;
+                }
+            }
+            folds = folds && (code == 2 || (code == 1 && round_first) || c0 + at >= n_seg);
+            w.code[at] = code;
+            w.a[at] = fa;
+            w.b[at] = fb;
+            w.lb[at] = lb;
+        }
+        const unsigned long long every = __ballot(folds), held = HOLD == 64 ? ~0ull : ((1ull << HOLD) - 1ull);
+        if (lane % HOLD == 0)
+            w.round_plain[tid / HOLD] = ((every >> lane) & held) == held ? (mv[0] != -INFINITY && before[0] == -INFINITY ? 2 : 1) : 0;
+    }
+    M = fmaxf(M, all);
+    __syncthreads();
+}
+
+// merge: merge item: {row, head, first_slot, column, slots}; a workgroup folds 64 * OW dims of an output (row, head), so
+// ceil(D / (64 * OW)) workgroups an item.  The row's segments are folded in key order with the formula the attention
+// kernel uses for a tile's segments.  The fold's weights depend on the segments' maxima only, so they are formed for 512
+// segments at a time by the first OW waves (a prefix maximum, then fold_weights per segment); what is left of the chain
+// is O = O * a + o * b per segment, with a thread of the first OW waves owning one dim and 64 segments' loads in flight
+// (two rounds of 32 whose registers are asked for again as soon as they are folded), and L = L * a + l * b, which the
+// last wave keeps (LW): two multiply-adds fewer a segment for the waves whose chain sets the time; with very many short
+// columns the waves' number counts for more, and each thread keeps L itself.  A round in which every
+// segment folds (none empty, none the first) runs the bare chain; the others choose per segment.  Same operations on the
+// same values as a sequential fold: the same bits.  SHORT: no column has more than MERGE_PAD segments; the loads before
+// the loop are all there are.  Loads run up to MERGE_PAD segments past a row's last one and are never used: part_o has
+// that many rows more than its slots.
+template <int OW, bool SHORT, bool LW>
+__global__ void __launch_bounds__(64 * (OW + (LW ? 1 : 0))) attention_merge_kernel(const int* __restrict__ merges, const int* __restrict__ pos,
+                                                                      const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                                      bf16_t* __restrict__ out, int n_heads, int D, int window, int parts) {
+    static_assert(MERGE_CHUNK % (MERGE_DEPTH * MERGE_RING) == 0, "a chunk is a whole number of turns of the ring");
+    __shared__ MergeWeights w;
+    const int tid = threadIdx.x, wave = tid >> 6;
+    const int* mi = merges + (size_t)(blockIdx.x / parts) * AM_ITEM_INTS;
     const int t = mi[0], h = mi[1], first = mi[2], c = mi[3], slots = mi[4];
     const int p = pos[t];
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int n_seg = p / AM_SEG - lo / AM_SEG + 1;
     const float* base_o = part_o + ((size_t)first * 16 + (size_t)c * slots) * D;
     const float* base_ml = part_ml + ((size_t)first * 16 + (size_t)c * slots) * 2;
-    float M = -INFINITY, L = 0.0f;   // the same in every thread
-    float O[WIDE ? 2 : 1] = {};       // dims tid and tid + 128
-    const int d0 = tid < D ? tid : 0, d1 = tid + 128 < D ? tid + 128 : 0;
-    float ring[MERGE_RING][WIDE ? 2 : 1][MERGE_DEPTH];
+    float M = -INFINITY, L = 0.0f;   // M the same in every thread; L kept by the last wave, or by every thread
+    float O = 0.0f;
+    const int dim = (blockIdx.x % parts) * 64 * OW + tid;      // of the first OW waves
+    const int d0 = dim < D ? dim : 0;
+    float ring[MERGE_RING][MERGE_DEPTH];
     // a column's segments lie within a few hundred KB of its base: 32-bit byte offsets from it
     const uint32_t seg_bytes = (uint32_t)D * 4u;
-    auto fetch = [&](float (&to)[WIDE ? 2 : 1][MERGE_DEPTH], int first_seg) {
-        const uint32_t at0 = (uint32_t)first_seg * seg_bytes + (uint32_t)d0 * 4u, at1 = (uint32_t)first_seg * seg_bytes + (uint32_t)d1 * 4u;
+    auto fetch = [&](float (&to)[MERGE_DEPTH], int first_seg) {
+        const uint32_t at0 = (uint32_t)first_seg * seg_bytes + (uint32_t)d0 * 4u;
 #pragma unroll
-        for (int u = 0; u < MERGE_DEPTH; ++u) {
-            to[0][u] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(base_o) + (at0 + (uint32_t)u * seg_bytes));
-            if constexpr (WIDE) to[1][u] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(base_o) + (at1 + (uint32_t)u * seg_bytes));
-        }
+        for (int u = 0; u < MERGE_DEPTH; ++u)
+            to[u] = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(base_o) + (at0 + (uint32_t)u * seg_bytes));
     };
+    // Within the loop of the waves that fold values every load stands outside every branch (a round past the row's end
+    // asks for the last round again, and is not folded): the compiler counts the loads in flight exactly only along
+    // straight code, and after a branch that holds loads it waits for all of them, which would leave one round in flight
+    // instead of the ring.
+    const int last_round = (n_seg - 1) / MERGE_DEPTH * MERGE_DEPTH;
+    if (wave < OW) {
 #pragma unroll
-    for (int r = 0; r < MERGE_RING; ++r)
-        if (MERGE_DEPTH * r < n_seg) fetch(ring[r], MERGE_DEPTH * r);
+        for (int r = 0; r < MERGE_RING; ++r) fetch(ring[r], min(MERGE_DEPTH * r, last_round));
+    }
     for (int c0 = 0; c0 < n_seg; c0 += MERGE_CHUNK) {
-        // the thread's 4 segments of the chunk: maxima and sums
-        float mv[4], lv[4], before[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int sg = c0 + 4 * tid + u;
-            const bool in = sg < n_seg;
-            mv[u] = in ? base_ml[(size_t)sg * 2] : -INFINITY;
-            lv[u] = in ? base_ml[(size_t)sg * 2 + 1] : 0.0f;
-        }
-        // the maximum of everything before each segment: earlier chunks, earlier threads, the thread's earlier segments
-        float mine = fmaxf(fmaxf(mv[0], mv[1]), fmaxf(mv[2], mv[3]));
-        float incl = mine;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const float o = __shfl_up(incl, d, 64);
-            if (lane >= d) incl = fmaxf(incl, o);
-        }
-        if (lane == 63) wave_top[wave] = incl;
-        float excl = __shfl_up(incl, 1, 64);
-        if (lane == 0) excl = -INFINITY;
-        __syncthreads();
-        if (wave == 1) excl = fmaxf(excl, wave_top[0]);
-        float run = fmaxf(M, excl);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            before[u] = run;
-            run = fmaxf(run, mv[u]);
-        }
-        bool folds = true;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int at = 4 * tid + u;
-            const bool round_first = (at % MERGE_DEPTH) == 0;
-            int code = 0;
-            float fa = 1.0f, fb = 0.0f;
-            if (mv[u] != -INFINITY) {
-                code = before[u] == -INFINITY ? 1 : 2;
-                if (code == 2) {
-                    float mn;
-                    fold_weights(before[u], mv[u], fa, fb, mn);
-                }
-            }
-            folds = folds && (code == 2 || (code == 1 && round_first) || c0 + at >= n_seg);
-            seg_code[at] = code;
-            seg_a[at] = fa;
-            seg_b[at] = fb;
-            seg_l[at] = lv[u];
-        }
-        // 8 threads hold a round's 32 segments
-        const unsigned long long every = __ballot(folds);
-        if ((lane & 7) == 0) round_plain[tid >> 3] = ((every >> lane) & 0xffull) == 0xffull ? (mv[0] != -INFINITY && before[0] == -INFINITY ? 2 : 1) : 0;
-        M = fmaxf(M, fmaxf(wave_top[0], wave_top[1]));
-        __syncthreads();
+        merge_chunk_weights<64 * OW>(base_ml, c0, n_seg, M, w);
         const int n = min(MERGE_CHUNK, n_seg - c0);
-        for (int s0 = 0; s0 < n; s0 += MERGE_DEPTH * MERGE_RING) {
+        if (wave < OW) {
+            for (int s0 = 0; s0 < n; s0 += MERGE_DEPTH * MERGE_RING) {
 #pragma unroll
-            for (int r = 0; r < MERGE_RING; ++r) {
-                const int at = s0 + MERGE_DEPTH * r;      // the round's first segment within the chunk
-                if (at < n) {                             // the same for every thread
-                    f32x4_t fa[MERGE_DEPTH / 4], fb[MERGE_DEPTH / 4], fl[MERGE_DEPTH / 4];
-#pragma unroll
-                    for (int u = 0; u < MERGE_DEPTH / 4; ++u) {
-                        fa[u] = *reinterpret_cast<const f32x4_t*>(&seg_a[at + 4 * u]);
-                        fb[u] = *reinterpret_cast<const f32x4_t*>(&seg_b[at + 4 * u]);
-                        fl[u] = *reinterpret_cast<const f32x4_t*>(&seg_l[at + 4 * u]);
-                    }
-                    const int plain = round_plain[at / MERGE_DEPTH];
-                    const int count = min(MERGE_DEPTH, n - at);     // the round's segments that exist
-                    if (plain) {
-                        if (plain == 2) {
-                            L = fl[0][0];
-                            O[0] = ring[r][0][0];
-                            if constexpr (WIDE) O[1] = ring[r][1][0];
-                        } else {
-                            L = folded(L, fa[0][0], fl[0][0], fb[0][0]);
-                            O[0] = folded(O[0], fa[0][0], ring[r][0][0], fb[0][0]);
-                            if constexpr (WIDE) O[1] = folded(O[1], fa[0][0], ring[r][1][0], fb[0][0]);
-                        }
-                        if (count == MERGE_DEPTH) {
-#pragma unroll
-                            for (int u = 1; u < MERGE_DEPTH; ++u) {
-                                const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
-                                L = folded(L, a, l, b);
-                                O[0] = folded(O[0], a, ring[r][0][u], b);
-                                if constexpr (WIDE) O[1] = folded(O[1], a, ring[r][1][u], b);
-                            }
-                        } else {
-#pragma unroll
-                            for (int u = 1; u < MERGE_DEPTH; ++u) {
-                                if (u < count) {    // the same for every thread
-                                    const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
-                                    L = folded(L, a, l, b);
-                                    O[0] = folded(O[0], a, ring[r][0][u], b);
-                                    if constexpr (WIDE) O[1] = folded(O[1], a, ring[r][1][u], b);
-                                }
-                            }
-                        }
-                    } else {
-                        u32x4_t fc[MERGE_DEPTH / 4];
-#pragma unroll
-                        for (int u = 0; u < MERGE_DEPTH / 4; ++u) fc[u] = *reinterpret_cast<const u32x4_t*>(&seg_code[at + 4 * u]);
-#pragma unroll
-                        for (int u = 0; u < MERGE_DEPTH; ++u) {
-                            const uint32_t code = (at + u < n) ? fc[u / 4][u % 4] : 0u;
-                            const float a = fa[u / 4][u % 4], b = fb[u / 4][u % 4], l = fl[u / 4][u % 4];
-                            const float l_fold = folded(L, a, l, b), o0_fold = folded(O[0], a, ring[r][0][u], b);
-                            L = code == 2u ? l_fold : (code == 1u ? l : L);
-                            O[0] = code == 2u ? o0_fold : (code == 1u ? ring[r][0][u] : O[0]);
-                            if constexpr (WIDE) {
-                                const float o1_fold = folded(O[1], a, ring[r][1][u], b);
-                                O[1] = code == 2u ? o1_fold : (code == 1u ? ring[r][1][u] : O[1]);
-                            }
-                        }
+                for (int r = 0; r < MERGE_RING; ++r) {
+                    const int at = s0 + MERGE_DEPTH * r;      // the round's first segment within the chunk
+                    if (at < n) {                             // the same for every thread
+                        fold_round_o(O, ring[r], w, w.round_plain[at / MERGE_DEPTH], at, n);
+                        if constexpr (!LW) fold_round_l(L, w, w.round_plain[at / MERGE_DEPTH], at, n);
                     }
                     // the round's registers are free: ask for the round one turn of the ring ahead
-                    const int next = c0 + at + MERGE_DEPTH * MERGE_RING;
-                    if (next < n_seg) fetch(ring[r], next);
+                    if constexpr (!SHORT) fetch(ring[r], min(c0 + at + MERGE_DEPTH * MERGE_RING, last_round));
                 }
             }
+        } else {
+            for (int at = 0; at < n; at += MERGE_DEPTH) fold_round_l(L, w, w.round_plain[at / MERGE_DEPTH], at, n);
         }
         __syncthreads();
     }
-    const float inv = 1.0f / L;
-    if (tid < D) out[((size_t)t * n_heads + h) * D + tid] = f32_to_bf16(O[0] * inv);
-    if (WIDE && tid + 128 < D) out[((size_t)t * n_heads + h) * D + tid + 128] = f32_to_bf16(O[WIDE ? 1 : 0] * inv);
+    if constexpr (LW) {
+        if (tid == 64 * OW) w.l_total = L;
+        __syncthreads();
+        L = w.l_total;
+    }
+    if (wave < OW && dim < D) out[((size_t)t * n_heads + h) * D + dim] = f32_to_bf16(O * (1.0f / L));
 }
 
 // Rows part_o must have beyond its slots' (see the merge).
@@ -1047,13 +1108,15 @@ extern "C" int llmx_attention_partial_pad() { return MERGE_PAD; }
 // `items` holds first the n_shared items of the prompt tiles that share keys (a multiple of 12: one workgroup each 12, or
 // each 4 for head sizes other than 128),
 // then the n_direct items that fold their segments themselves (slot < 0), then the n_partial items that write them
-// (slot >= 0).  wide_items: a decoding item is worked on by a workgroup of 4 waves instead of one wave (head_dim 128 only;
-// the form for steps of few items; the same bits).
+// (slot >= 0).  forms, bit 0: a decoding item is worked on by a workgroup of 4 waves instead of one wave (head_dim 128 only;
+// the form for steps of few items; the same bits); bit 1: no merged column has more than
+// llmx_attention_partial_pad() segment slots (the merge then asks for all its loads at once).
 extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int* pos, const int* row_entry,
                                          const int* tables, const int* items, int n_shared, int n_direct, int n_partial, const int* merges,
                                          int n_merges,
                                          void* out, float* part_o, float* part_ml, float scale, int n_heads, int n_kv_heads, int head_dim,
-                                         int page_tokens, int max_blocks, int window, int wide_items, hipStream_t stream) {
+                                         int page_tokens, int max_blocks, int window, int forms, hipStream_t stream) {
+    const int wide_items = forms & 1;
     if (n_shared + n_direct + n_partial <= 0) return 0;
     if (n_shared % 12) return -2;
     if (head_dim % 16 || head_dim > AM_MAX_D || page_tokens % 16 || n_heads % n_kv_heads) return -2;
@@ -1070,7 +1133,9 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
     if (n_shared > 0) llmx_note_launch(tiles128 ? LK_ATTENTION_TILES128 : LK_ATTENTION_TILES);
     if (n_direct > 0) llmx_note_launch(LK_ATTENTION_DIRECT);
     if (n_partial > 0) llmx_note_launch(split4 ? LK_ATTENTION_SPLIT4 : LK_ATTENTION_PARTIAL);
-    if (n_merges > 0) llmx_note_launch(LK_ATTENTION_MERGE);
+    // few long columns: 64 dims a workgroup, so that more compute units bring the segments in
+    const bool short_merge = forms & 2, narrow_merge = !short_merge && n_merges * ((head_dim + 127) / 128) <= MERGE_NARROW_COLUMNS;
+    if (n_merges > 0) llmx_note_launch(narrow_merge ? LK_ATTENTION_MERGE_NARROW : LK_ATTENTION_MERGE);
     switch (head_dim / 16) {
 #define AM_CASE(DT)                                                                                                          \
     case DT:                                                                                                                 \
@@ -1089,12 +1154,19 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
         default: return -2;
     }
     if (n_merges > 0) {
-        if (head_dim > 128)
-            hipLaunchKernelGGL(attention_merge_kernel<true>, dim3(n_merges), dim3(128), 0, stream, merges, pos, part_o, part_ml, (bf16_t*)out, n_heads,
-                               head_dim, window);
-        else
-            hipLaunchKernelGGL(attention_merge_kernel<false>, dim3(n_merges), dim3(128), 0, stream, merges, pos, part_o, part_ml, (bf16_t*)out, n_heads,
-                               head_dim, window);
+#define AM_MERGE(OW, SHORT, LW)                                                                                                \
+    hipLaunchKernelGGL((attention_merge_kernel<OW, SHORT, LW>), dim3(n_merges * parts), dim3(64 * (OW + (LW ? 1 : 0))), 0, stream, merges, pos, part_o, part_ml, \
+                       (bf16_t*)out, n_heads, head_dim, window, parts)
+        if (narrow_merge) {
+            const int parts = (head_dim + 63) / 64;
+            AM_MERGE(1, false, true);
+        } else {
+            const int parts = (head_dim + 127) / 128;
+            if (short_merge && n_merges * parts > MERGE_CROWD_COLUMNS) AM_MERGE(2, true, false);
+            else if (short_merge) AM_MERGE(2, true, true);
+            else AM_MERGE(2, false, true);
+        }
+#undef AM_MERGE
     }
     return LLMX_CHECK_LAUNCH();
 }

@@ -38,6 +38,7 @@
     X(ATTENTION_PARTIAL, "attention.partial")                                                                             \
     X(ATTENTION_SPLIT4, "attention.split4")                                                                               \
     X(ATTENTION_MERGE, "attention.merge")                                                                                 \
+    X(ATTENTION_MERGE_NARROW, "attention.merge_narrow")                                                                   \
     X(ROUTE_TOPK, "route_topk")                                                                                           \
     X(MOE_ALIGN, "moe_align")                                                                                             \
     X(ROUTE_TOPK_ALIGN, "route_topk_align")                                                                               \

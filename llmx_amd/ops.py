@@ -341,7 +341,7 @@ class AttentionPlan:
     """Work items of the matrix-core attention kernel for one step's rows (they hold no positions, so a plan serves
     every step with the same rows per request) and the merge list of the items that were split over the context."""
 
-    def __init__(self, shared, items, merges, n_slots, device):
+    def __init__(self, shared, items, merges, n_slots, device, merge_slots=0):
         import numpy as np
         self.n_shared = len(shared)          # prompt tiles, 12 (or three times 4) to a workgroup that shares their keys
         self.n_direct = sum(1 for i in items if i[6] < 0)
@@ -351,6 +351,8 @@ class AttentionPlan:
         self.n_slots = n_slots
         # few decoding items: each is worked on by a workgroup of 4 waves (the kernel takes this form for head_dim 128)
         self.wide_items = 0 < self.n_items - self.n_shared <= ATTENTION_WIDE_ITEMS
+        # no merged column longer than the merge's first loads reach
+        self.short_merge = 0 < merge_slots <= lib().llmx_attention_partial_pad()
         self.items = torch.tensor(np.asarray(items, dtype=np.int32).reshape(-1, 8), device=device) if items else None
         self.merges = torch.tensor(np.asarray(merges, dtype=np.int32).reshape(-1, 8), device=device) if merges else None
 
@@ -411,7 +413,7 @@ def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, 
             for sp in range(n_splits):
                 items.append([row0s[i], 1, head0, nh, sp, n_splits, slot, seg_cap])
             slot += seg_cap
-    plan = AttentionPlan(shared, items, merges, slot, device)
+    plan = AttentionPlan(shared, items, merges, slot, device, seg_cap)
     if len(_PLAN_CACHE) > 256:
         _PLAN_CACHE.clear()
     _PLAN_CACHE[key] = plan
@@ -448,7 +450,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                                plan.n_items - plan.n_shared - plan.n_direct,
                                                _dev(plan.merges, "merges", torch.int32), plan.n_merges, _dev(out, "out"),
                                                _dev(part_o, "part_o"), _dev(part_ml, "part_ml"), float(scale), n_heads, n_kv_heads,
-                                               head_dim, page_tokens, tables.shape[1], int(window), 1 if plan.wide_items else 0, _stream()),
+                                               head_dim, page_tokens, tables.shape[1], int(window), (1 if plan.wide_items else 0) | (2 if plan.short_merge else 0), _stream()),
                "paged_attention_mfma")
         return
     _check(lib().llmx_paged_attention_generic(*common, _dev(out, "out"), _code(q.dtype), float(scale), rows, n_heads, n_kv_heads,

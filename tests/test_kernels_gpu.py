@@ -646,6 +646,77 @@ def test_decoding_items_worked_on_by_four_waves_give_the_bits_of_one_wave(contex
         assert (outs[0][i, h * D:(h + 1) * D].double() - want).abs().max() <= 1.2e-2 * want.abs().max() + 2e-4
 
 
+MERGE_CASES = [
+    ((1, 130, 517, 2000, 64, 129, 4100, 8300, 4097), 12, 2, 128, 0),     # few columns, up to 65 segments
+    ((3000, 129, 8191), 8, 2, 128, 0),                                   # few short columns
+    (tuple(300 + 181 * i for i in range(20)), 12, 4, 128, 0),            # many short columns
+    (tuple(200 + 5 * i for i in range(130)), 12, 4, 128, 0),             # a crowd of short columns: every thread keeps the sum itself
+    (tuple(9000 - 37 * i for i in range(17)), 12, 4, 128, 0),            # many columns of more than 64 segments
+    ((70000,), 3, 1, 48, 0), ((33000, 900, 41111), 8, 8, 64, 20000), ((66000, 12345), 2, 2, 112, 0),
+    ((131072 + 515,), 6, 1, 128, 0),                                     # more than 1,024 segments: three chunks of weights
+    ((5000, 300), 4, 2, 256, 0), (tuple(600 + 7 * i for i in range(25)), 4, 1, 256, 0), ((9000, 8000, 140), 2, 1, 160, 0),
+]
+
+
+@pytest.mark.parametrize("contexts,Hq,Hkv,D,window", MERGE_CASES)
+def test_merged_columns_give_the_bits_of_an_item_that_walks_its_context(contexts, Hq, Hkv, D, window):
+    """The merge of a column's segments, by workgroups of 128 or of 64 dims (few long columns) and with all its loads asked
+    for at once (no column above 64 segments) or round by round: the bits of one item per KV head walking the context, for
+    columns of 1 segment up to more than 1,024, counts that end anywhere in a round of 32, a window, head sizes up to
+    256; and the launch says which form ran."""
+    o = ops()
+    page = 16
+    n = len(contexts)
+    blocks = [-(-c // page) for c in contexts]
+    order = list(range(sum(blocks)))
+    random.Random(n + D).shuffle(order)
+    table = torch.full((n, max(blocks)), -1, dtype=torch.int32)
+    at = 0
+    for i, b in enumerate(blocks):
+        table[i, :b] = torch.tensor(order[at:at + b])
+        at += b
+    table = table.to(DEV)
+    k_cache = rnd(sum(blocks), Hkv, page, D, dtype=torch.bfloat16, scale=0.5)
+    v_cache = rnd(sum(blocks), Hkv, D, page, dtype=torch.bfloat16, seed=2)
+    q = rnd(n, Hq * D, dtype=torch.bfloat16, seed=3)
+    pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device=DEV)
+    ent = torch.arange(n, dtype=torch.int32, device=DEV)
+    outs = []
+    saved = o.ATTENTION_TARGET_WAVES
+    for target in (100000, 1):
+        o.ATTENTION_TARGET_WAVES = target
+        o._PLAN_CACHE.clear()
+        try:
+            plan = o.attention_plan([1] * n, list(contexts), Hq, Hkv, DEV, window)
+        finally:
+            o.ATTENTION_TARGET_WAVES = saved
+        assert plan.n_merges == (n * Hq if target > 1 else 0)
+        out = torch.zeros(n, Hq * D, dtype=torch.bfloat16, device=DEV)
+        o.take_launches()
+        o.paged_attention(q, k_cache, v_cache, pos, ent, table, out, 1.0 / math.sqrt(D), Hq, window, plan=plan)
+        ran = o.take_launches()
+        if target > 1:
+            longest = min(max(contexts), window + 128) if window else max(contexts)
+            assert plan.short_merge == (-(-(-(-longest // 128) + 1) // 8) * 8 <= 64)
+            narrow = not plan.short_merge and n * Hq * -(-D // 128) <= 192
+            assert ran.get("attention.merge_narrow", 0) == (1 if narrow else 0) and ran.get("attention.merge", 0) == (0 if narrow else 1)
+        else:
+            assert not ran.get("attention.merge_narrow", 0) and not ran.get("attention.merge", 0)
+        outs.append(out)
+    o._PLAN_CACHE.clear()
+    assert torch.equal(outs[0], outs[1])
+    for i, c in enumerate(contexts):       # and the plain softmax for one head of every row
+        pages = table[i, :blocks[i]].long()
+        keys = k_cache[pages].permute(1, 0, 2, 3).reshape(Hkv, -1, D)[:, :c].double()
+        values = v_cache[pages].permute(1, 0, 3, 2).reshape(Hkv, -1, D)[:, :c].double()
+        lo = max(0, c - window) if window else 0
+        h = (i * 5) % Hq
+        kv = h // (Hq // Hkv)
+        w = torch.softmax((keys[kv, lo:] @ q[i, h * D:(h + 1) * D].double()) / math.sqrt(D), dim=0)
+        want = w @ values[kv, lo:]
+        assert (outs[0][i, h * D:(h + 1) * D].double() - want).abs().max() <= 1.2e-2 * want.abs().max() + 2e-4
+
+
 @pytest.mark.parametrize("L,Hq,Hkv,D", [(70000, 2, 1, 32), (66000, 4, 2, 160)])
 def test_attention_very_long_context(L, Hq, Hkv, D):
     """A decoded row over more than 512 segments of keys (the merge works through them in several rounds): the same bits
