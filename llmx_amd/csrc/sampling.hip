@@ -945,10 +945,32 @@ __device__ bool ranked_find(int n, KeyFn key, WeightFn weight, unsigned long lon
     }
 }
 
+// A token's weight as a fixed-point number: exp((score - best) / temp) * scale; a score equal to an infinite best
+// (inf - inf) weighs 1 like the best itself, and a NaN (which takes no part anyway) weighs 0, so that no NaN is ever
+// turned into an integer.
+__device__ __forceinline__ float ranked_rel_weight(float v, float best_score, float tmp) {
+    if (v != v) return 0.0f;
+    const float d = v - best_score;
+    return d != d ? 1.0f : expf(d / tmp);
+}
+// The weights' scale for rows of n tokens: a row's sum stays below 2^62.
+__device__ __forceinline__ double ranked_scale(int n) {
+    int scale_bits = 62;
+    while ((1ll << (62 - scale_bits)) < (long long)n) --scale_bits;
+    return (double)(1ull << scale_bits);
+}
+
+// ITEMS: the row's tokens are those of `items` (stage 2 of the search by slices, see ranked_slices_kernel) and
+// the weight of the whole row comes from the slices' sums; a row this stage cannot finish (a top_k, no nucleus, or a
+// nucleus that reaches past what the candidates are certain to hold) gets its flag set and is left to the kernel over
+// the whole row, which with `flags` takes only such rows.
+template <bool ITEMS>
 __global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const float* __restrict__ scores, const float* __restrict__ temp,
                                                                       const int* __restrict__ top_k, const float* __restrict__ top_p,
                                                                       const float* __restrict__ min_p, const float* __restrict__ unit,
-                                                                      const int* __restrict__ skip, int* __restrict__ out, int n) {
+                                                                      const int* __restrict__ skip, int* __restrict__ out, int n,
+                                                                      const int* __restrict__ items, int per_slice, int n_slices,
+                                                                      const unsigned long long* __restrict__ slice_sums, int* __restrict__ flags) {
     __shared__ RankedShared sh;
     const int r = blockIdx.x, tid = threadIdx.x;
     const float* s = scores + (size_t)r * n;
@@ -957,42 +979,54 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const flo
     int keep = top_k[r];
     if (keep <= 0 || keep > m) keep = m;
     const float tmp = temp[r], p = top_p[r], cut = min_p ? min_p[r] : 0.0f;
-    if (!(tmp > 0.0f)) return;   // a greedy row is not this kernel's: its entry of `out` is not written
+    if (!(tmp > 0.0f)) {   // a greedy row is not this kernel's: its entry of `out` is not written
+        if (ITEMS && tid == 0) flags[r] = 0;
+        return;
+    }
+    if (ITEMS) {
+        if (keep < m || p >= 1.0f) {   // not a nucleus over the whole row
+            if (tid == 0) flags[r] = 1;
+            return;
+        }
+    } else if (flags && !flags[r]) {
+        return;
+    }
+    const int count = ITEMS ? per_slice * n_slices : n;
+    const int* mine_items = ITEMS ? items + (size_t)r * count : nullptr;
+    auto id_of = [&](int j) -> int { return ITEMS ? mine_items[j] : j; };
     const unsigned long long all_lo = 1ull, all_hi = ~0ull;
     // a NaN score takes no part, like the masked token (the arg-max never lets a NaN lead either)
-    auto key_of = [&](int i) -> unsigned long long {
+    auto key_of = [&](int j) -> unsigned long long {
+        const int i = id_of(j);
+        if (i < 0 || i == sk) return 0ull;
         const float v = s[i];
-        return i == sk || v != v ? 0ull : rank_key(v, i);
+        return v != v ? 0ull : rank_key(v, i);
     };
 
     // the best token: the largest key
     unsigned long long top = 0;
-    for (int i = tid; i < n; i += SAMPLE_THREADS) {
-        const unsigned long long k = key_of(i);
+    for (int j = tid; j < count; j += SAMPLE_THREADS) {
+        const unsigned long long k = key_of(j);
         top = k > top ? k : top;
     }
     top = block_max_u64(top, sh.wave_q);
     if (top == 0ull) {   // nothing takes part (every score a NaN): the first id that is not masked, as the arg-max gives
-        if (tid == 0) out[r] = sk == 0 && n > 1 ? 1 : 0;
+        if (tid == 0) {
+            if (ITEMS) flags[r] = 1;
+            else out[r] = sk == 0 && n > 1 ? 1 : 0;
+        }
         return;
     }
     const int best = (int)(0xFFFFFFFFu - (uint32_t)top);
     const float best_score = s[best];
-    // fixed-point weights: a row's sum stays below 2^62
-    int scale_bits = 62;
-    while ((1ll << (62 - scale_bits)) < (long long)n) --scale_bits;
-    const double scale = (double)(1ull << scale_bits);
-    // exp((score - best) / temp); a score equal to an infinite best (inf - inf) weighs 1 like the best itself, and a
-    // NaN (which takes no part anyway) weighs 0, so that no NaN is ever turned into an integer
-    auto rel_weight = [&](int i) -> float {
-        const float v = s[i];
-        if (v != v) return 0.0f;
-        const float d = v - best_score;
-        return d != d ? 1.0f : expf(d / tmp);
+    const double scale = ranked_scale(n);
+    auto rel_weight = [&](int j) -> float {
+        const int i = id_of(j);
+        return i < 0 ? 0.0f : ranked_rel_weight(s[i], best_score, tmp);
     };
-    auto weight_of = [&](int i) -> unsigned long long { return (unsigned long long)((double)rel_weight(i) * scale); };
-    auto cut_weight_of = [&](int i) -> unsigned long long {
-        const float w = rel_weight(i);
+    auto weight_of = [&](int j) -> unsigned long long { return (unsigned long long)((double)rel_weight(j) * scale); };
+    auto cut_weight_of = [&](int j) -> unsigned long long {
+        const float w = rel_weight(j);
         return w < cut ? 0ull : (unsigned long long)((double)w * scale);
     };
 
@@ -1000,10 +1034,10 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const flo
     unsigned long long kept_from = all_lo, unused;
     if (keep < m) {
         auto one = [&](int) -> unsigned long long { return 1ull; };
-        if (!ranked_find(n, key_of, one, all_lo, all_hi, (unsigned long long)keep, sh, &kept_from, &unused)) kept_from = all_lo;
+        if (!ranked_find(count, key_of, one, all_lo, all_hi, (unsigned long long)keep, sh, &kept_from, &unused)) kept_from = all_lo;
     }
-    auto kept_key = [&](int i) -> unsigned long long {
-        const unsigned long long k = key_of(i);
+    auto kept_key = [&](int j) -> unsigned long long {
+        const unsigned long long k = key_of(j);
         return k >= kept_from ? k : 0ull;
     };
 
@@ -1011,47 +1045,148 @@ __global__ void __launch_bounds__(SAMPLE_THREADS) sample_ranked_kernel(const flo
     if (p >= 1.0f) {
         // no nucleus: the draw walks the kept tokens in id order, weights below min_p counting 0 (sampler.hpp:341-352)
         unsigned long long mine = 0;
-        for (int i = tid; i < n; i += SAMPLE_THREADS)
-            if (kept_key(i)) mine += cut_weight_of(i);
+        for (int j = tid; j < count; j += SAMPLE_THREADS)
+            if (kept_key(j)) mine += cut_weight_of(j);
         const unsigned long long total = block_sum_u64(mine, sh.wave_q);
         const unsigned long long goal = (unsigned long long)floor((double)unit[r] * (double)total) + 1ull;
-        auto id_order = [&](int i) -> unsigned long long { return kept_key(i) ? (unsigned long long)(0xFFFFFFFFu - (uint32_t)i) + 1ull : 0ull; };
+        auto id_order = [&](int j) -> unsigned long long { return kept_key(j) ? (unsigned long long)(0xFFFFFFFFu - (uint32_t)id_of(j)) + 1ull : 0ull; };
         unsigned long long at = 0;
-        if (ranked_find(n, id_order, cut_weight_of, all_lo, 1ull << 32, goal, sh, &at, &unused)) pick = (int)(0xFFFFFFFFu - (uint32_t)(at - 1ull));
+        if (ranked_find(count, id_order, cut_weight_of, all_lo, 1ull << 32, goal, sh, &at, &unused)) pick = (int)(0xFFFFFFFFu - (uint32_t)(at - 1ull));
     } else {
         // the nucleus: the shortest ranked prefix of the kept set whose weight reaches top_p of the kept weight (:354-363)
-        unsigned long long mine = 0;
-        for (int i = tid; i < n; i += SAMPLE_THREADS)
-            if (kept_key(i)) mine += weight_of(i);
-        const unsigned long long total = block_sum_u64(mine, sh.wave_q);
+        unsigned long long total;
+        unsigned long long certain_from = all_lo;   // every token of the row with a key from here up is among the items
+        if (ITEMS) {
+            total = 0;
+            for (int sl = 0; sl < n_slices; ++sl) total += slice_sums[(size_t)r * n_slices + sl];
+            // a slice that filled its list may hold better tokens than its list's worst outside it; none as good
+            unsigned long long from = all_lo;
+            for (int sl = tid >> 6; sl < n_slices; sl += SAMPLE_WAVES) {
+                if (mine_items[(size_t)sl * per_slice + per_slice - 1] < 0) continue;   // the list has room left: the slice is all there
+                unsigned long long worst = ~0ull;
+                for (int c = tid & 63; c < per_slice; c += 64) {
+                    const unsigned long long k = key_of(sl * per_slice + c);
+                    if (k != 0ull && k < worst) worst = k;
+                }
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) {
+                    const unsigned long long other = __shfl_xor(worst, o, 64);
+                    worst = other < worst ? other : worst;
+                }
+                from = worst > from ? worst : from;
+            }
+            certain_from = block_max_u64(from, sh.wave_q);
+        } else {
+            unsigned long long mine = 0;
+            for (int j = tid; j < count; j += SAMPLE_THREADS)
+                if (kept_key(j)) mine += weight_of(j);
+            total = block_sum_u64(mine, sh.wave_q);
+        }
         unsigned long long goal = (unsigned long long)ceil((double)p * (double)total);
         if (goal < 1ull) goal = 1ull;   // the nucleus holds at least the best token
         unsigned long long nucleus_from = kept_from;
-        if (!ranked_find(n, kept_key, weight_of, all_lo, all_hi, goal, sh, &nucleus_from, &unused)) nucleus_from = kept_from;
+        const bool reached = ranked_find(count, kept_key, weight_of, all_lo, all_hi, goal, sh, &nucleus_from, &unused);
+        if (ITEMS) {
+            // the running weight down to the nucleus' last token is the row's only if every better token is an item
+            const bool certain = reached && nucleus_from >= certain_from;
+            if (tid == 0) flags[r] = certain ? 0 : 1;
+            if (!certain) return;
+        } else if (!reached) {
+            nucleus_from = kept_from;
+        }
         // min_p cuts the nucleus' tail: weights fall along the ranking, so that is every weight below it (:364-372)
-        auto nucleus_key = [&](int i) -> unsigned long long {
-            const unsigned long long k = key_of(i);
+        auto nucleus_key = [&](int j) -> unsigned long long {
+            const unsigned long long k = key_of(j);
             if (k < nucleus_from) return 0ull;
-            return (cut > 0.0f && rel_weight(i) < cut) ? 0ull : k;
+            return (cut > 0.0f && rel_weight(j) < cut) ? 0ull : k;
         };
-        mine = 0;
-        for (int i = tid; i < n; i += SAMPLE_THREADS)
-            if (nucleus_key(i)) mine += weight_of(i);
+        unsigned long long mine = 0;
+        for (int j = tid; j < count; j += SAMPLE_THREADS)
+            if (nucleus_key(j)) mine += weight_of(j);
         const unsigned long long nucleus_weight = block_sum_u64(mine, sh.wave_q);
         const unsigned long long target = (unsigned long long)floor((double)unit[r] * (double)nucleus_weight) + 1ull;
         unsigned long long at = 0;
-        if (ranked_find(n, nucleus_key, weight_of, all_lo, all_hi, target, sh, &at, &unused)) pick = (int)(0xFFFFFFFFu - (uint32_t)at);
+        if (ranked_find(count, nucleus_key, weight_of, all_lo, all_hi, target, sh, &at, &unused)) pick = (int)(0xFFFFFFFFu - (uint32_t)at);
     }
     if (tid == 0) out[r] = pick;
 }
 
+// Stage 1 of the nucleus over a wide row by many workgroups (after argmax_slices_kernel has left the slices' leaders):
+// workgroup (slice, row) merges the leaders (the row's best score is what the weights are taken against), adds up its
+// slice's weights (integers: any order) and keeps the RANKED_SLICE_KEEP best of its slice in id order, -1 where it has
+// fewer.  Whatever the row's nucleus holds of the slice is among them, unless the slice's list is full and the nucleus
+// reaches past its worst entry: stage 2 tells.
+#define RANKED_SLICE_KEEP 256
+__global__ void __launch_bounds__(SAMPLE_THREADS) ranked_slices_kernel(const float* __restrict__ scores, const float* __restrict__ temp,
+                                                                      const int* __restrict__ skip, const Leader* __restrict__ partial,
+                                                                      unsigned long long* __restrict__ slice_sums, int* __restrict__ cand,
+                                                                      int n, int n_slices) {
+    __shared__ TopkShared sh;
+    __shared__ unsigned long long wave_q[SAMPLE_WAVES];
+    __shared__ int best_s;
+    const int r = blockIdx.y, sl = blockIdx.x, tid = threadIdx.x;
+    const float tmp = temp[r];
+    if (!(tmp > 0.0f)) return;   // a greedy row has no nucleus
+    const float* s = scores + (size_t)r * n;
+    const int sk = skip ? (skip[r] >= 0 && skip[r] < n && n > 1 ? skip[r] : n) : n;
+    if (tid < 64) {
+        const int best = merged_leader(s, partial + (size_t)r * n_slices, n_slices, n, sk);
+        if (tid == 0) best_s = best;
+    }
+    __syncthreads();
+    const float best_score = s[best_s];
+    const double scale = ranked_scale(n);
+    const int begin = sl * ARGMAX_SLICE, count = max(0, min(n, begin + ARGMAX_SLICE) - begin);
+    unsigned long long mine = 0;
+    for (int c = tid; c < count; c += SAMPLE_THREADS) {
+        const int id = begin + c;
+        if (id != sk) mine += (unsigned long long)((double)ranked_rel_weight(s[id], best_score, tmp) * scale);
+    }
+    const unsigned long long total = block_sum_u64(mine, wave_q);
+    if (tid == 0) slice_sums[(size_t)r * n_slices + sl] = total;
+    int* list = cand + ((size_t)r * n_slices + sl) * RANKED_SLICE_KEEP;
+    const int kept = select_topk(s, count, [&](int c) {
+                                     const int id = begin + c;
+                                     const float v = s[id];
+                                     return id == sk || v != v ? -1 : id; },
+                                 RANKED_SLICE_KEEP, [&](int place, int id, float) { list[place] = id; }, sh);
+    for (int i = kept + tid; i < RANKED_SLICE_KEEP; i += SAMPLE_THREADS) list[i] = -1;
+}
+
+// Bytes of scratch llmx_sample_ranked wants for rows of n scores (0: a row is narrow enough for one workgroup).
+extern "C" long llmx_sample_ranked_scratch(int rows, int n) {
+    if (n <= 2 * ARGMAX_SLICE || rows <= 0) return 0;
+    const long n_slices = (n + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
+    return (long)rows * n_slices * (long)(sizeof(Leader) + sizeof(unsigned long long) + RANKED_SLICE_KEEP * sizeof(int)) + (long)rows * sizeof(int);
+}
+
 // Rows with any top_k (0 or above the row keeps every token) and any top_p; the sampler sends here the rows that
 // llmx_sample_topk (kept sets of at most 1,024, ranked exactly) and llmx_sample_all (everything kept, no nucleus) do not take.
+// scratch: llmx_sample_ranked_scratch(rows, n) bytes, 8-byte aligned, or null.  With it a nucleus over a whole wide row
+// is looked for among the best of every slice of 8,192 scores, found by many workgroups; the rows whose nucleus is not
+// certain to lie among those (and the rows with a top_k) are then walked whole by one workgroup each, as all rows are
+// without scratch.  The token is the same either way.
 extern "C" int llmx_sample_ranked(const float* scores, const float* temp, const int* top_k, const float* top_p, const float* min_p,
-                                  const float* unit, const int* skip, int* out, int rows, int n, hipStream_t stream) {
+                                  const float* unit, const int* skip, int* out, int rows, int n, void* scratch, hipStream_t stream) {
     if (rows <= 0) return 0;
     llmx_note_launch(LK_SAMPLE_RANKED);
     if (n <= 0 || n > (1 << 30)) return -2;
-    hipLaunchKernelGGL(sample_ranked_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n);
+    int* flags = nullptr;
+    if (scratch && n > 2 * ARGMAX_SLICE) {
+        if (rows > 65535 || ((uintptr_t)scratch & 7)) return -2;
+        const int n_slices = (n + ARGMAX_SLICE - 1) / ARGMAX_SLICE;
+        unsigned long long* sums = (unsigned long long*)scratch;
+        Leader* partial = (Leader*)(sums + (size_t)rows * n_slices);
+        int* cand = (int*)(partial + (size_t)rows * n_slices);
+        flags = cand + (size_t)rows * n_slices * RANKED_SLICE_KEEP;
+        llmx_note_launch(LK_SAMPLE_RANKED_SLICES);
+        hipLaunchKernelGGL(argmax_slices_kernel, dim3(n_slices, rows), dim3(256), 0, stream, scores, skip, partial, n, n_slices);
+        hipLaunchKernelGGL(ranked_slices_kernel, dim3(n_slices, rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, skip, (const Leader*)partial, sums,
+                           cand, n, n_slices);
+        hipLaunchKernelGGL(sample_ranked_kernel<true>, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n,
+                           (const int*)cand, RANKED_SLICE_KEEP, n_slices, (const unsigned long long*)sums, flags);
+    }
+    hipLaunchKernelGGL(sample_ranked_kernel<false>, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, scores, temp, top_k, top_p, min_p, unit, skip, out, n,
+                       (const int*)nullptr, 0, 0, (const unsigned long long*)nullptr, flags);
     return LLMX_CHECK_LAUNCH();
 }

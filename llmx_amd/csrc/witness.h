@@ -46,6 +46,7 @@
     X(SAMPLE_ALL, "sample_all")                                                                                           \
     X(SAMPLE_TOPK, "sample_topk")                                                                                         \
     X(SAMPLE_RANKED, "sample_ranked")                                                                                     \
+    X(SAMPLE_RANKED_SLICES, "sample_ranked.slices")                                                                       \
     X(PENALIZE, "penalize")
 
 enum LlmxLaunchKind : int {

@@ -76,7 +76,7 @@ def _declare(h) -> None:
         "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P, I, P],
-        "llmx_sample_ranked": [P, P, P, P, P, P, P, P, I, I, P],
+        "llmx_sample_ranked": [P, P, P, P, P, P, P, P, I, I, P, P],
         "llmx_penalize": [P, P, P, P, P, P, P, I, I, P],
     }
     sigs.update({"llmx_note_launch": [I], "llmx_launch_kinds": [], "llmx_launch_name": [I], "llmx_take_launches": [P, I]})
@@ -91,6 +91,8 @@ def _declare(h) -> None:
     h.llmx_sample_topk_scratch.restype = c_long
     h.llmx_sample_all_scratch.argtypes = [I, I]
     h.llmx_sample_all_scratch.restype = c_long
+    h.llmx_sample_ranked_scratch.argtypes = [I, I]
+    h.llmx_sample_ranked_scratch.restype = c_long
     h.llmx_launch_name.restype = ctypes.c_char_p
     h.llmx_note_launch.restype = None
 
@@ -644,14 +646,24 @@ def sample_topk(scores: torch.Tensor, temp: torch.Tensor, top_k: torch.Tensor, t
 
 
 def sample_ranked(scores: torch.Tensor, temp: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, min_p: torch.Tensor,
-                  unit: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Tensor] = None) -> None:
-    """Top-k of any size (0 keeps all), top-p, min-p and the draw, without sorting; rows with temp <= 0 are left unwritten."""
+                  unit: torch.Tensor, out: torch.Tensor, skip: Optional[torch.Tensor] = None, slices: bool = True) -> Optional[torch.Tensor]:
+    """Top-k of any size (0 keeps all), top-p, min-p and the draw, without sorting; rows with temp <= 0 are left unwritten.
+    A nucleus over a whole row of many scores is looked for among the best 256 of every slice of 8,192 scores, which many
+    workgroups find; a row whose nucleus is not certain to lie among them (or that has a top_k) is then walked whole by
+    one workgroup, as every row is with `slices=False`.  The token is the same either way.  Returns, when the search by
+    slices ran, a device tensor with 1 for every row that was walked whole after it (a view of scratch the next call
+    overwrites), else None."""
     rows, n = scores.shape
+    need = lib().llmx_sample_ranked_scratch(rows, n) if slices else 0
+    scratch = _scratch("sample_ranked.slices", -(-need // 8), torch.float64, scores.device) if need else None
     _check(lib().llmx_sample_ranked(_dev(scores, "scores", torch.float32), _dev(temp, "temp", torch.float32, (rows,)),
                                     _dev(top_k, "top_k", torch.int32, (rows,)), _dev(top_p, "top_p", torch.float32, (rows,)),
                                     _dev(min_p, "min_p", torch.float32, (rows,)), _dev(unit, "unit", torch.float32, (rows,)),
-                                    _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n, _stream()),
-           "sample_ranked")
+                                    _dev(skip, "skip", torch.int32, (rows,)), _dev(out, "out", torch.int32, (rows,)), rows, n,
+                                    _dev(scratch, "scratch"), _stream()), "sample_ranked")
+    if scratch is None:
+        return None
+    return scratch.view(torch.int32)[need // 4 - rows:need // 4]
 
 
 def penalize(scores: torch.Tensor, rows: torch.Tensor, ids: torch.Tensor, counts: torch.Tensor, penalty: torch.Tensor,

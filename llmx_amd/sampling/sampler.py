@@ -68,7 +68,7 @@ class Sampler:
             ops.sample_topk(logits, temp, st["top_k"], st["top_p"], min_p, unit, results["topk"], skip, max_keep=st["max_keep"])
         if "ranked" in which:
             results["ranked"] = torch.zeros(W, dtype=torch.int32, device=self.device)
-            ops.sample_ranked(logits, temp, st["top_k"], st["top_p"], min_p, unit, results["ranked"], skip)
+            ops.sample_ranked(logits, temp, st["top_k"], st["top_p"], min_p, unit, results["ranked"], skip, slices=st["nucleus_rows"])
         if len(results) == 1:
             return next(iter(results.values())).tolist()
         lists = {name: t.tolist() for name, t in results.items()}
@@ -102,5 +102,7 @@ class Sampler:
                 st["top_k"], st["top_p"] = self._i32([p.top_k for p in params]), self._f32([p.top_p for p in params])
                 # the largest top_k among the rows the exact kernel takes: it sizes that kernel's candidate lists
                 st["max_keep"] = max([p.top_k for p, w in zip(params, st["which"]) if w == "topk"] or [1])
+                # a nucleus over a whole row is first looked for by slices; a top-k above what is ranked whole never is
+                st["nucleus_rows"] = any(w == "ranked" and (p.top_k <= 0 or p.top_k >= mr) for p, w, mr in zip(params, st["which"], m))
         self._kept = (key, st)
         return st

@@ -1110,6 +1110,82 @@ def test_temperature_draw_by_slices_gives_the_token_of_one_workgroup(V):
     assert int(sliced[2]) == int(host[2].argmax()) and len(seen) > 100
 
 
+@pytest.mark.parametrize("V", [16385, 50000, 200064])
+def test_nucleus_searched_by_slices_gives_the_token_of_one_workgroup(V):
+    """A nucleus over a whole wide row is looked for among the 256 best of every slice of 8,192 scores; rows it cannot
+    be certain of are walked whole afterwards.  Every token must be the one the walk over the whole row gives, and the
+    rows must be told apart rightly: a peaked row is finished by the slices, a flat row is not, and neither is a row whose
+    nucleus needs more of one slice than the slice's list holds (the case a wrong bound would get wrong), while a smaller
+    nucleus in that same row is.  With ties across slices, a masked best token, min_p, NaN and infinite scores, a greedy
+    row and a row with a top_k."""
+    o = ops()
+    from llmx_amd.sampling import XorShift64
+    g = torch.Generator().manual_seed(V)
+    rows = 11
+    logits = torch.randn(rows, V, generator=g)
+    head = torch.randperm(V, generator=g)[:30]
+    logits[0, head] += torch.linspace(8.0, 12.0, 30)                 # 0: thirty tokens hold nearly all the weight
+    ranks = torch.randperm(V, generator=g).float() + 1.0
+    logits[1] = -1.2 * torch.log(ranks)                              # 1: a long tail
+    logits[2] *= 2.0                                                 # 2: flat
+    logits[3] = -20.0 + 0.01 * torch.randn(V, generator=g)           # 3, 4: 400 good tokens, all inside the second slice
+    logits[3, 8300:8700] = 5.0 + 0.5 * torch.randn(400, generator=g)
+    logits[4] = logits[3]
+    logits[5] = torch.round(logits[0] * 2.0) / 2.0                   # 5: ties, also across slices
+    logits[6] = logits[0]                                            # 6: the best token masked, min_p
+    logits[7] = logits[0]                                            # 7: greedy
+    logits[8] = logits[0]                                            # 8: a top_k above what is ranked whole
+    logits[9] = logits[0]                                            # 9: NaN and infinite scores
+    logits[9, head[:3]] = float("nan")
+    logits[9, head[3]] = float("inf")
+    logits[9, V - 1] = float("inf")
+    logits[10] = logits[0]                                           # 10: a nucleus of one token
+    settings = [dict(temp=0.9, top_k=0, top_p=0.9, min_p=0.0), dict(temp=1.0, top_k=0, top_p=0.9, min_p=0.0),
+                dict(temp=1.0, top_k=0, top_p=0.9, min_p=0.0), dict(temp=1.0, top_k=0, top_p=0.95, min_p=0.0),
+                dict(temp=1.0, top_k=0, top_p=0.3, min_p=0.0), dict(temp=0.7, top_k=0, top_p=0.99, min_p=0.0),
+                dict(temp=1.1, top_k=0, top_p=0.8, min_p=0.05), dict(temp=0.0, top_k=0, top_p=0.9, min_p=0.0),
+                dict(temp=1.0, top_k=5000, top_p=0.9, min_p=0.0), dict(temp=1.0, top_k=0, top_p=0.9, min_p=0.0),
+                dict(temp=0.3, top_k=0, top_p=0.01, min_p=0.0)]
+    skip_ids = [-1] * rows
+    skip_ids[6] = int(logits[6].argmax())
+    host = logits.clone()
+    logits = logits.to(DEV)
+    skip = torch.tensor(skip_ids, dtype=torch.int32, device=DEV)
+    f = lambda key: torch.tensor([s[key] for s in settings], dtype=torch.float32, device=DEV)
+    top_k = torch.tensor([s["top_k"] for s in settings], dtype=torch.int32, device=DEV)
+    rng = XorShift64(V + 5)
+    seen = [set() for _ in range(rows)]
+    for draw in range(40):
+        units = [rng.unit() for _ in range(rows)]
+        if draw == 0:
+            units[0], units[1] = 0.0, 1.0 - 2.0 ** -24
+        unit = torch.tensor(units, dtype=torch.float32, device=DEV)
+        whole = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        sliced = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        assert o.sample_ranked(logits, f("temp"), top_k, f("top_p"), f("min_p"), unit, whole, skip, slices=False) is None
+        o.take_launches()
+        left = o.sample_ranked(logits, f("temp"), top_k, f("top_p"), f("min_p"), unit, sliced, skip)
+        assert o.take_launches().get("sample_ranked.slices", 0) == 1
+        assert sliced.tolist() == whole.tolist(), f"draw {draw}: by slices {sliced.tolist()}, whole {whole.tolist()}"
+        left = left.tolist()
+        assert [left[r] for r in (0, 2, 3, 4, 7, 8, 10)] == [0, 1, 1, 0, 0, 1, 0], left
+        for r, t in enumerate(whole.tolist()):
+            seen[r].add(t)
+    assert seen[7] == {-1} and len(seen[0]) > 5 and len(seen[4]) > 20 and len(seen[10]) == 1
+    assert not seen[9] & set(head[:3].tolist()) and seen[9] <= {int(head[3]), V - 1}
+    assert skip_ids[6] not in seen[6]
+    # and the reference's own token for the rows the slices finished
+    for r in (0, 4, 5, 6):
+        ref = sampler_reference.prepare(host[r].tolist(), settings[r]["temp"], 0, settings[r]["top_p"], settings[r]["min_p"],
+                                        skip=skip_ids[r] if skip_ids[r] >= 0 else None)
+        rng = XorShift64(r + 1)
+        for _ in range(12):
+            u = rng.unit()
+            out = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+            o.sample_ranked(logits, f("temp"), top_k, f("top_p"), f("min_p"), torch.full((rows,), u, dtype=torch.float32, device=DEV), out, skip)
+            assert int(out[r]) == ref(u)
+
+
 def test_ranked_sampler_over_the_whole_vocabulary_200_draws():
     """The search by histograms forms its sums in 64-bit fixed point where the reference sums doubles: 200 draws a row at
     the real vocabulary (a nucleus over the whole row; a top-k of 5,000; a nucleus with min_p inside a top-k of 50,000),
