@@ -28,6 +28,7 @@ enum : int { TL_STORE = 0, TL_ADD = 1, TL_SWIGLU = 2 };
 #define TL_BN 128
 #define TL_BK 64
 #define TL_LD 72  // padded row length in bf16 elements (144 bytes)
+#define TILE_RUNS_APART_BELOW 256   // dense products with fewer 64 x 128 tiles than this multiply K's runs in workgroups of their own (measured: 8,192 features up to 192 rows, 3,072 features of K 6,144 up to 640 rows)
 #define TL_STAGES 2  // tiles in LDS in the lean loop: one being multiplied, the other on its way (48 KB: three workgroups a CU; measured better than deeper stages with fewer workgroups)
 
 // Lane l of the wave: 16 bytes from base + offset (bytes, per lane) to LDS at lds + 16 l (lds the same for the whole
@@ -83,6 +84,7 @@ struct TileArgs {
     int bm;       // rows a workgroup covers: 64 or 128
     const int* tile_stats;  // grouped, optional: [0] = sum over groups of ceil(rows / 128)
     int run_if_big;         // with tile_stats: 1: this launch works only if the groups fill 128-row tiles, 0: only if not
+    int run_tiles;          // dense lean form, > 0: workgroup z multiplies only K's run z (this many 64-wide tiles) and stores its sums at C + z * M * ldc
 };
 
 // Whether the groups' rows fill tiles of 128 rows well enough: the tiles hold at most 1.6 times the rows (measured on
@@ -262,7 +264,9 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
         // c ^ ((r >> 1) & 7) of the row, so that the operand reads of 16 rows at one k fall into different banks.  The
         // lane that fills place p of row r therefore fetches chunk p ^ ((r >> 1) & 7) of that row.
         constexpr int A_LOADS = BM / 32, LOADS = 4 + A_LOADS;   // load instructions a wave issues per tile
-        const int n_tiles = K / TL_BK;
+        // the 64-wide tiles of K this workgroup multiplies: all of them, or one run's (run_tiles > 0: the runs lie apart)
+        const int t_first = g.run_tiles > 0 ? (int)blockIdx.z * g.run_tiles : 0;
+        const int n_tiles = g.run_tiles > 0 ? min(K / TL_BK, t_first + g.run_tiles) : K / TL_BK;
         const int tiles_per_run = SPLIT ? per / 2 : n_tiles;
         uint32_t w_at[4], a_at[A_LOADS];
         const int place = lane & 7;
@@ -335,11 +339,11 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
             }
             __builtin_amdgcn_sched_group_barrier(0x008, 8 * TT - (4 + TT), 0);
         };
-        issue(0, 0);
+        issue(t_first, 0);
 #pragma unroll
         for (int ahead = 1; ahead < STAGES - 1; ++ahead)
-            if (ahead < n_tiles) issue(ahead, ahead);
-        int t = 0, stage = 0;
+            if (t_first + ahead < n_tiles) issue(t_first + ahead, ahead);
+        int t = t_first, stage = 0;
         for (int run_end = tiles_per_run;; run_end += tiles_per_run) {
             const int stop = min(run_end, n_tiles);
             for (; t < stop; ++t) {
@@ -428,7 +432,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(TileArgs g) {
     for (int t = 0; t < TT; ++t) {
         const int rc = rows_c[BM / 2 * wm + 16 * t + lr];
         if (rc < 0) continue;
-        TC* crow = (TC*)g.C + (size_t)rc * g.ldc;
+        TC* crow = (TC*)g.C + (size_t)rc * g.ldc + (g.run_tiles > 0 ? (size_t)blockIdx.z * g.M * g.ldc : 0);
         if (EPI == TL_SWIGLU) {
 #pragma unroll
             for (int f = 0; f < 2; ++f) {
@@ -766,6 +770,33 @@ extern "C" int llmx_gemm_tile_offsets_fit(int M, int N, int K, int lda, int epi,
     return w_rows * (size_t)K * sizeof(bf16_t) < limit && a_rows * (size_t)lda * sizeof(bf16_t) < limit ? 1 : 0;
 }
 
+// The runs' sums of a product whose runs were multiplied apart (TileArgs::run_tiles), added in run order as the kernel
+// that holds all runs adds them, then stored as the epilogue says.  Four neighbouring features a thread.
+template <bool ADD, typename TC>
+__global__ void __launch_bounds__(256) gemm_runs_sum_kernel(const float* __restrict__ partial, TC* __restrict__ C, int M, int N, int ldc, int runs) {
+    const int quads = (N + 3) / 4;
+    const long at = (long)blockIdx.x * 256 + threadIdx.x;
+    if (at >= (long)M * quads) return;
+    const int m = (int)(at / quads), n = (int)(at % quads) * 4;
+    const bool whole = n + 3 < N && N % 4 == 0;
+    float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int r = 0; r < runs; ++r) {
+        const float* src = partial + ((size_t)r * M + m) * N + n;
+        float x[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (whole) {
+            const f32x4_t q = *reinterpret_cast<const f32x4_t*>(src);
+            x[0] = q[0], x[1] = q[1], x[2] = q[2], x[3] = q[3];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n + i < N) x[i] = src[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = r == 0 ? x[i] : v[i] + x[i];
+    }
+    store_quad<ADD>(C + (size_t)m * ldc, n, N, ldc % 4 == 0 && ((uintptr_t)C & 15) == 0, v);
+}
+
 static int form_rows(int form) { return form == FORM_64 || form == FORM_BOUNDED ? 64 : 128; }
 static int form_feats(int form, int epi) { return (epi == TL_SWIGLU ? 64 : 128) * (form == FORM_WIDE ? 2 : 1); }
 
@@ -778,11 +809,24 @@ static int form_feats(int form, int epi) { return (epi == TL_SWIGLU ? 64 : 128) 
 //   dense: the wide form (8 waves, 128 x 256, three tiles deep) where it has at least 192 tiles for the 256 CUs
 //     (measured on 2,048 rows: 8,192 features 113 against 165 us, 3,072 features 100 against 108 us), else 64-row
 //     tiles (three workgroups a CU; more, smaller tiles fill the chip better when there are few).
+//     With `runs_scratch` (llmx_gemm_tile_runs_scratch floats) a product of few tiles and several runs of K gives each
+//     run a workgroup of its own and adds the runs' sums in a second kernel, in the order the one kernel adds them.
 //   grouped with tile_stats: both a 128-row form (wide for long K, 4 waves for short K) and the 64-row form are
 //     launched; on the device the one that fits the groups' rows works and the other leaves at once.
+// Floats of scratch with which llmx_gemm_tile multiplies the runs of a dense product apart (0: it would not).
+extern "C" long llmx_gemm_tile_runs_scratch(int M, int N, int K, int epi, int ks, int n_groups) {
+    if (n_groups > 0 || epi == TL_SWIGLU || ks < 2 || K % TL_BK || M <= 0 || N <= 0) return 0;
+    const int steps = (K + 31) / 32, per = (steps + ks - 1) / ks;
+    if (per % 2) return 0;
+    const long tiles = (long)((M + 63) / 64) * ((N + TL_BN - 1) / TL_BN);
+    if (tiles >= TILE_RUNS_APART_BELOW) return 0;     // enough workgroups without
+    const int runs = (K / TL_BK + per / 2 - 1) / (per / 2);
+    return runs < 2 ? 0 : (long)runs * M * N;
+}
+
 extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldc, int epi, int ks,
                               int n_groups, int max_tiles, const int* group_offsets, const int* list, int a_div, long w_group_stride,
-                              int up_offset, const int* tile_stats, hipStream_t stream) {
+                              int up_offset, const int* tile_stats, float* runs_scratch, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     if (K % 8) return -2;
     const bool grouped = n_groups > 0;
@@ -790,7 +834,7 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
     const int steps = (K + 31) / 32, per = (steps + ks - 1) / ks;
     const bool lean = K % TL_BK == 0 && (ks == 1 || per % 2 == 0) && llmx_gemm_tile_offsets_fit(M, N, K, lda, epi, n_groups, a_div, up_offset);
     TileArgs g{(const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldc, group_offsets, list, n_groups, a_div > 0 ? a_div : 1,
-               w_group_stride, up_offset, 0, ks, 64, nullptr, 0};
+               w_group_stride, up_offset, 0, ks, 64, nullptr, 0, 0};
     auto launch = [&](int form, int tiles_y) -> int {
         g.bm = form_rows(form);
         g.m_tiles = (M + g.bm - 1) / g.bm;
@@ -806,6 +850,30 @@ extern "C" int llmx_gemm_tile(const void* A, const void* W, void* C, int c_dtype
     int rc;
     if (!lean) {
         rc = launch(FORM_BOUNDED, max_tiles);
+    } else if (!grouped && runs_scratch && llmx_gemm_tile_runs_scratch(M, N, K, epi, ks, 0) > 0) {
+        // few tiles (a step of some tens of rows): a workgroup a run of K, then the runs' sums added in run order
+        const int tiles_per_run = per / 2, runs = (K / TL_BK + tiles_per_run - 1) / tiles_per_run;
+        TileArgs part = g;
+        part.C = runs_scratch;
+        part.ldc = N;
+        part.ks = 1;
+        part.bm = 64;
+        part.m_tiles = (M + 63) / 64;
+        part.run_tiles = tiles_per_run;
+        llmx_note_launch(LK_GEMM_TILE_RUNS_APART);
+        hipLaunchKernelGGL((gemm_tile_kernel<TL_STORE, float, false, false, true, 64>), dim3((N + TL_BN - 1) / TL_BN, part.m_tiles, runs), dim3(256), 0,
+                           stream, part);
+        const long quads = (long)M * ((N + 3) / 4);
+        const dim3 sum_grid((unsigned)((quads + 255) / 256));
+        if (epi == TL_ADD) {
+            if (c_dtype != LLMX_F32) return -2;
+            hipLaunchKernelGGL((gemm_runs_sum_kernel<true, float>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (float*)C, M, N, ldc, runs);
+        } else if (c_dtype == LLMX_BF16) {
+            hipLaunchKernelGGL((gemm_runs_sum_kernel<false, bf16_t>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (bf16_t*)C, M, N, ldc, runs);
+        } else {
+            hipLaunchKernelGGL((gemm_runs_sum_kernel<false, float>), sum_grid, dim3(256), 0, stream, (const float*)runs_scratch, (float*)C, M, N, ldc, runs);
+        }
+        rc = 0;
     } else if (!grouped) {
         const long wide_tiles = (long)((M + WD_BM - 1) / WD_BM) * ((N + form_feats(FORM_WIDE, epi) - 1) / form_feats(FORM_WIDE, epi));
         rc = launch(wide_tiles >= 192 ? FORM_WIDE : FORM_64, 0);

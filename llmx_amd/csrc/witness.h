@@ -21,6 +21,7 @@
     X(GEMM_TILE_64, "gemm_tile.64")                                                                                       \
     X(GEMM_TILE_WIDE, "gemm_tile.wide")                                                                                   \
     X(GEMM_TILE_BOUNDED, "gemm_tile.bounded")                                                                             \
+    X(GEMM_TILE_RUNS_APART, "gemm_tile.runs_apart")                                                                       \
     X(GEMM_TILE_GROUPED_64, "gemm_tile.grouped_64")                                                                       \
     X(GEMM_TILE_GROUPED_128, "gemm_tile.grouped_128")                                                                     \
     X(GEMM_TILE_GROUPED_WIDE, "gemm_tile.grouped_wide")                                                                   \

@@ -72,7 +72,7 @@ def _declare(h) -> None:
         "llmx_gemm_skinny_f32_normed_ok": [I, I],
         "llmx_argmax_rows": [P, P, P, P, I, I, P],
         "llmx_gemm_skinny_f32": [P, P, P, I, I, I, I, I, I, I, I, L, P, F, P],
-        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P],
+        "llmx_gemm_tile": [P, P, P, I, I, I, I, I, I, I, I, I, I, P, P, I, L, I, P, P, P],
         "llmx_gemm_tile_offsets_fit": [I, I, I, I, I, I, I, I],
         "llmx_sample_all": [P, P, P, P, P, P, I, I, P, P],
         "llmx_sample_topk": [P, P, P, P, P, P, P, P, I, I, P, I, P],
@@ -93,6 +93,8 @@ def _declare(h) -> None:
     h.llmx_sample_all_scratch.restype = c_long
     h.llmx_sample_ranked_scratch.argtypes = [I, I]
     h.llmx_sample_ranked_scratch.restype = c_long
+    h.llmx_gemm_tile_runs_scratch.argtypes = [I, I, I, I, I, I]
+    h.llmx_gemm_tile_runs_scratch.restype = c_long
     h.llmx_launch_name.restype = ctypes.c_char_p
     h.llmx_note_launch.restype = None
 
@@ -176,6 +178,7 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[tor
 
 
 SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores
+TILE_RUNS_APART_MIN_ROWS = 17  # dense products from this many rows on take the tiled kernel with K's runs in workgroups of their own, where it offers that
 TILE_FILL = 1024              # feature tiles of 128 from which the tiled kernel fills the chip with one tile of rows
 SKINNY_MAX_GROUPED_ROWS = 16   # routed products of at most this many token rows do (measured: beyond it the tiled kernel streams the experts faster)
 
@@ -236,9 +239,11 @@ def gemm_f32_takes_normed_rows(rows: int, w: torch.Tensor) -> bool:
     return rows <= NORMED_ROWS_PAY and gemm_f32_can_norm_rows(rows, w)
 
 
-def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False) -> None:
+def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_generic: bool = False, scratch=None) -> None:
     """c[M,N] (+)= a[M,K] @ w[N,K]^T, accumulated in float32; EPI_SWIGLU: c = silu(a @ w[:N]^T) * (a @ w[N:]^T).
-    `a` may be NormedRows where gemm_takes_normed_rows says so: the product reads bfloat16(norm(x))."""
+    `a` may be NormedRows where gemm_takes_normed_rows says so: the product reads bfloat16(norm(x)).
+    `scratch(name, shape, dtype)` gives storage that lives as long as the caller's step (a step's workspace): with it,
+    products of some tens of rows multiply K's runs in workgroups of their own; the bits are the same either way."""
     M, K = a.shape
     N = w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]   # swiglu: w holds gate rows, then up rows
     if w.shape[1] != K or tuple(c.shape) != (M, N):
@@ -253,14 +258,23 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
     # beyond 16 rows a product wide enough to fill the chip with tiles streams its weights faster through the tiled kernel
     # (the LM head); both kernels give a row the same bits
     skinny = M <= 16 or (M <= SKINNY_MAX_ROWS and -(-N // 128) < TILE_FILL)
+    ks = _split_k(-(-N // 16), K)
+    # some tens of rows: every 16-feature strip of the weight-streaming kernel reads all rows again; tiles of 128 features
+    # do not, and are enough workgroups once each run of K has its own
+    runs_apart = 0
+    if scratch is not None and not force_generic and M >= TILE_RUNS_APART_MIN_ROWS and _skinny_ok(a, w, c, epilogue):
+        runs_apart = lib().llmx_gemm_tile_runs_scratch(M, N, K, epilogue, ks, 0)
+    if runs_apart:
+        skinny = False
     if not force_generic and skinny and _skinny_ok(a, w, c, epilogue):
         _check(lib().llmx_gemm_skinny(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
                                       _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *_NO_NORM, _stream()),
                "gemm_skinny")
         return
     if not force_generic and _skinny_ok(a, w, c, epilogue):
+        runs = scratch("gemm_tile.runs", (runs_apart,), torch.float32) if runs_apart else None
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), M, N, K, K, N, epilogue,
-                                    _split_k(-(-N // 16), K), 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, 0, _stream()), "gemm_tile")
+                                    ks, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, 0, _dev(runs, "runs"), _stream()), "gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),
                                    M, N, K, K, K, N, epilogue, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, _stream()), "gemm")
@@ -305,7 +319,7 @@ def grouped_gemm(a: torch.Tensor, w: torch.Tensor, c: torch.Tensor, offsets: tor
         _check(lib().llmx_gemm_tile(_dev(a, "a"), _dev(w, "w"), _dev(c, "c"), _code(c.dtype), n_pairs, N, K, K, N, epilogue,
                                     _split_k(-(-N // 16), K), G, min(G, n_pairs) + n_pairs // 64, _dev(offsets, "offsets", torch.int32, (G + 1,)),
                                     _dev(pairs, "pairs", torch.int32), a_div, NW * K, N if epilogue == EPI_SWIGLU else 0,
-                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), _stream()),
+                                    _dev(tile_stats if n_pairs >= TILE_STATS_MIN_PAIRS else None, "tile_stats", torch.int32, (1,)), 0, _stream()),
                "grouped_gemm_tile")
         return
     _check(lib().llmx_gemm_generic(_dev(a, "a"), _code(a.dtype), _dev(w, "w"), _code(w.dtype), _dev(c, "c"), _code(c.dtype),

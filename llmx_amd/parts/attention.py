@@ -100,7 +100,7 @@ class Attention(Mixer):
         T = step.rows
         act = step.act_dtype
         qkv = step.buf("attention.qkv", (T, self.q_width + 2 * self.kv_width), torch.float32)
-        ops.gemm(h, self.wqkv, qkv)
+        ops.gemm(h, self.wqkv, qkv, scratch=step.buf)
         q = step.buf("attention.q", (T, self.q_width), act)
         cos_sin, rotary = self.position.rotation()
         tables = step.tables(cache.group)
@@ -111,7 +111,7 @@ class Attention(Mixer):
         plan = self._plan(step) if ops.attention_mfma_ok(act, self.head_dim, cache.k.shape[2]) else None
         ops.paged_attention(q, cache.k, cache.v, step.positions, step.row_entry, tables, o, self.scale, self.heads,
                             window=int(self.window or 0), plan=plan, scratch=step.buf)
-        ops.gemm(o, self.wo, out, ops.EPI_ADD if accumulate else ops.EPI_STORE)
+        ops.gemm(o, self.wo, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 
 register("mixer", "attention", Attention)

@@ -136,7 +136,7 @@ class DenseGLU(FeedForward):
     def forward(self, step, h, out, accumulate, h32=None):
         act = step.buf("glu.act", (step.rows, self.intermediate), step.act_dtype)
         ops.gemm(h, self.w_gate_up, act, ops.EPI_SWIGLU)
-        ops.gemm(act, self.w_down, out, ops.EPI_ADD if accumulate else ops.EPI_STORE)
+        ops.gemm(act, self.w_down, out, ops.EPI_ADD if accumulate else ops.EPI_STORE, scratch=step.buf)
 
 
 register("feed_forward", "routed_experts", RoutedExperts)

@@ -139,8 +139,8 @@ def test_many_requests_decoded_together_at_the_real_sizes(real_layer_engine, n_r
     every request's logits over the whole vocabulary are those of its run alone."""
     launched = check_decoding_together(real_layer_engine, REAL_LAYER["vocab_size"], n_requests, 16, seed=1000 + n_requests)
     assert not set(launched) & UNIVERSAL, f"the bfloat16 engine fell to {sorted(set(launched) & UNIVERSAL)}"
-    # dense products of 17 to 64 rows: QKV on two strips a workgroup, the output projection on one
-    assert "gemm_skinny.two_strips" in launched and "gemm_skinny" in launched
+    # dense products of 17 to 64 rows: tiles of 128 features with K's runs in workgroups of their own
+    assert "gemm_tile.runs_apart" in launched and "gemm_skinny.two_strips" not in launched, sorted(launched)
     # routed products above 16 token rows and the head above 16 rows: the tiled kernels
     assert "gemm_tile.grouped_64" in launched and ("gemm_tile.wide" in launched or "gemm_tile.64" in launched)
     assert "route_topk" in launched and "moe_align" in launched and "route_topk_align" not in launched

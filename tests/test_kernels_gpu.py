@@ -127,6 +127,50 @@ def test_gemm_matrix_cores_bf16(M, N, K):
             assert torch.equal(few, c[rows]), "a row's bits depend on how many rows the product has"
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 8192, 3072), (64, 3072, 6144), (33, 3080, 6144), (130, 3072, 6144), (47, 8200, 3072), (100, 520, 4096)])
+def test_gemm_with_runs_apart_gives_the_bits_of_the_other_forms(M, N, K):
+    """Dense products of some tens of rows and few tiles, given a step's scratch, multiply each run of K in a workgroup of
+    its own and add the runs' sums in a second kernel: the bits of the weight-streaming kernel (a row alone, 16 rows) and
+    of the tiled kernel that holds all runs itself (the same call without scratch), for every epilogue, ragged N; and
+    the launch says which ran."""
+    o = ops()
+    a = rnd(M, K, dtype=torch.bfloat16)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=1, scale=0.2)
+    held = {}
+
+    def scratch(name, shape, dtype):
+        key = (name, dtype)
+        if key not in held or held[key].numel() < math.prod(shape):
+            held[key] = torch.full((math.prod(shape),), float("nan"), dtype=dtype, device=DEV)
+        return held[key][:math.prod(shape)].view(*shape)
+
+    c = torch.full((M, N), float("nan"), dtype=torch.float32, device=DEV)
+    o.take_launches()
+    o.gemm(a, w, c, scratch=scratch)
+    ran = o.take_launches()
+    assert ran.get("gemm_tile.runs_apart", 0) == 1 and not ran.get("gemm_skinny", 0) and not ran.get("gemm_tile.64", 0), ran
+    plain = torch.empty_like(c)
+    o.gemm(a, w, plain)
+    ran = o.take_launches()
+    assert not ran.get("gemm_tile.runs_apart", 0)
+    assert torch.equal(c, plain)
+    for rows in ([0], [M - 1], list(range(M - 16, M))):
+        few = torch.empty(len(rows), N, dtype=torch.float32, device=DEV)
+        o.gemm(a[rows].contiguous(), w, few, scratch=scratch)
+        assert torch.equal(few, c[rows]), "a row's bits depend on how many rows the product has"
+    assert o.take_launches().get("gemm_tile.runs_apart", 0) == 0
+    want = a.double() @ w.double().T
+    assert (c.double() - want).abs().max() <= 1e-5 * math.sqrt(K) * want.abs().max()
+    cb = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    o.gemm(a, w, cb, scratch=scratch)
+    assert torch.equal(cb, c.to(torch.bfloat16))
+    base = rnd(M, N, seed=9)
+    acc = base.clone()
+    o.gemm(a, w, acc, o.EPI_ADD, scratch=scratch)
+    assert torch.equal(acc, base + c)
+    assert o.take_launches().get("gemm_tile.runs_apart", 0) == 2
+
+
 @pytest.mark.parametrize("M,N,K", [(1500, 8200, 128), (1536, 8192, 768), (1408, 8320, 3072)])
 def test_gemm_wide_tiles_give_the_bits_of_small_tiles(M, N, K):
     """Products of many rows and features run on 128 x 256 tiles (8 waves); a row's bits are those of the 64-row tiles

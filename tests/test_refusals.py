@@ -136,5 +136,5 @@ def test_the_launch_witness_counts_by_name_and_clears():
     assert ops.take_launches() == {"gemm_tile.wide": 3, "attention.merge": 1}
     assert ops.take_launches() == {}
     # a product of no rows returns before its launch site
-    assert h.llmx_gemm_tile(0, 0, 0, 1, 0, 128, 64, 64, 128, 0, 1, 0, 0, 0, 0, 1, 0, 0, 0, 0) == 0
+    assert h.llmx_gemm_tile(0, 0, 0, 1, 0, 128, 64, 64, 128, 0, 1, 0, 0, 0, 0, 1, 0, 0, 0, 0, 0) == 0
     assert ops.take_launches() == {}
