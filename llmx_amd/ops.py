@@ -179,6 +179,7 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[tor
 
 SKINNY_MAX_ROWS = 64          # dense products of at most this many rows stream the weights once on the matrix cores
 TILE_RUNS_APART_MIN_ROWS = 17  # dense products from this many rows on take the tiled kernel with K's runs in workgroups of their own, where it offers that
+SKINNY_WIDE_MAX_ROWS = 4      # ... and of at most this many rows however wide they are
 TILE_FILL = 1024              # feature tiles of 128 from which the tiled kernel fills the chip with one tile of rows
 SKINNY_MAX_GROUPED_ROWS = 16   # routed products of at most this many token rows do (measured: beyond it the tiled kernel streams the experts faster)
 
@@ -255,9 +256,10 @@ def gemm(a, w: torch.Tensor, c: torch.Tensor, epilogue: int = EPI_STORE, force_g
                                       _split_k(-(-N // 16), K), 0, 0, 0, 0, 0, 0, 1, 0, N if epilogue == EPI_SWIGLU else 0, *a.args(), _stream()),
                "gemm_skinny (normed rows)")
         return
-    # beyond 16 rows a product wide enough to fill the chip with tiles streams its weights faster through the tiled kernel
-    # (the LM head); both kernels give a row the same bits
-    skinny = M <= 16 or (M <= SKINNY_MAX_ROWS and -(-N // 128) < TILE_FILL)
+    # a product wide enough to fill the chip with tiles (the LM head) streams its weights faster through the tiled kernel
+    # from 5 rows on (every 16-feature strip of the weight-streaming kernel reads all rows again: 200,064 features at 8 rows
+    # 264 against 239 us, at 16 rows 308 against 246 us); both kernels give a row the same bits
+    skinny = M <= SKINNY_WIDE_MAX_ROWS or (M <= SKINNY_MAX_ROWS and -(-N // 128) < TILE_FILL)
     ks = _split_k(-(-N // 16), K)
     # some tens of rows: every 16-feature strip of the weight-streaming kernel reads all rows again; tiles of 128 features
     # do not, and are enough workgroups once each run of K has its own
