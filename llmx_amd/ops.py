@@ -377,6 +377,7 @@ class AttentionPlan:
 
 _PLAN_CACHE: dict = {}
 ATTENTION_TARGET_WAVES = 2048   # work items wanted before long contexts stop being split further
+ATTENTION_WHOLE_ITEMS = 1024    # from this many items on (rows x KV heads) no context is split (batch 128 at 4,096 tokens: 43.9 -> 41.2 ms a step)
 ATTENTION_SEGMENT = 128         # keys in a segment: the unit contexts are split in (the kernel's AM_SEG)
 ATTENTION_WIDE_ITEMS = 1024     # up to this many decoding items a step, an item gets a workgroup of 4 waves instead of one wave
 
@@ -399,6 +400,8 @@ def attention_plan(row_counts, contexts, n_heads: int, n_kv_heads: int, device, 
         seg_cap = -(-longest // ATTENTION_SEGMENT) + 1
         seg_cap = -(-seg_cap // 8) * 8       # in steps of 8, so a growing context reuses a plan for 1,024 tokens
         n_splits = max(1, min(-(-ATTENTION_TARGET_WAVES // base), seg_cap))
+        if base >= ATTENTION_WHOLE_ITEMS:     # enough items as they are: sharing out would cost the partial results and their merge
+            n_splits = 1
     key = (tuple(row_counts), n_heads, n_kv_heads, n_splits, seg_cap, str(device))
     plan = _PLAN_CACHE.get(key)
     if plan is not None:
