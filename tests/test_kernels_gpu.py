@@ -726,14 +726,14 @@ def test_merged_columns_give_the_bits_of_an_item_that_walks_its_context(contexts
     pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device=DEV)
     ent = torch.arange(n, dtype=torch.int32, device=DEV)
     outs = []
-    saved = o.ATTENTION_TARGET_WAVES
+    saved = o.ATTENTION_TARGET_WAVES, o.ATTENTION_WHOLE_ITEMS
     for target in (100000, 1):
-        o.ATTENTION_TARGET_WAVES = target
+        o.ATTENTION_TARGET_WAVES, o.ATTENTION_WHOLE_ITEMS = target, 1 << 30     # split however many items there are
         o._PLAN_CACHE.clear()
         try:
             plan = o.attention_plan([1] * n, list(contexts), Hq, Hkv, DEV, window)
         finally:
-            o.ATTENTION_TARGET_WAVES = saved
+            o.ATTENTION_TARGET_WAVES, o.ATTENTION_WHOLE_ITEMS = saved
         assert plan.n_merges == (n * Hq if target > 1 else 0)
         out = torch.zeros(n, Hq * D, dtype=torch.bfloat16, device=DEV)
         o.take_launches()
