@@ -181,7 +181,7 @@ template <int DT, bool PARTIAL>
 __global__ void __launch_bounds__(256, (PARTIAL && DT <= 8) ? 2 : 1) paged_attention_mfma_kernel(AttnMfmaArgs a) {
     constexpr int QS = (DT + 1) / 2;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int item_no = blockIdx.x * 4 + wave;
+    const int item_no = blockIdx.x * (int)(blockDim.x >> 6) + wave;   // 1, 2 or 4 waves a workgroup, as the launch spreads the items over the chip
     if (item_no >= a.n_items) return;
     const int* it = a.items + (size_t)item_no * AM_ITEM_INTS;   // the same for the whole wave
     const int row0 = __builtin_amdgcn_readfirstlane(it[0]), n_rows = __builtin_amdgcn_readfirstlane(it[1]);
@@ -1136,13 +1136,16 @@ extern "C" int llmx_paged_attention_mfma(const void* q, const void* k_cache, con
     // few long columns: 64 dims a workgroup, so that more compute units bring the segments in
     const bool short_merge = forms & 2, narrow_merge = !short_merge && n_merges * ((head_dim + 127) / 128) <= MERGE_NARROW_COLUMNS;
     if (n_merges > 0) llmx_note_launch(narrow_merge ? LK_ATTENTION_MERGE_NARROW : LK_ATTENTION_MERGE);
+    // items that walk a whole context: nothing is shared between an item's waves, so few items go out as workgroups of one
+    // wave, over all the compute units instead of a quarter of them
+    const int dw = n_direct <= 512 ? 1 : 4;   // measured at 4,096 and 8,192 tokens: 512 items 208 -> 176 us, 384 items 199 -> 160 us; 640 items and more are faster by fours
     switch (head_dim / 16) {
 #define AM_CASE(DT)                                                                                                          \
     case DT:                                                                                                                 \
         if (n_shared > 0 && DT == 8 && page_tokens % 16 == 0)                                                               \
             hipLaunchKernelGGL(paged_attention_tiles128_kernel, dim3(n_shared / AM_TILES128_WAVES), dim3(64 * AM_TILES128_WAVES), 0, stream, sh); \
         else if (n_shared > 0) hipLaunchKernelGGL((paged_attention_tiles_kernel<DT>), dim3(n_shared / 4), block, 0, stream, sh);        \
-        if (n_direct > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, false>), dim3((n_direct + 3) / 4), block, 0, stream, a);  \
+        if (n_direct > 0) hipLaunchKernelGGL((paged_attention_mfma_kernel<DT, false>), dim3((n_direct + dw - 1) / dw), dim3(64 * dw), 0, stream, a);  \
         if (n_partial > 0 && DT == 8 && wide_items)                                                                          \
             hipLaunchKernelGGL(paged_attention_split4_kernel, dim3(n_partial), block, 0, stream, b);                                    \
         else if (n_partial > 0)                                                                                              \

@@ -377,7 +377,7 @@ class AttentionPlan:
 
 _PLAN_CACHE: dict = {}
 ATTENTION_TARGET_WAVES = 2048   # work items wanted before long contexts stop being split further
-ATTENTION_WHOLE_ITEMS = 512     # from this many items on (rows x KV heads) no context is split: one wave an item walks its context at 5.2-6.2 TB/s, and sharing out would cost the partial results and their merge (64 rows at 4,096 tokens: 227 -> 207 us a layer, at 8,192: 463 -> 401; 128 rows: 447 -> 348)
+ATTENTION_WHOLE_ITEMS = 320     # from this many items on (rows x KV heads) no context is split: one wave an item walks its context (up to 512 items a workgroup each, over all the chip) at 5-6 TB/s, and sharing out would cost the partial results and their merge (4,096 tokens: 40 rows 163 -> 152 us a layer, 48 rows 190 -> 154, 64 rows 227 -> 176, 128 rows 447 -> 348; 32 rows are faster split: 114 against 139)
 ATTENTION_SEGMENT = 128         # keys in a segment: the unit contexts are split in (the kernel's AM_SEG)
 ATTENTION_WIDE_ITEMS = 1024     # up to this many decoding items a step, an item gets a workgroup of 4 waves instead of one wave
 
