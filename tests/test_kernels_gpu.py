@@ -761,6 +761,66 @@ def test_merged_columns_give_the_bits_of_an_item_that_walks_its_context(contexts
         assert (outs[0][i, h * D:(h + 1) * D].double() - want).abs().max() <= 1.2e-2 * want.abs().max() + 2e-4
 
 
+@pytest.mark.parametrize("contexts,Hq,Hkv,D,target,wide", [
+    ((4100, 4097, 8192, 5000, 6111, 4225, 7000, 4096), 16, 8, 128, 2048, False),   # 32 splits of 33 to 64 segments: dealt out evenly
+    ((1500, 1400, 1100), 6, 2, 128, 48, True),                                     # 8 splits of 9 to 12 segments, four waves an item
+    ((1500, 1025, 2048, 1153), 8, 4, 64, 128, False), ((2300,), 4, 1, 48, 10, False)])
+def test_splits_that_would_take_two_segments_each_deal_them_out_evenly(contexts, Hq, Hkv, D, target, wide):
+    """Contexts of more segments than splits but at most twice as many: every split takes one or two segments instead of
+    half of the splits taking two and the rest none.  The bits are those of items that walk their contexts whole, for
+    the one-wave and the four-wave form, rows of different lengths in one step, and a context that is exactly two
+    segments a split."""
+    o = ops()
+    page = 16
+    n = len(contexts)
+    blocks = [-(-c // page) for c in contexts]
+    order = list(range(sum(blocks)))
+    random.Random(n + D).shuffle(order)
+    table = torch.full((n, max(blocks)), -1, dtype=torch.int32)
+    at = 0
+    for i, b in enumerate(blocks):
+        table[i, :b] = torch.tensor(order[at:at + b])
+        at += b
+    table = table.to(DEV)
+    k_cache = rnd(sum(blocks), Hkv, page, D, dtype=torch.bfloat16, scale=0.5)
+    v_cache = rnd(sum(blocks), Hkv, D, page, dtype=torch.bfloat16, seed=2)
+    q = rnd(n, Hq * D, dtype=torch.bfloat16, seed=3)
+    pos = torch.tensor([c - 1 for c in contexts], dtype=torch.int32, device=DEV)
+    ent = torch.arange(n, dtype=torch.int32, device=DEV)
+    outs = []
+    saved = o.ATTENTION_TARGET_WAVES, o.ATTENTION_WHOLE_ITEMS
+    for tw in (target, 1):
+        o.ATTENTION_TARGET_WAVES, o.ATTENTION_WHOLE_ITEMS = tw, 1 << 30
+        o._PLAN_CACHE.clear()
+        try:
+            plan = o.attention_plan([1] * n, list(contexts), Hq, Hkv, DEV)
+        finally:
+            o.ATTENTION_TARGET_WAVES, o.ATTENTION_WHOLE_ITEMS = saved
+        if tw > 1:
+            n_splits = plan.items[-1, 5].item()
+            segs = [-(-c // 128) for c in contexts]
+            assert any(n_splits < sg <= 2 * n_splits for sg in segs), (n_splits, segs)
+            assert plan.n_merges == n * Hq and (plan.wide_items and D == 128) == wide
+        out = torch.zeros(n, Hq * D, dtype=torch.bfloat16, device=DEV)
+        o.take_launches()
+        o.paged_attention(q, k_cache, v_cache, pos, ent, table, out, 1.0 / math.sqrt(D), Hq, plan=plan)
+        ran = o.take_launches()
+        if tw > 1:
+            assert ran.get("attention.split4" if wide else "attention.partial", 0) == 1, ran
+        outs.append(out)
+    o._PLAN_CACHE.clear()
+    assert torch.equal(outs[0], outs[1])
+    for i, c in enumerate(contexts):       # and the plain softmax for one head of every row
+        pages = table[i, :blocks[i]].long()
+        keys = k_cache[pages].permute(1, 0, 2, 3).reshape(Hkv, -1, D)[:, :c].double()
+        values = v_cache[pages].permute(1, 0, 3, 2).reshape(Hkv, -1, D)[:, :c].double()
+        h = (i * 5) % Hq
+        kv = h // (Hq // Hkv)
+        w = torch.softmax((keys[kv] @ q[i, h * D:(h + 1) * D].double()) / math.sqrt(D), dim=0)
+        want = w @ values[kv]
+        assert (outs[0][i, h * D:(h + 1) * D].double() - want).abs().max() <= 1.2e-2 * want.abs().max() + 2e-4
+
+
 @pytest.mark.parametrize("L,Hq,Hkv,D", [(70000, 2, 1, 32), (66000, 4, 2, 160)])
 def test_attention_very_long_context(L, Hq, Hkv, D):
     """A decoded row over more than 512 segments of keys (the merge works through them in several rounds): the same bits
