@@ -79,7 +79,7 @@ class Generator:
         by_id = {r.id: r for r in sch.running}
         reqs = [by_id[e.request] for e in wanting]
         tokens = self.sampler.sample(logits, [r.params for r in reqs], [r.generated for r in reqs], [r.rng for r in reqs],
-                                     self.engine.spec.eos_token_id)
+                                     self.engine.spec.eos_token_id, keys=[r.id for r in reqs])
         dt = time.perf_counter() - t0
         prompt_rows = sum(len(e.tokens) for e in plan if len(e.tokens) > 1 or not by_id[e.request].generated)
         self.stats.steps += 1

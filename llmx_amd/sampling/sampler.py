@@ -17,11 +17,34 @@ from .. import ops
 from .params import MAX_EXACT_TOP_K, SamplingParams, XorShift64
 
 
+class _Seen:
+    """The distinct tokens of one request's history and how often each was seen, kept up as the history grows."""
+
+    __slots__ = ("n", "index", "ids", "counts")
+
+    def __init__(self):
+        self.n, self.index, self.ids, self.counts = 0, {}, [], []
+
+    def follow(self, history: Sequence[int]) -> None:
+        if len(history) < self.n:      # the history was cut: count again
+            self.__init__()
+        for tok in history[self.n:]:
+            at = self.index.get(tok)
+            if at is None:
+                self.index[tok] = len(self.ids)
+                self.ids.append(tok)
+                self.counts.append(1)
+            else:
+                self.counts[at] += 1
+        self.n = len(history)
+
+
 class Sampler:
     def __init__(self, vocab_size: int, device: torch.device):
         self.vocab = vocab_size
         self.device = device
         self._kept = None     # (key, settings) of the last rows sampled
+        self._seen = {}       # request key -> _Seen, for the rows whose penalties need their histories' counts
 
     def _f32(self, values) -> torch.Tensor:
         return torch.tensor(np.asarray(values, dtype=np.float32), device=self.device)
@@ -30,24 +53,34 @@ class Sampler:
         return torch.tensor(np.asarray(values, dtype=np.int32), device=self.device)
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], generated: Sequence[Sequence[int]],
-               rngs: Sequence[XorShift64], eos: Optional[int]) -> List[int]:
+               rngs: Sequence[XorShift64], eos: Optional[int], keys: Optional[Sequence] = None) -> List[int]:
         """One token id for each row of `logits` [W, vocab]; `generated` holds each row's tokens so far (for the penalties).
 
-        The logits are scratch of the step and are changed in place by the penalties.
+        The logits are scratch of the step and are changed in place by the penalties.  `keys` (one hashable a row, a
+        request's id for instance): a row's history is the history the same key had at the last call, grown at its end;
+        its counts are then kept up token by token instead of being formed again from the whole history at every step.
         """
         W = logits.shape[0]
-        if not (len(params) == len(generated) == len(rngs) == W):
+        if not (len(params) == len(generated) == len(rngs) == W) or (keys is not None and len(keys) != W):
             raise ValueError("sampler: one set of settings, one history and one generator per row")
         if W == 0:
             return []
         # penalties, in place: one list entry per (row, distinct seen token)
         rows, ids, counts = [], [], []
+        seen_now = {}
         for r, (p, gen) in enumerate(zip(params, generated)):
             if p.penalized and gen:
-                for tok, c in Counter(gen).items():
-                    rows.append(r)
-                    ids.append(tok)
-                    counts.append(c)
+                if keys is None:
+                    seen = Counter(gen)
+                    row_ids, row_counts = list(seen.keys()), list(seen.values())
+                else:
+                    seen = seen_now[keys[r]] = self._seen.get(keys[r]) or _Seen()
+                    seen.follow(gen)
+                    row_ids, row_counts = seen.ids, seen.counts
+                rows += [r] * len(row_ids)
+                ids += row_ids
+                counts += row_counts
+        self._seen = seen_now     # requests that are no longer sampled are forgotten
         if rows:
             ops.penalize(logits, self._i32(rows), self._i32(ids), self._i32(counts), self._f32([p.penalty for p in params]),
                          self._f32([p.presence_penalty for p in params]), self._f32([p.frequency_penalty for p in params]))

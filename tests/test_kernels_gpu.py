@@ -1431,6 +1431,32 @@ def test_penalties():
     assert row == [3.0 - 0.5 - 0.5, 1.0 - 0.5 - 0.25, 0.0]
 
 
+def test_sampler_keeps_the_counts_of_growing_histories():
+    """With request keys the sampler keeps each request's seen tokens and counts up as its history grows, instead of
+    counting the whole history at every step: the tokens are those of a sampler without keys, over 60 steps of three
+    requests of which one leaves and comes back with a shorter history and one has no penalty."""
+    from llmx_amd.sampling import Sampler, SamplingParams, XorShift64
+    V = 500
+    params = [SamplingParams(temp=0.9, top_k=20, penalty=1.3, presence_penalty=0.2, frequency_penalty=0.1), SamplingParams(temp=0.0, penalty=1.8),
+              SamplingParams(temp=1.1, top_k=0, top_p=0.9)]
+    keyed, plain = Sampler(V, torch.device(DEV)), Sampler(V, torch.device(DEV))
+    histories = [[3, 3, 7], [], [1]]
+    rng_a = [XorShift64(5 + i) for i in range(3)]
+    rng_b = [XorShift64(5 + i) for i in range(3)]
+    for step in range(60):
+        rows = [0, 1, 2] if step % 7 else [0, 2]          # the second request sits a step out now and then
+        if step == 30:
+            histories[0] = histories[0][:5]                # ... and the first one's history is cut once
+        logits = rnd(len(rows), V, scale=3.0, seed=100 + step)
+        a = keyed.sample(logits.clone(), [params[r] for r in rows], [histories[r] for r in rows], [rng_a[r] for r in rows], None,
+                         keys=[f"request {r}" for r in rows])
+        b = plain.sample(logits.clone(), [params[r] for r in rows], [list(histories[r]) for r in rows], [rng_b[r] for r in rows], None)
+        assert a == b, f"step {step}: with keys {a}, without {b}"
+        for r, t in zip(rows, a):
+            histories[r].append(t)
+    assert len(set(histories[1])) > 3, "the penalty never moved the greedy request off its token"
+
+
 def test_fill_random_matches_host():
     from llmx_amd.parts.spec import TensorSpec
     from llmx_amd.weights import RandomInit, host_values
