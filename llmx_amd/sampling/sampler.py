@@ -45,9 +45,24 @@ class Sampler:
         self.device = device
         self._kept = None     # (key, settings) of the last rows sampled
         self._seen = {}       # request key -> _Seen, for the rows whose penalties need their histories' counts
+        self._unit_host = self._unit_dev = None    # the rows' uniform numbers: pinned host memory and its place on the device
 
     def _f32(self, values) -> torch.Tensor:
         return torch.tensor(np.asarray(values, dtype=np.float32), device=self.device)
+
+    def _units(self, values) -> torch.Tensor:
+        """The step's uniform numbers on the device, copied from pinned memory without waiting for the stream: the copy and
+        the sampling kernels queue up behind the step while it still runs.  (A copy from pageable memory would hold the
+        host until the step is over, and the kernels' launches would then follow it with the device idle.)  The buffers
+        are free again when a call's tokens have been read back, which every call that uses them ends with."""
+        W = len(values)
+        if self._unit_host is None or self._unit_host.numel() < W:
+            n = max(64, 2 * W)
+            self._unit_host = torch.empty(n, dtype=torch.float32, pin_memory=True)
+            self._unit_dev = torch.empty(n, dtype=torch.float32, device=self.device)
+        self._unit_host[:W] = torch.from_numpy(np.asarray(values, dtype=np.float32))
+        self._unit_dev[:W].copy_(self._unit_host[:W], non_blocking=True)
+        return self._unit_dev[:W]
 
     def _i32(self, values) -> torch.Tensor:
         return torch.tensor(np.asarray(values, dtype=np.int32), device=self.device)
@@ -90,7 +105,7 @@ class Sampler:
         if st["greedy"]:
             ops.argmax_rows(logits, out, skip)
             return out.tolist()
-        unit = self._f32([0.0 if p.greedy else rng.unit() for p, rng in zip(params, rngs)])
+        unit = self._units([0.0 if p.greedy else rng.unit() for p, rng in zip(params, rngs)])
         temp, min_p, which = st["temp"], st["min_p"], st["which"]
         results = {}
         if "all" in which:
